@@ -1,0 +1,113 @@
+"""Regenerate tests/golden/graphs/*.json from the reference DSL (run in the authoring container only).
+
+The reference package cannot be imported whole here: ``pccl/__init__`` pulls in the superoptimizer,
+which needs ``z3`` (not installed), and ``pccl.engine`` needs the compiled CUDA extension.  The
+schedule templates and the JSON generator depend on neither, so this script loads exactly those
+modules (``nodes``, ``graph``, ``decorators``, ``passes.{dependency_analysis,dce}``,
+``codegen.{mapping,json_generator}``, ``algorithms.{base,ring,recursive_hd,tree}``) under a synthetic package skeleton and writes the JSON v2 text the reference
+emits for a handful of small configurations.  The fixtures are data (compiler output), not source.
+
+Usage:  python tests/golden/make_graph_fixtures.py [/root/reference]
+"""
+import importlib.util
+import json
+import os
+import sys
+import types
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "graphs")
+
+
+def _pkg(name, path):
+    m = types.ModuleType(name)
+    m.__path__ = [path]
+    m.__package__ = name
+    sys.modules[name] = m
+    return m
+
+
+def _load(name, relpath):
+    spec = importlib.util.spec_from_file_location(name, os.path.join(REF, relpath))
+    m = importlib.util.module_from_spec(spec)
+    sys.modules[name] = m
+    spec.loader.exec_module(m)
+    return m
+
+
+def load_reference_dsl():
+    _pkg("pccl", os.path.join(REF, "pccl"))
+    _pkg("pccl.dsl", os.path.join(REF, "pccl/dsl"))
+    _pkg("pccl.dsl.algorithms", os.path.join(REF, "pccl/dsl/algorithms"))
+    _load("pccl.dsl.nodes", "pccl/dsl/nodes.py")
+    _load("pccl.dsl.graph", "pccl/dsl/graph.py")
+    _load("pccl.dsl.decorators", "pccl/dsl/decorators.py")
+    # ``passes/__init__`` and ``compiler.py`` import the channelize pass, which imports the
+    # superoptimizer (z3).  The default pipeline of ``compile_to_json_string`` never runs that pass
+    # (enable_channelize=False, enable_superopt=False): it is DependencyAnalysis -> DCE ->
+    # DependencyAnalysis -> RuntimeGraphGenerator (pccl/dsl/compiler.py:33-54,67-69), so those
+    # three reference classes are loaded directly and driven in that order below.
+    _pkg("pccl.dsl.passes", os.path.join(REF, "pccl/dsl/passes"))
+    _pkg("pccl.dsl.codegen", os.path.join(REF, "pccl/dsl/codegen"))
+    dep = _load("pccl.dsl.passes.dependency_analysis", "pccl/dsl/passes/dependency_analysis.py")
+    dce = _load("pccl.dsl.passes.dce", "pccl/dsl/passes/dce.py")
+    _load("pccl.dsl.codegen.mapping", "pccl/dsl/codegen/mapping.py")
+    gen = _load("pccl.dsl.codegen.json_generator", "pccl/dsl/codegen/json_generator.py")
+
+    def compile_to_json_string(graph):
+        dep.DependencyAnalysisPass().run(graph)
+        dce.DeadCodeEliminationPass().run(graph)
+        dep.DependencyAnalysisPass().run(graph)
+        return gen.RuntimeGraphGenerator(indent=2).generate_string(graph)
+
+    comp = types.SimpleNamespace(compile_to_json_string=compile_to_json_string)
+    _load("pccl.dsl.algorithms.base", "pccl/dsl/algorithms/base.py")
+    ring = _load("pccl.dsl.algorithms.ring", "pccl/dsl/algorithms/ring.py")
+    rhd = _load("pccl.dsl.algorithms.recursive_hd", "pccl/dsl/algorithms/recursive_hd.py")
+    tree = _load("pccl.dsl.algorithms.tree", "pccl/dsl/algorithms/tree.py")
+    return comp, ring, rhd, tree
+
+
+CASES = [
+    # (file stem, algorithm, method, world, tensor_size, dtype, executor, channels)
+    ("ring_ar_sm_w2_n2048_bf16_c1", "ring", "build_allreduce", 2, 2048, "bfloat16", "sm", 1),
+    ("ring_ar_sm_w4_n4096_f32_c2", "ring", "build_allreduce", 4, 4096, "float32", "sm", 2),
+    ("ring_ar_tma_w8_n8192_bf16_c4", "ring", "build_allreduce", 8, 8192, "bfloat16", "tma", 4),
+    ("ring_rs_sm_w4_n4096_f16_c1", "ring", "build_reduce_scatter", 4, 4096, "float16", "sm", 1),
+    ("ring_ag_sm_w4_n4096_f16_c1", "ring", "build_allgather", 4, 4096, "float16", "sm", 1),
+    ("ring_a2a_sm_w4_n4096_bf16_c1", "ring", "build_alltoall", 4, 4096, "bfloat16", "sm", 1),
+    ("rhd_ar_sm_w8_n4096_f32_c1", "rhd", "build_allreduce", 8, 4096, "float32", "sm", 1),
+    ("rhd_ar_tma_w4_n1024_bf16_c1", "rhd", "build_allreduce", 4, 1024, "bfloat16", "tma", 1),
+    ("tree_ar_sm_w8_n1024_f32_c1", "tree", "build_allreduce", 8, 1024, "float32", "sm", 1),
+    ("tree_ar_tma_w4_n512_f16_c1", "tree", "build_allreduce", 4, 512, "float16", "tma", 1),
+]
+
+
+def main():
+    comp, ring, rhd, tree = load_reference_dsl()
+    algs = {"ring": ring.RingAllreduce, "rhd": rhd.RecursiveHalvingDoubling,
+            "tree": tree.TreeAllreduce}
+    os.makedirs(OUT, exist_ok=True)
+    index = []
+    for stem, alg, method, world, n, dtype, executor, ch in CASES:
+        for rank in range(world):
+            g = getattr(algs[alg](), method)(rank, world, n, dtype=dtype, executor=executor,
+                                             num_channels=ch)
+            text = comp.compile_to_json_string(g)
+            # compact re-serialisation keeps key order and values, drops the indent whitespace
+            doc = json.loads(text)
+            path = os.path.join(OUT, f"{stem}_rank{rank}.json")
+            with open(path, "w") as f:
+                json.dump(doc, f, separators=(",", ":"))
+                f.write("\n")
+        index.append({"stem": stem, "algorithm": alg, "method": method, "world_size": world,
+                      "tensor_size": n, "dtype": dtype, "executor": executor,
+                      "num_channels": ch})
+    with open(os.path.join(OUT, "index.json"), "w") as f:
+        json.dump(index, f, indent=1)
+        f.write("\n")
+    print(f"wrote {sum(c[3] for c in CASES)} graphs to {OUT}")
+
+
+if __name__ == "__main__":
+    main()
