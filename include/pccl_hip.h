@@ -1,0 +1,222 @@
+/*
+ * pccl_hip.h — C ABI of the MI355X (gfx950) executor plugin for PCCL's SM data path.
+ *
+ * One process, one GPU.  The R ranks of a schedule are R "virtual ranks": R rank buffers in this
+ * GPU's HBM, R per-rank graphs, R semaphore arrays folded into one linked program.  Each entry
+ * point names the reference interface it stands in for.  No C++ or torch types cross this
+ * boundary: plain pointers, sizes and ints.  Every function returns 0 on success or a negative
+ * pccl_status; the message of the last failure on the calling thread is pccl_hip_last_error().
+ */
+#ifndef PCCL_HIP_H_
+#define PCCL_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PCCL_HIP_MAX_VRANKS 64
+#define PCCL_HIP_MAX_CHANNELS 8     /* reference include/common/config.h:27 */
+#define PCCL_HIP_NUM_SIGNALS 4096   /* reference include/common/config.h:24 (ints per rank) */
+#define PCCL_HIP_MAX_FUSED_STEPS 128 /* reference include/common/config.h:28 */
+
+typedef enum {
+    PCCL_OK = 0,
+    PCCL_ERR_INVALID = -1,     /* bad argument */
+    PCCL_ERR_NOT_FOUND = -2,   /* unknown operation name / missing file */
+    PCCL_ERR_PARSE = -3,       /* malformed graph document, unknown primitive or dtype */
+    PCCL_ERR_LINK = -4,        /* ranks missing, deadlock, unbalanced signals, data race */
+    PCCL_ERR_HIP = -5,         /* a HIP runtime call failed */
+    PCCL_ERR_UNSUPPORTED = -6  /* valid request this build does not implement */
+} pccl_status;
+
+/* Element types, numbered like the reference's DataType (csrc/plugins/cuda/kernel/compute.h:13-19);
+ * PCCL_I32 is an extension (the reference rejects integer dtypes). */
+typedef enum { PCCL_F32 = 0, PCCL_F16 = 1, PCCL_BF16 = 2, PCCL_F8E4M3 = 3, PCCL_F8E5M2 = 4, PCCL_I32 = 5 } pccl_dtype;
+
+/* Reduction operators.  The reference runtime always sums; MAX / MIN honour the graph's
+ * params.reduce_op and are an extension. */
+typedef enum { PCCL_SUM = 0, PCCL_MAX = 1, PCCL_MIN = 2 } pccl_redop;
+
+/* Primitive type ids: reference csrc/plugins/cuda/kernel/primitive_config.h:7-57. */
+enum {
+    PCCL_PT_NOOP = 0,
+    PCCL_PT_REDUCE_F32 = 1,      /* +dtype 0..4 */
+    PCCL_PT_COPY_F32 = 6,        /* +dtype 0..4 */
+    PCCL_PT_WAIT_NOTIFY = 21,
+    PCCL_PT_NOTIFY = 22,
+    PCCL_PT_TMA_COPY_F32 = 28,   /* +dtype 0..4: executed as plain copy (the reference's SM fallback) */
+    PCCL_PT_TMA_REDUCE_F32 = 33, /* +dtype 0..4: executed as plain reduce */
+    PCCL_PT_REDUCE_I32 = 64,     /* extension ids, outside the reference's table */
+    PCCL_PT_COPY_I32 = 65
+};
+
+/* 32-byte trigger, field offsets of the reference's OpProxyTriggerCudaHandle /
+ * SignalProxyTriggerCudaHandle (csrc/plugins/cuda/kernel/proxy_trigger.h:8-30):
+ * data ops: offset_0/1/2 = remote/src/dst (reduce) or src/dst/- (copy), size in elements;
+ * signals: peer_rank = target (notify) or source (wait), offset_0 = signal id. */
+typedef struct {
+    int8_t primitive_type;
+    int8_t redop;       /* pccl_redop; byte 1 is padding in the reference */
+    int8_t pad_[2];
+    int32_t op_index;
+    int32_t peer_rank;
+    int32_t offset_0;
+    int32_t offset_1;
+    int32_t offset_2;
+    int32_t size;
+    int32_t reserved_;
+} pccl_trigger;
+
+/* Graph metadata per op: layout of the reference's PrimitiveMeta (include/engine/primitive.h:8-17). */
+typedef struct {
+    int32_t op_seq_index;
+    int32_t num_next_ops;
+    int32_t num_dependencies;
+    int32_t next_primitive_index[8];
+    int32_t device_type;   /* 0 host, 1 device */
+    int32_t channel;
+    uint64_t params[4];
+} pccl_primitive_meta;
+
+/* One fused step: layout of the reference's FusedStep (include/engine/fused_step.h:7-22). */
+typedef struct {
+    int8_t primitive_type;
+    int8_t pad_[3];
+    int32_t peer_rank;
+    int32_t offset_0;
+    int32_t offset_1;
+    int32_t offset_2;
+    int32_t size;
+    int32_t notify_signal_id;
+    int32_t notify_peer_rank;
+    int32_t wait_signal_id;
+    int32_t wait_peer_rank;
+    uint8_t has_notify;
+    uint8_t has_wait;
+    uint8_t pad2_[2];
+} pccl_fused_step;
+
+/* ------------------------------------------------------------------------------------------
+ * Host-only graph tools (no GPU needed).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct pccl_graph pccl_graph;
+typedef struct pccl_program pccl_program;
+
+/* Load one rank's JSON v2 graph.  Replaces GraphBuilder::loadFromFile + SmChannel/TmaChannel::parse
+ * (reference csrc/engine/graph_builder.cc:12-107; csrc/plugins/cuda/channels/sm_channel.h:26-96,
+ * tma_channel.h:27-81).  Missing file / no "operations" / an op without index|executor|primitive
+ * -> PCCL_ERR_NOT_FOUND / PCCL_ERR_PARSE (the reference returns false); unknown primitive or
+ * dtype -> PCCL_ERR_PARSE (the reference throws). */
+int pccl_graph_load_file(const char* path, pccl_graph** out);
+int pccl_graph_load_json(const char* text, size_t len, pccl_graph** out);
+/* Build a graph from arrays an engine has already parsed (reference GraphBuilder's operators_ /
+ * metadata_ vectors, include/engine/graph_builder.h).  dtype is taken from the primitive ids. */
+int pccl_graph_from_triggers(const pccl_trigger* triggers, const pccl_primitive_meta* meta, int n,
+                             const char* collective_type, pccl_graph** out);
+void pccl_graph_free(pccl_graph* g);
+int pccl_graph_num_ops(const pccl_graph* g);
+int pccl_graph_dtype(const pccl_graph* g);            /* pccl_dtype of tensor_info.dtype */
+int64_t pccl_graph_tensor_elems(const pccl_graph* g); /* product of tensor_info.shape, 0 if absent */
+const char* pccl_graph_collective_type(const pccl_graph* g);
+int pccl_graph_get_triggers(const pccl_graph* g, pccl_trigger* out, int cap);
+int pccl_graph_get_meta(const pccl_graph* g, pccl_primitive_meta* out, int cap);
+/* Collapse per-channel linear chains into fused steps.  Replaces GraphBuilder::buildFusedDescriptor
+ * (reference csrc/engine/graph_builder.cc:163-316).  Returns the number of steps, or
+ * PCCL_ERR_UNSUPPORTED when the reference would fall back to its dependency-counter runner
+ * (an op with >1 dependency or successor, a chain starting with a data op, >128 steps).
+ * channel_offsets must hold PCCL_HIP_MAX_CHANNELS+1 ints. */
+int pccl_graph_fused_steps(const pccl_graph* g, pccl_fused_step* steps, int cap,
+                           int* channel_offsets, int* num_channels);
+
+/* What the linker derived from R per-rank graphs. */
+typedef struct {
+    int32_t num_vranks;
+    int32_t dtype;
+    int32_t num_ops;            /* all primitives over all ranks */
+    int32_t num_data_ops;
+    int32_t num_levels;         /* longest dependency chain over data ops */
+    int32_t position_aligned;   /* 1 if every data op reads and writes the same element positions */
+    int32_t num_segments;       /* column plan: maximal position ranges with one op list */
+    int32_t residual_signals;   /* semaphores left non-zero by one execution (0 for balanced graphs) */
+    int64_t buffer_elems;       /* rank-buffer elements the graphs address (max offset+size) */
+    int64_t algorithmic_bytes;  /* sum over data ops: reduce 3*n*esize, copy 2*n*esize */
+    int64_t column_load_bytes;  /* bytes the column plan loads / stores from memory per execution */
+    int64_t column_store_bytes;
+    int32_t num_items;          /* stepwise plan: (op, tile) work items */
+    int32_t reserved_;
+} pccl_program_info;
+
+/* One data op of the linked program, for inspection and tests. */
+typedef struct {
+    int32_t rank, channel, op_index, is_reduce, redop, peer_rank, level, num_deps;
+    int64_t offset_0, offset_1, offset_2, size;
+    int32_t deps[8];            /* indices into the linked op array (first 8) */
+} pccl_linked_op;
+
+/* Link R graphs (index = rank) into one program: pair the k-th notify arriving at (target, id) with
+ * the k-th wait on it (counting semaphores, reference cuda_executor.cu:414-445), derive data
+ * dependencies, detect deadlock and unordered conflicting accesses.  No reference counterpart:
+ * the reference runs one process per rank and synchronises at run time. */
+int pccl_program_link(const pccl_graph* const* graphs, int num_vranks, pccl_program** out);
+void pccl_program_free(pccl_program* p);
+int pccl_program_get_info(const pccl_program* p, pccl_program_info* out);
+int pccl_program_get_ops(const pccl_program* p, pccl_linked_op* out, int cap);
+
+/* ------------------------------------------------------------------------------------------
+ * Device executor.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct pccl_hip_ctx pccl_hip_ctx;
+
+/* Engine construction: replaces Engine::Engine() + BufferManager + MemoryLayout::initialize
+ * (reference csrc/engine_c.cc:82-164, csrc/engine/memory_layout.cc:8-138).  Rank buffers are
+ * sized on demand from the registered graphs instead of one fixed 1 GiB buffer. */
+int pccl_hip_create(pccl_hip_ctx** out, int device, int num_vranks);
+int pccl_hip_destroy(pccl_hip_ctx* ctx);
+
+/* Engine::regOp(name, filename) for one virtual rank (reference csrc/engine_c.cc:166-201). */
+int pccl_hip_register_file(pccl_hip_ctx* ctx, const char* name, int vrank, const char* path);
+int pccl_hip_register_json(pccl_hip_ctx* ctx, const char* name, int vrank, const char* text, size_t len);
+int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
+                               const pccl_trigger* triggers, const pccl_primitive_meta* meta, int n,
+                               const char* collective_type);
+
+/* Options, the counterpart of the reference's environment switches (csrc/plugins/cuda/cuda_device.cc:
+ * 289-298, csrc/engine_c.cc:351): key "mode" = "auto" | "column" | "stepwise";
+ * "num_blocks" = workgroups of the persistent launch (0 = fill the device);
+ * "check_races" = "0" | "1". */
+int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
+
+/* Engine::exeOp / exeOpAsync (reference csrc/engine_c.cc:269-560): for every virtual rank r copy
+ * inputs[r] into rank buffer r (allgather: at r*in_bytes), run the program, copy the result to
+ * outputs[r] (allreduce/default: buffer[0..out_bytes); reduce_scatter: chunk r; alltoall: own chunk
+ * + scratch region).  All work is enqueued on `stream` (a hipStream_t, NULL = default stream);
+ * sync != 0 waits for it. */
+int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inputs,
+                     void* const* outputs, size_t in_bytes, size_t out_bytes, void* stream, int sync);
+/* Zero-copy variant: bufs[r] IS rank buffer r (buf_bytes each, 16-byte aligned); no staging. */
+int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
+                             void* stream, int sync);
+/* Engine::syncOp / Engine::resetSignals (reference csrc/engine_c.cc:562-593). */
+int pccl_hip_sync(pccl_hip_ctx* ctx, const char* name);
+int pccl_hip_reset_signals(pccl_hip_ctx* ctx, const char* name);
+
+int pccl_hip_op_info(pccl_hip_ctx* ctx, const char* name, pccl_program_info* out);
+/* Duration of the most recent program launch of `name` (kernel only, HIP events on its stream). */
+int pccl_hip_last_kernel_ms(pccl_hip_ctx* ctx, const char* name, float* ms);
+
+/* The two data primitives on their own (reference executeReduce / executeCopy,
+ * csrc/plugins/cuda/cuda_executor.cu:60-101 -> vector_add / vector_copy, kernel/compute.h:21-102):
+ * c[i] = a[i] (+|max|min) b[i], dst[i] = src[i]; any alignment, any n. */
+int pccl_hip_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream);
+int pccl_hip_copy(int dtype, const void* src, void* dst, size_t n, void* stream);
+
+const char* pccl_hip_last_error(void);
+const char* pccl_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PCCL_HIP_H_ */

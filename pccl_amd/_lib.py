@@ -1,0 +1,236 @@
+"""ctypes binding of libpccl_hip.so (the C ABI declared in include/pccl_hip.h).
+
+There is no fallback: if the library is missing the import of anything that needs it raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libpccl_hip.so")
+
+MAX_VRANKS = 64
+MAX_CHANNELS = 8
+
+OK, ERR_INVALID, ERR_NOT_FOUND, ERR_PARSE, ERR_LINK, ERR_HIP, ERR_UNSUPPORTED = 0, -1, -2, -3, -4, -5, -6
+
+DTYPE_ID = {"float32": 0, "float16": 1, "bfloat16": 2, "float8_e4m3": 3, "float8_e5m2": 4, "int32": 5}
+REDOP_ID = {"sum": 0, "max": 1, "min": 2}
+
+
+class Trigger(ctypes.Structure):
+    _fields_ = [("primitive_type", ctypes.c_int8), ("redop", ctypes.c_int8), ("pad_", ctypes.c_int8 * 2),
+                ("op_index", ctypes.c_int32), ("peer_rank", ctypes.c_int32), ("offset_0", ctypes.c_int32),
+                ("offset_1", ctypes.c_int32), ("offset_2", ctypes.c_int32), ("size", ctypes.c_int32),
+                ("reserved_", ctypes.c_int32)]
+
+
+class PrimitiveMeta(ctypes.Structure):
+    _fields_ = [("op_seq_index", ctypes.c_int32), ("num_next_ops", ctypes.c_int32),
+                ("num_dependencies", ctypes.c_int32), ("next_primitive_index", ctypes.c_int32 * 8),
+                ("device_type", ctypes.c_int32), ("channel", ctypes.c_int32), ("params", ctypes.c_uint64 * 4)]
+
+
+class FusedStep(ctypes.Structure):
+    _fields_ = [("primitive_type", ctypes.c_int8), ("pad_", ctypes.c_int8 * 3), ("peer_rank", ctypes.c_int32),
+                ("offset_0", ctypes.c_int32), ("offset_1", ctypes.c_int32), ("offset_2", ctypes.c_int32),
+                ("size", ctypes.c_int32), ("notify_signal_id", ctypes.c_int32),
+                ("notify_peer_rank", ctypes.c_int32), ("wait_signal_id", ctypes.c_int32),
+                ("wait_peer_rank", ctypes.c_int32), ("has_notify", ctypes.c_uint8), ("has_wait", ctypes.c_uint8),
+                ("pad2_", ctypes.c_uint8 * 2)]
+
+
+class ProgramInfo(ctypes.Structure):
+    _fields_ = [("num_vranks", ctypes.c_int32), ("dtype", ctypes.c_int32), ("num_ops", ctypes.c_int32),
+                ("num_data_ops", ctypes.c_int32), ("num_levels", ctypes.c_int32),
+                ("position_aligned", ctypes.c_int32), ("num_segments", ctypes.c_int32),
+                ("residual_signals", ctypes.c_int32), ("buffer_elems", ctypes.c_int64),
+                ("algorithmic_bytes", ctypes.c_int64), ("column_load_bytes", ctypes.c_int64),
+                ("column_store_bytes", ctypes.c_int64), ("num_items", ctypes.c_int32),
+                ("reserved_", ctypes.c_int32)]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_ if not n.endswith("_")}
+
+
+class LinkedOp(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("rank", "channel", "op_index", "is_reduce", "redop",
+                                              "peer_rank", "level", "num_deps")] + \
+               [(n, ctypes.c_int64) for n in ("offset_0", "offset_1", "offset_2", "size")] + \
+               [("deps", ctypes.c_int32 * 8)]
+
+
+class PcclError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(message)
+        self.code = code
+
+
+_lib = None
+
+# every symbol include/pccl_hip.h declares
+EXPORTS = [
+    "pccl_graph_load_file", "pccl_graph_load_json", "pccl_graph_from_triggers", "pccl_graph_free",
+    "pccl_graph_num_ops", "pccl_graph_dtype", "pccl_graph_tensor_elems", "pccl_graph_collective_type",
+    "pccl_graph_get_triggers", "pccl_graph_get_meta", "pccl_graph_fused_steps", "pccl_program_link",
+    "pccl_program_free", "pccl_program_get_info", "pccl_program_get_ops", "pccl_hip_create",
+    "pccl_hip_destroy", "pccl_hip_register_file", "pccl_hip_register_json", "pccl_hip_register_triggers",
+    "pccl_hip_set_option", "pccl_hip_execute", "pccl_hip_execute_inplace", "pccl_hip_sync",
+    "pccl_hip_reset_signals", "pccl_hip_op_info", "pccl_hip_last_kernel_ms", "pccl_hip_reduce",
+    "pccl_hip_copy", "pccl_hip_last_error", "pccl_hip_version",
+]
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m pccl_amd.build` (hipcc, gfx950). "
+            "The executor has no CPU or PyTorch fallback.")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, cp, i32, i64, sz = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
+    P = ctypes.POINTER
+    sigs = {
+        "pccl_graph_load_file": (i32, [cp, P(vp)]),
+        "pccl_graph_load_json": (i32, [cp, sz, P(vp)]),
+        "pccl_graph_from_triggers": (i32, [P(Trigger), P(PrimitiveMeta), i32, cp, P(vp)]),
+        "pccl_graph_free": (None, [vp]),
+        "pccl_graph_num_ops": (i32, [vp]),
+        "pccl_graph_dtype": (i32, [vp]),
+        "pccl_graph_tensor_elems": (i64, [vp]),
+        "pccl_graph_collective_type": (cp, [vp]),
+        "pccl_graph_get_triggers": (i32, [vp, P(Trigger), i32]),
+        "pccl_graph_get_meta": (i32, [vp, P(PrimitiveMeta), i32]),
+        "pccl_graph_fused_steps": (i32, [vp, P(FusedStep), i32, P(ctypes.c_int), P(ctypes.c_int)]),
+        "pccl_program_link": (i32, [P(vp), i32, P(vp)]),
+        "pccl_program_free": (None, [vp]),
+        "pccl_program_get_info": (i32, [vp, P(ProgramInfo)]),
+        "pccl_program_get_ops": (i32, [vp, P(LinkedOp), i32]),
+        "pccl_hip_create": (i32, [P(vp), i32, i32]),
+        "pccl_hip_destroy": (i32, [vp]),
+        "pccl_hip_register_file": (i32, [vp, cp, i32, cp]),
+        "pccl_hip_register_json": (i32, [vp, cp, i32, cp, sz]),
+        "pccl_hip_register_triggers": (i32, [vp, cp, i32, P(Trigger), P(PrimitiveMeta), i32, cp]),
+        "pccl_hip_set_option": (i32, [vp, cp, cp]),
+        "pccl_hip_execute": (i32, [vp, cp, P(vp), P(vp), sz, sz, vp, i32]),
+        "pccl_hip_execute_inplace": (i32, [vp, cp, P(vp), sz, vp, i32]),
+        "pccl_hip_sync": (i32, [vp, cp]),
+        "pccl_hip_reset_signals": (i32, [vp, cp]),
+        "pccl_hip_op_info": (i32, [vp, cp, P(ProgramInfo)]),
+        "pccl_hip_last_kernel_ms": (i32, [vp, cp, P(ctypes.c_float)]),
+        "pccl_hip_reduce": (i32, [i32, i32, vp, vp, vp, sz, vp]),
+        "pccl_hip_copy": (i32, [i32, vp, vp, sz, vp]),
+        "pccl_hip_last_error": (cp, []),
+        "pccl_hip_version": (cp, []),
+    }
+    for name, (res, args) in sigs.items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = L
+    return L
+
+
+def check(rc: int) -> int:
+    if rc < 0:
+        raise PcclError(rc, lib().pccl_hip_last_error().decode(errors="replace"))
+    return rc
+
+
+# -- host-only helpers (no GPU needed) ---------------------------------------------------------
+
+class HostGraph:
+    """One rank's loaded graph (host side only)."""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    @classmethod
+    def from_json(cls, text: str) -> "HostGraph":
+        h = ctypes.c_void_p()
+        data = text.encode()
+        check(lib().pccl_graph_load_json(data, len(data), ctypes.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def from_file(cls, path: str) -> "HostGraph":
+        h = ctypes.c_void_p()
+        check(lib().pccl_graph_load_file(path.encode(), ctypes.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def from_triggers(cls, triggers, meta, collective_type: str = "") -> "HostGraph":
+        h = ctypes.c_void_p()
+        n = len(triggers)
+        check(lib().pccl_graph_from_triggers(triggers, meta, n, collective_type.encode(), ctypes.byref(h)))
+        return cls(h)
+
+    def __del__(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.pccl_graph_free(self._h)
+            self._h = None
+
+    @property
+    def num_ops(self) -> int:
+        return lib().pccl_graph_num_ops(self._h)
+
+    @property
+    def dtype(self) -> int:
+        return lib().pccl_graph_dtype(self._h)
+
+    @property
+    def tensor_elems(self) -> int:
+        return lib().pccl_graph_tensor_elems(self._h)
+
+    @property
+    def collective_type(self) -> str:
+        return lib().pccl_graph_collective_type(self._h).decode()
+
+    def triggers(self):
+        n = self.num_ops
+        arr = (Trigger * max(n, 1))()
+        check(lib().pccl_graph_get_triggers(self._h, arr, n))
+        return arr, n
+
+    def meta(self):
+        n = self.num_ops
+        arr = (PrimitiveMeta * max(n, 1))()
+        check(lib().pccl_graph_get_meta(self._h, arr, n))
+        return arr, n
+
+    def fused_steps(self):
+        """Returns (steps, channel_offsets) or raises PcclError(ERR_UNSUPPORTED)."""
+        steps = (FusedStep * 128)()
+        offs = (ctypes.c_int * (MAX_CHANNELS + 1))()
+        nch = ctypes.c_int()
+        n = check(lib().pccl_graph_fused_steps(self._h, steps, 128, offs, ctypes.byref(nch)))
+        return [steps[i] for i in range(n)], [offs[i] for i in range(nch.value + 1)]
+
+
+class HostProgram:
+    """R graphs linked into one program (host side only)."""
+
+    def __init__(self, graphs):
+        arr = (ctypes.c_void_p * len(graphs))(*[g._h for g in graphs])
+        h = ctypes.c_void_p()
+        check(lib().pccl_program_link(arr, len(graphs), ctypes.byref(h)))
+        self._h = h
+        self._graphs = graphs
+
+    def __del__(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.pccl_program_free(self._h)
+            self._h = None
+
+    def info(self) -> dict:
+        out = ProgramInfo()
+        check(lib().pccl_program_get_info(self._h, ctypes.byref(out)))
+        return out.as_dict()
+
+    def ops(self):
+        n = self.info()["num_data_ops"]
+        arr = (LinkedOp * max(n, 1))()
+        check(lib().pccl_program_get_ops(self._h, arr, n))
+        return [arr[i] for i in range(n)]

@@ -1,0 +1,621 @@
+// C ABI: host-only graph tools and the device executor context.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "graph.h"
+#include "kernels.h"
+#include "program.h"
+
+using namespace pccl_hip;
+
+struct pccl_graph { RankGraph g; };
+struct pccl_program { Program p; };
+
+namespace {
+
+thread_local std::string t_err;
+
+int fail(int code, const std::string& msg) {
+    t_err = msg;
+    return code;
+}
+
+template <class F>
+int guarded(F&& f) {
+    try {
+        return f();
+    } catch (const Error& e) {
+        return fail(e.code, e.msg);
+    } catch (const std::bad_alloc&) {
+        return fail(PCCL_ERR_INVALID, "out of host memory");
+    } catch (const std::exception& e) {
+        return fail(PCCL_ERR_INVALID, e.what());
+    }
+}
+
+#define HIP_TRY(expr)                                                                                   \
+    do {                                                                                                \
+        hipError_t e_ = (expr);                                                                         \
+        if (e_ != hipSuccess) throw Error{PCCL_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)}; \
+    } while (0)
+
+void fill_info(const Program& p, pccl_program_info* out) {
+    std::memset(out, 0, sizeof(*out));
+    out->num_vranks = p.R;
+    out->dtype = p.dtype;
+    out->num_ops = p.num_all_ops;
+    out->num_data_ops = (int)p.ops.size();
+    out->num_levels = p.num_levels;
+    out->position_aligned = p.position_aligned;
+    out->num_segments = (int)p.segs.size();
+    out->residual_signals = p.residual_signals;
+    out->buffer_elems = p.buffer_elems;
+    out->algorithmic_bytes = p.algorithmic_bytes;
+    out->column_load_bytes = p.column_load_bytes;
+    out->column_store_bytes = p.column_store_bytes;
+    out->num_items = (int)p.num_items;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* pccl_hip_last_error(void) { return t_err.c_str(); }
+const char* pccl_hip_version(void) { return "pccl-hip 0.1 (gfx950)"; }
+
+// ------------------------------------------------------------------------------- graph tools
+
+int pccl_graph_load_file(const char* path, pccl_graph** out) {
+    return guarded([&] {
+        if (!path || !out) return fail(PCCL_ERR_INVALID, "null argument");
+        auto g = std::make_unique<pccl_graph>();
+        g->g = load_graph_file(path);
+        *out = g.release();
+        return 0;
+    });
+}
+
+int pccl_graph_load_json(const char* text, size_t len, pccl_graph** out) {
+    return guarded([&] {
+        if (!text || !out) return fail(PCCL_ERR_INVALID, "null argument");
+        auto g = std::make_unique<pccl_graph>();
+        g->g = load_graph_json(text, len);
+        *out = g.release();
+        return 0;
+    });
+}
+
+int pccl_graph_from_triggers(const pccl_trigger* triggers, const pccl_primitive_meta* meta, int n,
+                             const char* collective_type, pccl_graph** out) {
+    return guarded([&] {
+        if (!out) return fail(PCCL_ERR_INVALID, "null argument");
+        auto g = std::make_unique<pccl_graph>();
+        g->g = graph_from_triggers(triggers, meta, n, collective_type);
+        *out = g.release();
+        return 0;
+    });
+}
+
+void pccl_graph_free(pccl_graph* g) { delete g; }
+int pccl_graph_num_ops(const pccl_graph* g) { return g ? (int)g->g.ops.size() : PCCL_ERR_INVALID; }
+int pccl_graph_dtype(const pccl_graph* g) { return g ? g->g.dtype : PCCL_ERR_INVALID; }
+int64_t pccl_graph_tensor_elems(const pccl_graph* g) { return g ? g->g.tensor_elems : 0; }
+const char* pccl_graph_collective_type(const pccl_graph* g) { return g ? g->g.collective_type.c_str() : ""; }
+
+int pccl_graph_get_triggers(const pccl_graph* g, pccl_trigger* out, int cap) {
+    if (!g || !out) return fail(PCCL_ERR_INVALID, "null argument");
+    std::vector<pccl_trigger> t;
+    graph_to_triggers(g->g, &t, nullptr);
+    int n = std::min<int>(cap, (int)t.size());
+    std::memcpy(out, t.data(), sizeof(pccl_trigger) * n);
+    return (int)t.size();
+}
+
+int pccl_graph_get_meta(const pccl_graph* g, pccl_primitive_meta* out, int cap) {
+    if (!g || !out) return fail(PCCL_ERR_INVALID, "null argument");
+    std::vector<pccl_primitive_meta> m;
+    graph_to_triggers(g->g, nullptr, &m);
+    int n = std::min<int>(cap, (int)m.size());
+    std::memcpy(out, m.data(), sizeof(pccl_primitive_meta) * n);
+    return (int)m.size();
+}
+
+int pccl_graph_fused_steps(const pccl_graph* g, pccl_fused_step* steps, int cap, int* channel_offsets,
+                           int* num_channels) {
+    if (!g) return fail(PCCL_ERR_INVALID, "null argument");
+    std::vector<pccl_fused_step> s;
+    std::vector<int> off;
+    if (!build_fused_steps(g->g, &s, &off))
+        return fail(PCCL_ERR_UNSUPPORTED, "graph is not a set of per-channel linear chains of at most 128 steps");
+    if (steps) std::memcpy(steps, s.data(), sizeof(pccl_fused_step) * std::min<int>(cap, (int)s.size()));
+    if (channel_offsets)
+        for (size_t i = 0; i < off.size() && i <= PCCL_HIP_MAX_CHANNELS; ++i) channel_offsets[i] = off[i];
+    if (num_channels) *num_channels = (int)off.size() - 1;
+    return (int)s.size();
+}
+
+int pccl_program_link(const pccl_graph* const* graphs, int num_vranks, pccl_program** out) {
+    return guarded([&] {
+        if (!graphs || !out) return fail(PCCL_ERR_INVALID, "null argument");
+        std::vector<const RankGraph*> gs;
+        for (int r = 0; r < num_vranks; ++r) gs.push_back(graphs[r] ? &graphs[r]->g : nullptr);
+        auto p = std::make_unique<pccl_program>();
+        p->p = link_program(gs, LinkOptions{});
+        *out = p.release();
+        return 0;
+    });
+}
+
+void pccl_program_free(pccl_program* p) { delete p; }
+
+int pccl_program_get_info(const pccl_program* p, pccl_program_info* out) {
+    if (!p || !out) return fail(PCCL_ERR_INVALID, "null argument");
+    fill_info(p->p, out);
+    return 0;
+}
+
+int pccl_program_get_ops(const pccl_program* p, pccl_linked_op* out, int cap) {
+    if (!p || !out) return fail(PCCL_ERR_INVALID, "null argument");
+    int n = std::min<int>(cap, (int)p->p.ops.size());
+    for (int k = 0; k < n; ++k) {
+        const LinkedOp& L = p->p.ops[k];
+        pccl_linked_op& o = out[k];
+        std::memset(&o, 0, sizeof(o));
+        o.rank = L.rank; o.channel = L.channel; o.op_index = L.index; o.is_reduce = L.is_reduce;
+        o.redop = L.redop; o.peer_rank = L.peer; o.level = L.level; o.num_deps = (int)L.deps.size();
+        o.offset_0 = L.off0; o.offset_1 = L.off1; o.offset_2 = L.off2; o.size = L.size;
+        for (size_t d = 0; d < L.deps.size() && d < 8; ++d) o.deps[d] = L.deps[d];
+    }
+    return (int)p->p.ops.size();
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------------------- device context
+
+namespace {
+
+struct DevBuf {
+    void* p = nullptr;
+    size_t bytes = 0;
+    void release() { if (p) { (void)hipFree(p); p = nullptr; bytes = 0; } }
+    void upload(const void* src, size_t n) {
+        release();
+        if (n == 0) return;
+        HIP_TRY(hipMalloc(&p, n));
+        bytes = n;
+        HIP_TRY(hipMemcpy(p, src, n, hipMemcpyHostToDevice));
+    }
+};
+
+struct OpEntry {
+    std::vector<std::unique_ptr<RankGraph>> graphs;
+    bool linked = false;
+    Program prog;
+    DevBuf segs, instrs, fifo, step_ops, step_deps, item_op, state;
+    int64_t total_tiles = 0;
+    int vecs_per_thread = 0;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    bool timed = false;
+    void release() {
+        segs.release(); instrs.release(); fifo.release(); step_ops.release(); step_deps.release();
+        item_op.release(); state.release();
+        if (ev0) (void)hipEventDestroy(ev0);
+        if (ev1) (void)hipEventDestroy(ev1);
+        ev0 = ev1 = nullptr;
+        linked = false; timed = false;
+    }
+};
+
+enum class Mode { Auto, Column, Stepwise };
+
+}  // namespace
+
+struct pccl_hip_ctx {
+    int device = 0;
+    int R = 0;
+    std::mutex mu;
+    std::map<std::string, OpEntry> ops;
+    std::vector<char*> bufs;   // engine-owned rank buffers (staged execution)
+    size_t buf_bytes = 0;
+    Mode mode = Mode::Auto;
+    int num_blocks = 0;
+    int vecs_per_thread = 2;
+    bool check_races = true;
+    bool timing = false;
+    int fifo_depth = 0;
+    int64_t step_tile_bytes = 128 * 1024;
+    hipStream_t last_stream = nullptr;
+};
+
+namespace {
+
+void ensure_buffers(pccl_hip_ctx* ctx, size_t bytes) {
+    if (bytes <= ctx->buf_bytes) return;
+    // every registered op aliases the same rank buffers (as in the reference, engine_c.cc:191-196)
+    HIP_TRY(hipDeviceSynchronize());
+    for (char*& b : ctx->bufs) { if (b) (void)hipFree(b); b = nullptr; }
+    ctx->buf_bytes = 0;
+    size_t rounded = (bytes + 4095) & ~(size_t)4095;
+    for (int r = 0; r < ctx->R; ++r) {
+        void* p = nullptr;
+        HIP_TRY(hipMalloc(&p, rounded));
+        ctx->bufs[r] = (char*)p;
+    }
+    ctx->buf_bytes = rounded;
+}
+
+void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
+    if (e.linked) return;
+    std::vector<const RankGraph*> gs;
+    for (int r = 0; r < ctx->R; ++r) gs.push_back(e.graphs[r].get());
+    LinkOptions opt;
+    opt.check_races = ctx->check_races;
+    opt.fifo_depth = ctx->fifo_depth;
+    opt.step_tile_bytes = ctx->step_tile_bytes;
+    e.prog = link_program(gs, opt);
+    const Program& P = e.prog;
+    const int es = elem_size(P.dtype);
+    const int ve = 16 / es;
+    e.vecs_per_thread = ctx->vecs_per_thread;
+
+    // column plan
+    if (P.position_aligned) {
+        std::vector<DevColSegment> ds(P.segs.size());
+        int64_t tiles = 0;
+        const int64_t tile_v = 256 * (int64_t)e.vecs_per_thread;
+        for (size_t i = 0; i < P.segs.size(); ++i) {
+            const ColSegment& s = P.segs[i];
+            DevColSegment& d = ds[i];
+            d.start = s.start; d.end = s.end;
+            d.first_vec = s.start / ve;
+            int64_t last_vec = (s.end - 1) / ve;
+            d.first_tile = tiles;
+            tiles += (last_vec - d.first_vec + 1 + tile_v - 1) / tile_v;
+            d.prog_start = s.prog_start; d.prog_len = s.prog_len;
+            d.fifo_start = s.fifo_start; d.fifo_len = s.fifo_len;
+        }
+        e.total_tiles = tiles;
+        e.segs.upload(ds.data(), ds.size() * sizeof(DevColSegment));
+        e.instrs.upload(P.col_instrs.data(), P.col_instrs.size() * sizeof(ColInstr));
+        e.fifo.upload(P.col_fifo.data(), P.col_fifo.size());
+    }
+    // stepwise plan
+    {
+        std::vector<DevStepOp> so(P.ops.size());
+        std::vector<int32_t> item_op((size_t)P.num_items);
+        for (size_t k = 0; k < P.ops.size(); ++k) {
+            const LinkedOp& L = P.ops[k];
+            DevStepOp& d = so[k];
+            d.off0 = L.off0; d.off1 = L.off1; d.off2 = L.off2; d.size = L.size;
+            d.self = L.rank; d.peer = L.peer; d.is_reduce = L.is_reduce; d.redop = L.redop;
+            d.first_item = P.step_ops[k].first_item; d.ntiles = P.step_ops[k].ntiles;
+            d.dep_start = P.step_ops[k].dep_start; d.ndeps = P.step_ops[k].ndeps;
+            if (d.ndeps > 256) throw Error{PCCL_ERR_UNSUPPORTED, "a data op with more than 256 direct predecessors"};
+            for (int t = 0; t < d.ntiles; ++t) item_op[(size_t)d.first_item + t] = (int32_t)k;
+        }
+        e.step_ops.upload(so.data(), so.size() * sizeof(DevStepOp));
+        e.step_deps.upload(P.step_deps.data(), P.step_deps.size() * sizeof(int32_t));
+        e.item_op.upload(item_op.data(), item_op.size() * sizeof(int32_t));
+        std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * (P.ops.size() + 1), 0);
+        e.state.upload(zeros.data(), zeros.size());
+    }
+    HIP_TRY(hipEventCreate(&e.ev0));
+    HIP_TRY(hipEventCreate(&e.ev1));
+    e.linked = true;
+}
+
+OpEntry& find_entry(pccl_hip_ctx* ctx, const char* name) {
+    auto it = ctx->ops.find(name ? name : "");
+    if (it == ctx->ops.end()) throw Error{PCCL_ERR_NOT_FOUND, std::string("Unknown operation: ") + (name ? name : "(null)")};
+    return it->second;
+}
+
+// Enqueue the program on `stream` over the rank buffers `rank_bufs` (R pointers).
+void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t buf_bytes, hipStream_t stream) {
+    const Program& P = e.prog;
+    const int es = elem_size(P.dtype);
+    if ((size_t)P.buffer_elems * es > buf_bytes)
+        throw Error{PCCL_ERR_INVALID, "rank buffers of " + std::to_string(buf_bytes) + " bytes are smaller than the " + std::to_string((size_t)P.buffer_elems * es) + " bytes the graph addresses"};
+    if (P.ops.empty()) return;
+    RankPtrs ptrs;
+    std::memset(&ptrs, 0, sizeof(ptrs));
+    bool aligned16 = true;
+    for (int r = 0; r < ctx->R; ++r) {
+        if (!rank_bufs[r]) throw Error{PCCL_ERR_INVALID, "null rank buffer " + std::to_string(r)};
+        if ((uintptr_t)rank_bufs[r] % es) throw Error{PCCL_ERR_INVALID, "rank buffer " + std::to_string(r) + " is not aligned to the element size"};
+        if ((uintptr_t)rank_bufs[r] & 15) aligned16 = false;
+        ptrs.p[r] = rank_bufs[r];
+        ptrs.p[PCCL_HIP_MAX_VRANKS + r] = rank_bufs[r];
+    }
+    bool column = P.position_aligned && aligned16;
+    if (ctx->mode == Mode::Stepwise) column = false;
+    if (ctx->mode == Mode::Column && !column)
+        throw Error{PCCL_ERR_UNSUPPORTED, P.position_aligned ? "column mode needs 16-byte aligned rank buffers" : "column mode needs every data op to read and write the same element positions"};
+    if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
+    int rc;
+    if (column) {
+        ColumnLaunch L{};
+        L.segs = (const DevColSegment*)e.segs.p; L.num_segs = (int)P.segs.size();
+        L.instrs = (const uint64_t*)e.instrs.p; L.fifo = (const uint8_t*)e.fifo.p;
+        L.total_tiles = e.total_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
+        L.num_blocks = ctx->num_blocks;
+        rc = launch_column(L, ptrs, stream);
+    } else {
+        StepwiseLaunch L{};
+        L.ops = (const DevStepOp*)e.step_ops.p; L.num_ops = (int)P.ops.size();
+        L.deps = (const int32_t*)e.step_deps.p; L.item_op = (const int32_t*)e.item_op.p;
+        L.num_items = (int)P.num_items; L.tile_elems = P.tile_elems; L.state = (StepState*)e.state.p;
+        L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
+        rc = launch_stepwise(L, ptrs, stream);
+    }
+    if (rc != 0) throw Error{PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)};
+    if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, stream)); e.timed = true; }
+}
+
+int register_graph(pccl_hip_ctx* ctx, const char* name, int vrank, RankGraph&& g) {
+    if (!ctx || !name) return fail(PCCL_ERR_INVALID, "null argument");
+    if (vrank < 0 || vrank >= ctx->R) return fail(PCCL_ERR_INVALID, "virtual rank " + std::to_string(vrank) + " outside 0.." + std::to_string(ctx->R - 1));
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    HIP_TRY(hipSetDevice(ctx->device));
+    OpEntry& e = ctx->ops[name];
+    if (e.graphs.empty()) e.graphs.resize(ctx->R);
+    if (e.linked) { HIP_TRY(hipDeviceSynchronize()); e.release(); }  // re-registration replaces the op
+    e.graphs[vrank] = std::make_unique<RankGraph>(std::move(g));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pccl_hip_create(pccl_hip_ctx** out, int device, int num_vranks) {
+    return guarded([&] {
+        if (!out) return fail(PCCL_ERR_INVALID, "null argument");
+        if (num_vranks < 1 || num_vranks > PCCL_HIP_MAX_VRANKS)
+            return fail(PCCL_ERR_INVALID, "num_vranks must be 1.." + std::to_string(PCCL_HIP_MAX_VRANKS));
+        int count = 0;
+        if (hipGetDeviceCount(&count) != hipSuccess || count <= 0)
+            return fail(PCCL_ERR_HIP, "no HIP device is visible: the executor has no CPU fallback");
+        if (device < 0 || device >= count) return fail(PCCL_ERR_INVALID, "device index out of range");
+        HIP_TRY(hipSetDevice(device));
+        auto ctx = std::make_unique<pccl_hip_ctx>();
+        ctx->device = device;
+        ctx->R = num_vranks;
+        ctx->bufs.assign(num_vranks, nullptr);
+        if (const char* nb = std::getenv("PCCL_NUM_BLOCKS")) ctx->num_blocks = std::atoi(nb);
+        if (std::getenv("PCCL_DISABLE_FUSED")) ctx->mode = Mode::Stepwise;
+        *out = ctx.release();
+        return 0;
+    });
+}
+
+int pccl_hip_destroy(pccl_hip_ctx* ctx) {
+    if (!ctx) return 0;
+    (void)hipSetDevice(ctx->device);
+    (void)hipDeviceSynchronize();
+    for (auto& kv : ctx->ops) kv.second.release();
+    for (char* b : ctx->bufs) if (b) (void)hipFree(b);
+    delete ctx;
+    return 0;
+}
+
+int pccl_hip_register_file(pccl_hip_ctx* ctx, const char* name, int vrank, const char* path) {
+    return guarded([&] {
+        if (!path) return fail(PCCL_ERR_INVALID, "null path");
+        return register_graph(ctx, name, vrank, load_graph_file(path));
+    });
+}
+
+int pccl_hip_register_json(pccl_hip_ctx* ctx, const char* name, int vrank, const char* text, size_t len) {
+    return guarded([&] {
+        if (!text) return fail(PCCL_ERR_INVALID, "null text");
+        return register_graph(ctx, name, vrank, load_graph_json(text, len));
+    });
+}
+
+int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank, const pccl_trigger* triggers,
+                               const pccl_primitive_meta* meta, int n, const char* collective_type) {
+    return guarded([&] { return register_graph(ctx, name, vrank, graph_from_triggers(triggers, meta, n, collective_type)); });
+}
+
+int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
+    return guarded([&] {
+        if (!ctx || !key || !value) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        std::string k = key, v = value;
+        bool relink = false;
+        if (k == "mode") {
+            if (v == "auto") ctx->mode = Mode::Auto;
+            else if (v == "column") ctx->mode = Mode::Column;
+            else if (v == "stepwise") ctx->mode = Mode::Stepwise;
+            else return fail(PCCL_ERR_INVALID, "mode must be auto, column or stepwise");
+        } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
+        else if (k == "timing") ctx->timing = std::atoi(value) != 0;
+        else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
+        else if (k == "vecs_per_thread") {
+            int u = std::atoi(value);
+            if (u != 1 && u != 2 && u != 4) return fail(PCCL_ERR_INVALID, "vecs_per_thread must be 1, 2 or 4");
+            ctx->vecs_per_thread = u; relink = true;
+        } else if (k == "fifo_depth") { ctx->fifo_depth = std::atoi(value); relink = true; }
+        else if (k == "step_tile_bytes") {
+            int64_t b = std::atoll(value);
+            if (b < 4096 || b % 4096) return fail(PCCL_ERR_INVALID, "step_tile_bytes must be a positive multiple of 4096");
+            ctx->step_tile_bytes = b; relink = true;
+        } else return fail(PCCL_ERR_INVALID, "unknown option '" + k + "'");
+        if (relink) {
+            HIP_TRY(hipSetDevice(ctx->device));
+            HIP_TRY(hipDeviceSynchronize());
+            for (auto& kv : ctx->ops) kv.second.release();
+        }
+        return 0;
+    });
+}
+
+int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inputs, void* const* outputs,
+                     size_t in_bytes, size_t out_bytes, void* stream, int sync) {
+    return guarded([&] {
+        if (!ctx || !inputs || !outputs) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        HIP_TRY(hipSetDevice(ctx->device));
+        OpEntry& e = find_entry(ctx, name);
+        link_entry(ctx, e);
+        const Program& P = e.prog;
+        const int R = ctx->R;
+        const size_t es = elem_size(P.dtype);
+        const std::string& ct = P.collective_type;
+        hipStream_t s = (hipStream_t)stream;
+        for (int r = 0; r < R; ++r)
+            if (!inputs[r] || !outputs[r]) return fail(PCCL_ERR_INVALID, "null tensor for virtual rank " + std::to_string(r));
+
+        // layout of the staged data inside a rank buffer (reference engine_c.cc:468-548)
+        size_t need = (size_t)P.buffer_elems * es;
+        if (ct == "allgather") need = std::max(need, in_bytes * R);
+        else need = std::max(need, in_bytes);
+        if (ct == "alltoall") need = std::max(need, 2 * in_bytes);
+        else if (ct != "reduce_scatter") need = std::max(need, out_bytes);
+        ensure_buffers(ctx, need);
+
+        RankPtrs src{}, dst{}, bufp{};
+        StageOffsets off{};
+        for (int r = 0; r < R; ++r) {
+            src.p[r] = (char*)inputs[r]; bufp.p[r] = ctx->bufs[r]; dst.p[r] = (char*)outputs[r];
+            off.src[r] = 0;
+            off.dst[r] = ct == "allgather" ? (int64_t)r * (int64_t)in_bytes : 0;
+        }
+        int rc = launch_stage(src, bufp, off, R, in_bytes, s);
+        if (rc) return fail(PCCL_ERR_HIP, std::string("input staging: ") + hipGetErrorString((hipError_t)rc));
+
+        run_program(ctx, e, ctx->bufs.data(), ctx->buf_bytes, s);
+
+        if (ct == "reduce_scatter") {
+            size_t chunk = in_bytes / R;
+            if (out_bytes < chunk) return fail(PCCL_ERR_INVALID, "reduce_scatter output is smaller than one chunk");
+            for (int r = 0; r < R; ++r) { off.src[r] = (int64_t)r * (int64_t)chunk; off.dst[r] = 0; }
+            rc = launch_stage(bufp, dst, off, R, chunk, s);
+        } else if (ct == "alltoall") {
+            size_t chunk = in_bytes / R;
+            if (out_bytes < chunk * R) return fail(PCCL_ERR_INVALID, "alltoall output is smaller than the input");
+            rc = 0;
+            for (int p = 0; p < R && rc == 0; ++p) {
+                for (int r = 0; r < R; ++r) {
+                    off.src[r] = p == r ? (int64_t)r * (int64_t)chunk : (int64_t)in_bytes + (int64_t)p * (int64_t)chunk;
+                    off.dst[r] = (int64_t)p * (int64_t)chunk;
+                }
+                rc = launch_stage(bufp, dst, off, R, chunk, s);
+            }
+        } else {
+            for (int r = 0; r < R; ++r) { off.src[r] = 0; off.dst[r] = 0; }
+            rc = launch_stage(bufp, dst, off, R, out_bytes, s);
+        }
+        if (rc) return fail(PCCL_ERR_HIP, std::string("output staging: ") + hipGetErrorString((hipError_t)rc));
+        ctx->last_stream = s;
+        if (sync) HIP_TRY(hipStreamSynchronize(s));
+        return 0;
+    });
+}
+
+int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
+                             void* stream, int sync) {
+    return guarded([&] {
+        if (!ctx || !bufs) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        HIP_TRY(hipSetDevice(ctx->device));
+        OpEntry& e = find_entry(ctx, name);
+        link_entry(ctx, e);
+        hipStream_t s = (hipStream_t)stream;
+        run_program(ctx, e, (char* const*)bufs, buf_bytes, s);
+        ctx->last_stream = s;
+        if (sync) HIP_TRY(hipStreamSynchronize(s));
+        return 0;
+    });
+}
+
+int pccl_hip_sync(pccl_hip_ctx* ctx, const char* name) {
+    return guarded([&] {
+        if (!ctx) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        if (ctx->ops.find(name ? name : "") == ctx->ops.end()) return 0;  // the reference returns silently
+        HIP_TRY(hipSetDevice(ctx->device));
+        HIP_TRY(hipStreamSynchronize(ctx->last_stream));
+        return 0;
+    });
+}
+
+int pccl_hip_reset_signals(pccl_hip_ctx* ctx, const char* name) {
+    return guarded([&] {
+        if (!ctx) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        auto it = ctx->ops.find(name ? name : "");
+        if (it == ctx->ops.end()) return 0;
+        HIP_TRY(hipSetDevice(ctx->device));
+        HIP_TRY(hipStreamSynchronize(ctx->last_stream));
+        // Semaphores are resolved at link time, so no signal array survives an execution; what can
+        // be left over is the runner's progress block after an aborted launch.
+        OpEntry& e = it->second;
+        if (e.linked && e.state.p) {
+            int rc = launch_fill_zero(e.state.p, e.state.bytes, ctx->last_stream);
+            if (rc) return fail(PCCL_ERR_HIP, hipGetErrorString((hipError_t)rc));
+            HIP_TRY(hipStreamSynchronize(ctx->last_stream));
+        }
+        return 0;
+    });
+}
+
+int pccl_hip_op_info(pccl_hip_ctx* ctx, const char* name, pccl_program_info* out) {
+    return guarded([&] {
+        if (!ctx || !out) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        HIP_TRY(hipSetDevice(ctx->device));
+        OpEntry& e = find_entry(ctx, name);
+        link_entry(ctx, e);
+        fill_info(e.prog, out);
+        return 0;
+    });
+}
+
+int pccl_hip_last_kernel_ms(pccl_hip_ctx* ctx, const char* name, float* ms) {
+    return guarded([&] {
+        if (!ctx || !ms) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        OpEntry& e = find_entry(ctx, name);
+        if (!e.timed) return fail(PCCL_ERR_INVALID, "no timed launch: set option timing=1 and execute first");
+        HIP_TRY(hipEventSynchronize(e.ev1));
+        HIP_TRY(hipEventElapsedTime(ms, e.ev0, e.ev1));
+        return 0;
+    });
+}
+
+int pccl_hip_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream) {
+    return guarded([&] {
+        if (!a || !b || !c) return fail(PCCL_ERR_INVALID, "null argument");
+        if (dtype != PCCL_F32 && dtype != PCCL_F16 && dtype != PCCL_BF16 && dtype != PCCL_I32)
+            return fail(PCCL_ERR_UNSUPPORTED, "reduce supports float32, float16, bfloat16 and int32");
+        if (redop < PCCL_SUM || redop > PCCL_MIN) return fail(PCCL_ERR_INVALID, "bad reduce operator");
+        int es = elem_size(dtype);
+        if ((uintptr_t)a % es || (uintptr_t)b % es || (uintptr_t)c % es) return fail(PCCL_ERR_INVALID, "pointers must be aligned to the element size");
+        int rc = launch_reduce(dtype, redop, a, b, c, n, stream);
+        if (rc) return fail(PCCL_ERR_HIP, hipGetErrorString((hipError_t)rc));
+        return 0;
+    });
+}
+
+int pccl_hip_copy(int dtype, const void* src, void* dst, size_t n, void* stream) {
+    return guarded([&] {
+        if (!src || !dst) return fail(PCCL_ERR_INVALID, "null argument");
+        int es = elem_size(dtype);
+        if (!es) return fail(PCCL_ERR_INVALID, "bad dtype");
+        int rc = launch_copy_bytes(src, dst, n * es, stream);
+        if (rc) return fail(PCCL_ERR_HIP, hipGetErrorString((hipError_t)rc));
+        return 0;
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,73 @@
+// Device-side structures and launch wrappers of the gfx950 kernels.
+#pragma once
+
+#include <cstdint>
+
+#include "../../include/pccl_hip.h"
+
+namespace pccl_hip {
+
+// Rank-buffer base pointers handed to a kernel by value (kernarg segment).  Entry r is where
+// rank r's stores and non-first loads go; entry MAX+r is where a first-touch load of rank r reads
+// from (the same buffer, or the caller's input tensor when staging is fused into the program).
+struct RankPtrs {
+    char* p[2 * PCCL_HIP_MAX_VRANKS];
+};
+
+struct DevColSegment {
+    int64_t start, end;      // element positions
+    int64_t first_vec;       // start / vector elems
+    int64_t first_tile;      // prefix sum of tiles
+    int32_t prog_start, prog_len;
+    int32_t fifo_start, fifo_len;
+};
+
+struct DevStepOp {
+    int64_t off0, off1, off2, size;  // elements
+    int32_t self, peer, is_reduce, redop;
+    int32_t first_item, ntiles, dep_start, ndeps;
+};
+
+struct StepState {      // device memory, zero between launches (the kernel restores it on exit)
+    int32_t cursor;
+    int32_t exited;
+    int32_t pad[30];
+    // followed by int32 done[num_ops]
+};
+
+struct ColumnLaunch {
+    const DevColSegment* segs;
+    int32_t num_segs;
+    const uint64_t* instrs;   // ColInstr words
+    const uint8_t* fifo;
+    int64_t total_tiles;
+    int32_t dtype;
+    int32_t vecs_per_thread;  // 1, 2 or 4
+    int32_t num_blocks;       // 0: one workgroup per tile
+};
+
+struct StepwiseLaunch {
+    const DevStepOp* ops;
+    int32_t num_ops;
+    const int32_t* deps;
+    const int32_t* item_op;
+    int32_t num_items;
+    int64_t tile_elems;
+    StepState* state;
+    int32_t dtype;
+    int32_t num_blocks;
+};
+
+// All return a hipError_t value as int (0 = success).
+int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream);
+int launch_stepwise(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream);
+int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream);
+int launch_copy_bytes(const void* src, void* dst, size_t nbytes, void* stream);
+// One launch copying `bytes` from src.p[r] + src_off[r] to dst.p[r] + dst_off[r] for r < R.
+struct StageOffsets { int64_t src[PCCL_HIP_MAX_VRANKS]; int64_t dst[PCCL_HIP_MAX_VRANKS]; };
+int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& off, int R, size_t bytes, void* stream);
+int launch_fill_zero(void* dst, size_t nbytes, void* stream);
+
+int device_cu_count(int device);
+
+}  // namespace pccl_hip

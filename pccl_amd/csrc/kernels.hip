@@ -1,0 +1,512 @@
+// gfx950 kernels of the executor: element arithmetic, the chunk reduce/copy primitives, the
+// stepwise (flag-ordered) runner and the column runner.
+//
+// Arithmetic contract (what the reference's Vec<T>::operator+ computes on its hardware,
+// csrc/plugins/cuda/kernel/vec.h:104-111,170-177,232-239): one correctly rounded addition in the
+// storage type per element per reduce; NaN results are the canonical NaN (all mantissa bits set).
+// bf16 is computed as RNE(float(a) + float(b)), which equals the single bf16 rounding because the
+// float sum of two 8-bit-significand values is exact or rounds innocuously (24 >= 2*8+2).
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace pccl_hip {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int kMaxR = PCCL_HIP_MAX_VRANKS;
+
+// ------------------------------------------------------------------------------- arithmetic
+
+template <int DT> struct ElemBytes { static constexpr int value = (DT == PCCL_F32 || DT == PCCL_I32) ? 4 : (DT == PCCL_F16 || DT == PCCL_BF16) ? 2 : 1; };
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ uint32_t f32_op(uint32_t ua, uint32_t ub, int redop) {
+    float a = as_f32(ua), b = as_f32(ub), r;
+    if (redop == PCCL_SUM) r = a + b;
+    else if (redop == PCCL_MAX) r = (a != a || b != b) ? as_f32(0x7FFFFFFFu) : (a > b ? a : b);
+    else r = (a != a || b != b) ? as_f32(0x7FFFFFFFu) : (a < b ? a : b);
+    return (r != r) ? 0x7FFFFFFFu : as_u32(r);
+}
+
+// float -> bf16 bits in the HIGH half of the result, round to nearest even, canonical NaN
+__device__ __forceinline__ uint32_t bf16_round_hi(float f) {
+    uint32_t u = as_u32(f);
+    uint32_t r = u + 0x7FFFu + ((u >> 16) & 1u);
+    return (f != f) ? 0x7FFF0000u : (r & 0xFFFF0000u);
+}
+
+__device__ __forceinline__ float bf16_sel(float a, float b, int redop) {
+    if (redop == PCCL_SUM) return a + b;
+    if (a != a || b != b) return as_f32(0x7FFFFFFFu);
+    return redop == PCCL_MAX ? (a > b ? a : b) : (a < b ? a : b);
+}
+
+__device__ __forceinline__ uint32_t bf16x2_op(uint32_t a, uint32_t b, int redop) {
+    float lo = bf16_sel(as_f32(a << 16), as_f32(b << 16), redop);
+    float hi = bf16_sel(as_f32(a & 0xFFFF0000u), as_f32(b & 0xFFFF0000u), redop);
+    return bf16_round_hi(hi) | (bf16_round_hi(lo) >> 16);
+}
+
+__device__ __forceinline__ uint32_t f16x2_op(uint32_t ua, uint32_t ub, int redop) {
+    h2 a = __builtin_bit_cast(h2, ua), b = __builtin_bit_cast(h2, ub), r;
+    if (redop == PCCL_SUM) r = a + b;
+    else {
+        for (int k = 0; k < 2; ++k) {
+            _Float16 x = a[k], y = b[k];
+            bool nan = (x != x) || (y != y);
+            _Float16 m = redop == PCCL_MAX ? (x > y ? x : y) : (x < y ? x : y);
+            r[k] = nan ? __builtin_bit_cast(_Float16, (uint16_t)0x7FFF) : m;
+        }
+    }
+    uint32_t u = __builtin_bit_cast(uint32_t, r);
+    if (r[0] != r[0]) u = (u & 0xFFFF0000u) | 0x7FFFu;
+    if (r[1] != r[1]) u = (u & 0x0000FFFFu) | 0x7FFF0000u;
+    return u;
+}
+
+__device__ __forceinline__ uint32_t i32_op(uint32_t a, uint32_t b, int redop) {
+    if (redop == PCCL_SUM) return a + b;
+    int x = (int)a, y = (int)b;
+    return (uint32_t)(redop == PCCL_MAX ? (x > y ? x : y) : (x < y ? x : y));
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t word_op(uint32_t a, uint32_t b, int redop) {
+    if constexpr (DT == PCCL_F32) return f32_op(a, b, redop);
+    else if constexpr (DT == PCCL_I32) return i32_op(a, b, redop);
+    else if constexpr (DT == PCCL_BF16) return bf16x2_op(a, b, redop);
+    else if constexpr (DT == PCCL_F16) return f16x2_op(a, b, redop);
+    else return a;  // fp8: no reduce (rejected at graph load)
+}
+
+template <int DT>
+__device__ __forceinline__ u32x4 vec_op(u32x4 a, u32x4 b, int redop) {
+    u32x4 r;
+    r.x = word_op<DT>(a.x, b.x, redop);
+    r.y = word_op<DT>(a.y, b.y, redop);
+    r.z = word_op<DT>(a.z, b.z, redop);
+    r.w = word_op<DT>(a.w, b.w, redop);
+    return r;
+}
+
+// one element at byte address granularity (heads, tails, partial vectors, misaligned ranges)
+template <int DT>
+__device__ __forceinline__ uint32_t load_elem(const char* p) {
+    constexpr int ES = ElemBytes<DT>::value;
+    if constexpr (ES == 4) return *reinterpret_cast<const uint32_t*>(p);
+    else if constexpr (ES == 2) return *reinterpret_cast<const uint16_t*>(p);
+    else return *reinterpret_cast<const uint8_t*>(p);
+}
+template <int DT>
+__device__ __forceinline__ void store_elem(char* p, uint32_t v) {
+    constexpr int ES = ElemBytes<DT>::value;
+    if constexpr (ES == 4) *reinterpret_cast<uint32_t*>(p) = v;
+    else if constexpr (ES == 2) *reinterpret_cast<uint16_t*>(p) = (uint16_t)v;
+    else *reinterpret_cast<uint8_t*>(p) = (uint8_t)v;
+}
+template <int DT>
+__device__ __forceinline__ uint32_t elem_op(uint32_t a, uint32_t b, int redop) {
+    // 2-byte types ride in the low half of a word; the zero high halves reduce to zero
+    return word_op<DT>(a, b, redop);
+}
+
+__device__ __forceinline__ u32x4 ldv(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void stv(char* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+
+// ------------------------------------------------------------------------------- range primitives
+//
+// c[i] = a[i] (op) b[i] (IS_REDUCE) or c[i] = a[i], i in [0, n) elements, cooperatively by
+// `nthreads` threads.  Any alignment: when the three addresses are congruent modulo 16 the body runs
+// as 128-bit loads and stores with a scalar head and tail; otherwise element by element.
+
+template <int DT, bool IS_REDUCE>
+__device__ __forceinline__ void range_op(const char* a, const char* b, char* c, int64_t n, int redop,
+                                         int tid, int nthreads) {
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int VE = 16 / ES;
+    uintptr_t ua = (uintptr_t)a, ub = (uintptr_t)b, uc = (uintptr_t)c;
+    bool congruent = ((ua ^ uc) & 15) == 0 && (!IS_REDUCE || ((ub ^ uc) & 15) == 0);
+    if (!congruent) {
+        for (int64_t i = tid; i < n; i += nthreads) {
+            uint32_t x = load_elem<DT>(a + i * ES);
+            if constexpr (IS_REDUCE) x = elem_op<DT>(x, load_elem<DT>(b + i * ES), redop);
+            store_elem<DT>(c + i * ES, x);
+        }
+        return;
+    }
+    int64_t head = (int64_t)(((16 - (uc & 15)) & 15) / ES);
+    if (head > n) head = n;
+    if (tid < head) {
+        uint32_t x = load_elem<DT>(a + (int64_t)tid * ES);
+        if constexpr (IS_REDUCE) x = elem_op<DT>(x, load_elem<DT>(b + (int64_t)tid * ES), redop);
+        store_elem<DT>(c + (int64_t)tid * ES, x);
+    }
+    a += head * ES; b += head * ES; c += head * ES; n -= head;
+    int64_t nvec = n / VE;
+    int64_t v = tid;
+    // 4 vectors per thread per trip: all loads issued before the first store
+    for (; v + 3 * (int64_t)nthreads < nvec; v += 4 * (int64_t)nthreads) {
+        u32x4 x0 = ldv(a + v * 16), x1 = ldv(a + (v + nthreads) * 16), x2 = ldv(a + (v + 2 * nthreads) * 16), x3 = ldv(a + (v + 3 * nthreads) * 16);
+        if constexpr (IS_REDUCE) {
+            u32x4 y0 = ldv(b + v * 16), y1 = ldv(b + (v + nthreads) * 16), y2 = ldv(b + (v + 2 * nthreads) * 16), y3 = ldv(b + (v + 3 * nthreads) * 16);
+            x0 = vec_op<DT>(x0, y0, redop); x1 = vec_op<DT>(x1, y1, redop); x2 = vec_op<DT>(x2, y2, redop); x3 = vec_op<DT>(x3, y3, redop);
+        }
+        stv(c + v * 16, x0); stv(c + (v + nthreads) * 16, x1); stv(c + (v + 2 * nthreads) * 16, x2); stv(c + (v + 3 * nthreads) * 16, x3);
+    }
+    for (; v < nvec; v += nthreads) {
+        u32x4 x = ldv(a + v * 16);
+        if constexpr (IS_REDUCE) x = vec_op<DT>(x, ldv(b + v * 16), redop);
+        stv(c + v * 16, x);
+    }
+    int64_t tail0 = nvec * VE;
+    for (int64_t i = tail0 + tid; i < n; i += nthreads) {
+        uint32_t x = load_elem<DT>(a + i * ES);
+        if constexpr (IS_REDUCE) x = elem_op<DT>(x, load_elem<DT>(b + i * ES), redop);
+        store_elem<DT>(c + i * ES, x);
+    }
+}
+
+// byte copy with the same structure (used by copies of every dtype and by staging)
+__device__ __forceinline__ void range_copy_bytes(const char* a, char* c, int64_t nbytes, int tid, int nthreads) {
+    range_op<PCCL_F8E4M3, false>(a, nullptr, c, nbytes, 0, tid, nthreads);
+}
+
+template <int DT>
+__device__ __forceinline__ void range_dispatch(bool is_reduce, const char* a, const char* b, char* c, int64_t n,
+                                               int redop, int tid, int nthreads) {
+    if (is_reduce) range_op<DT, true>(a, b, c, n, redop, tid, nthreads);
+    else range_copy_bytes(a, c, n * ElemBytes<DT>::value, tid, nthreads);
+}
+
+// ------------------------------------------------------------------------------- standalone primitives
+
+constexpr int64_t kPrimTileBytes = 64 * 1024;
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void reduce_kernel(const char* a, const char* b, char* c, int64_t n, int redop) {
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int64_t TE = kPrimTileBytes / ES;
+    int64_t ntiles = (n + TE - 1) / TE;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        int64_t e0 = t * TE, cnt = n - e0 < TE ? n - e0 : TE;
+        range_op<DT, true>(a + e0 * ES, b + e0 * ES, c + e0 * ES, cnt, redop, threadIdx.x, kThreads);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void copy_kernel(const char* src, char* dst, int64_t nbytes) {
+    int64_t ntiles = (nbytes + kPrimTileBytes - 1) / kPrimTileBytes;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        int64_t b0 = t * kPrimTileBytes, cnt = nbytes - b0 < kPrimTileBytes ? nbytes - b0 : kPrimTileBytes;
+        range_copy_bytes(src + b0, dst + b0, cnt, threadIdx.x, kThreads);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void stage_kernel(RankPtrs src, RankPtrs dst, StageOffsets off, int64_t nbytes) {
+    int r = blockIdx.y;
+    const char* s = src.p[r] + off.src[r];
+    char* d = dst.p[r] + off.dst[r];
+    int64_t ntiles = (nbytes + kPrimTileBytes - 1) / kPrimTileBytes;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        int64_t b0 = t * kPrimTileBytes, cnt = nbytes - b0 < kPrimTileBytes ? nbytes - b0 : kPrimTileBytes;
+        range_copy_bytes(s + b0, d + b0, cnt, threadIdx.x, kThreads);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* dst, int64_t nwords) {
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * kThreads) dst[i] = 0;
+}
+
+// ------------------------------------------------------------------------------- stepwise runner
+//
+// One persistent launch executes every data op of the linked program.  Work items are (op, tile)
+// pairs in level order; a workgroup claims the next item from one atomic cursor, waits until every
+// tile of the op's predecessors has been published, runs the tile, then publishes it.  A claimed
+// item only ever waits for items claimed earlier by workgroups that are already running, so the
+// scheme cannot deadlock whatever the grid size.
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void stepwise_kernel(StepwiseLaunch L, RankPtrs ptrs) {
+    constexpr int ES = ElemBytes<DT>::value;
+    __shared__ int s_item;
+    __shared__ int s_last;
+    int32_t* done = reinterpret_cast<int32_t*>(L.state + 1);
+    const int tid = threadIdx.x;
+    for (;;) {
+        if (tid == 0) s_item = atomicAdd(&L.state->cursor, 1);
+        __syncthreads();
+        int item = s_item;
+        __syncthreads();
+        if (item >= L.num_items) break;
+        int opi = L.item_op[item];
+        DevStepOp op = L.ops[opi];
+        if (tid < op.ndeps) {
+            int d = L.deps[op.dep_start + tid];
+            int need = L.ops[d].ntiles;
+            while (__hip_atomic_load(&done[d], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) __builtin_amdgcn_s_sleep(4);
+        }
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
+        int64_t cnt = op.size - e0 < L.tile_elems ? op.size - e0 : L.tile_elems;
+        char* self = ptrs.p[op.self];
+        const char* peer = ptrs.p[op.peer];
+        if (op.is_reduce)
+            range_op<DT, true>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
+        else
+            range_copy_bytes(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
+        __syncthreads();  // every wave's stores are issued and counted before the publish
+        if (tid == 0) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __hip_atomic_fetch_add(&done[opi], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // the last workgroup out restores the state block for the next launch
+    if (tid == 0) s_last = (atomicAdd(&L.state->exited, 1) == (int)gridDim.x - 1);
+    __syncthreads();
+    if (s_last) {
+        for (int i = tid; i < L.num_ops; i += kThreads) done[i] = 0;
+        if (tid == 0) { L.state->cursor = 0; L.state->exited = 0; }
+    }
+}
+
+// ------------------------------------------------------------------------------- column runner
+//
+// When every data op reads and writes the same element positions in all buffers, the program
+// decomposes by position: what happens to position p involves only position p of the R buffers.
+// A segment is a maximal position range with one op list; a workgroup takes a tile of a segment
+// and runs the segment's column program on it start to finish, each thread on its own 16-byte
+// vectors.  No workgroup ever depends on another, so there are no flags and no fences; values
+// that the next instruction needs stay in registers (SRC_ACC) and writes that are overwritten
+// before anything re-reads them are dropped (store == 0).  Results are bit-identical to running
+// the ops one at a time in schedule order: every element sees the same operations in the same
+// order with the same per-step rounding.
+
+struct ColInstrDev { uint8_t self, peer, a_src, b_src, redop, store, a_first, b_first; };
+
+__device__ __forceinline__ ColInstrDev unpack_instr(uint64_t w) {
+    ColInstrDev i;
+    i.self = w & 0xFF; i.peer = (w >> 8) & 0xFF; i.a_src = (w >> 16) & 0xFF; i.b_src = (w >> 24) & 0xFF;
+    i.redop = (w >> 32) & 0xFF; i.store = (w >> 40) & 0xFF; i.a_first = (w >> 48) & 0xFF; i.b_first = (w >> 56) & 0xFF;
+    return i;
+}
+
+template <int DT, int U>
+__global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPtrs ptrs) {
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int VE = 16 / ES;
+    constexpr int64_t TILE_V = (int64_t)kThreads * U;
+    __shared__ char* s_ptr[2 * kMaxR];
+    const int tid = threadIdx.x;
+    if (tid < 2 * kMaxR) s_ptr[tid] = ptrs.p[tid];
+    __syncthreads();
+
+    for (int64_t tile = blockIdx.x; tile < L.total_tiles; tile += gridDim.x) {
+        // segment lookup (uniform)
+        int lo = 0, hi = L.num_segs;
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (L.segs[mid].first_tile <= tile) lo = mid; else hi = mid;
+        }
+        const DevColSegment seg = L.segs[lo];
+        const int64_t vfirst = seg.first_vec + (tile - seg.first_tile) * TILE_V;
+        const uint64_t* prog = L.instrs + seg.prog_start;
+        const bool interior = vfirst * VE >= seg.start && (vfirst + TILE_V) * VE <= seg.end;
+        if (interior) {
+            int64_t off[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) off[u] = (vfirst + (int64_t)u * kThreads + tid) * 16;
+            u32x4 acc[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) acc[u] = u32x4{0, 0, 0, 0};
+            for (int k = 0; k < seg.prog_len; ++k) {
+                const ColInstrDev in = unpack_instr(prog[k]);
+                char* self = s_ptr[in.self];
+                u32x4 a[U];
+                if (in.a_src == 2 /*SRC_ACC*/) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) a[u] = acc[u];
+                } else {
+                    const char* peer = s_ptr[in.peer + (in.a_first ? kMaxR : 0)];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) a[u] = ldv(peer + off[u]);
+                }
+                if (in.b_src != 0 /*reduce*/) {
+                    u32x4 b[U];
+                    if (in.b_src == 2) {
+#pragma unroll
+                        for (int u = 0; u < U; ++u) b[u] = acc[u];
+                    } else {
+                        const char* own = s_ptr[in.self + (in.b_first ? kMaxR : 0)];
+#pragma unroll
+                        for (int u = 0; u < U; ++u) b[u] = ldv(own + off[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) acc[u] = vec_op<DT>(a[u], b[u], in.redop);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) acc[u] = a[u];
+                }
+                if (in.store) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) stv(self + off[u], acc[u]);
+                }
+            }
+        } else {
+            // edge tile: vectors may be cut by the segment boundary or lie outside it
+            for (int64_t v = vfirst + tid; v < vfirst + TILE_V; v += kThreads) {
+                int64_t e0 = v * VE, e1 = e0 + VE;
+                if (e0 < seg.start) e0 = seg.start;
+                if (e1 > seg.end) e1 = seg.end;
+                if (e0 >= e1) continue;
+                if (e1 - e0 == VE) {
+                    int64_t o = v * 16;
+                    u32x4 acc = u32x4{0, 0, 0, 0};
+                    for (int k = 0; k < seg.prog_len; ++k) {
+                        const ColInstrDev in = unpack_instr(prog[k]);
+                        u32x4 a = in.a_src == 2 ? acc : ldv(s_ptr[in.peer + (in.a_first ? kMaxR : 0)] + o);
+                        if (in.b_src != 0) {
+                            u32x4 b = in.b_src == 2 ? acc : ldv(s_ptr[in.self + (in.b_first ? kMaxR : 0)] + o);
+                            acc = vec_op<DT>(a, b, in.redop);
+                        } else acc = a;
+                        if (in.store) stv(s_ptr[in.self] + o, acc);
+                    }
+                } else {
+                    for (int64_t e = e0; e < e1; ++e) {
+                        int64_t o = e * ES;
+                        uint32_t acc = 0;
+                        for (int k = 0; k < seg.prog_len; ++k) {
+                            const ColInstrDev in = unpack_instr(prog[k]);
+                            uint32_t a = in.a_src == 2 ? acc : load_elem<DT>(s_ptr[in.peer + (in.a_first ? kMaxR : 0)] + o);
+                            if (in.b_src != 0) {
+                                uint32_t b = in.b_src == 2 ? acc : load_elem<DT>(s_ptr[in.self + (in.b_first ? kMaxR : 0)] + o);
+                                acc = elem_op<DT>(a, b, in.redop);
+                            } else acc = a;
+                            if (in.store) store_elem<DT>(s_ptr[in.self] + o, acc);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------- launchers
+
+static int g_cu_count[16] = {0};
+
+int device_cu_count(int device) {
+    if (device < 0 || device >= 16) device = 0;
+    if (!g_cu_count[device]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+        g_cu_count[device] = n;
+    }
+    return g_cu_count[device];
+}
+
+static int current_cus() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    return device_cu_count(dev);
+}
+
+template <int DT>
+static int launch_column_dt(const ColumnLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
+    int64_t grid = L.total_tiles;
+    if (L.num_blocks > 0 && grid > L.num_blocks) grid = L.num_blocks;
+    if (grid > (1 << 30)) grid = 1 << 30;
+    if (grid <= 0) return 0;
+    switch (L.vecs_per_thread) {
+        case 1: hipLaunchKernelGGL((column_kernel<DT, 1>), dim3((unsigned)grid), dim3(kThreads), 0, s, L, ptrs); break;
+        case 2: hipLaunchKernelGGL((column_kernel<DT, 2>), dim3((unsigned)grid), dim3(kThreads), 0, s, L, ptrs); break;
+        default: hipLaunchKernelGGL((column_kernel<DT, 4>), dim3((unsigned)grid), dim3(kThreads), 0, s, L, ptrs); break;
+    }
+    return (int)hipGetLastError();
+}
+
+int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
+    hipStream_t s = (hipStream_t)stream;
+    switch (L.dtype) {
+        case PCCL_F32: return launch_column_dt<PCCL_F32>(L, ptrs, s);
+        case PCCL_F16: return launch_column_dt<PCCL_F16>(L, ptrs, s);
+        case PCCL_BF16: return launch_column_dt<PCCL_BF16>(L, ptrs, s);
+        case PCCL_I32: return launch_column_dt<PCCL_I32>(L, ptrs, s);
+        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_column_dt<PCCL_F8E4M3>(L, ptrs, s);
+        default: return (int)hipErrorInvalidValue;
+    }
+}
+
+template <int DT>
+static int launch_stepwise_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
+    int grid = L.num_blocks > 0 ? L.num_blocks : current_cus() * 8;
+    if (grid > L.num_items) grid = L.num_items;
+    if (grid <= 0) return 0;
+    hipLaunchKernelGGL((stepwise_kernel<DT>), dim3(grid), dim3(kThreads), 0, s, L, ptrs);
+    return (int)hipGetLastError();
+}
+
+int launch_stepwise(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream) {
+    hipStream_t s = (hipStream_t)stream;
+    switch (L.dtype) {
+        case PCCL_F32: return launch_stepwise_dt<PCCL_F32>(L, ptrs, s);
+        case PCCL_F16: return launch_stepwise_dt<PCCL_F16>(L, ptrs, s);
+        case PCCL_BF16: return launch_stepwise_dt<PCCL_BF16>(L, ptrs, s);
+        case PCCL_I32: return launch_stepwise_dt<PCCL_I32>(L, ptrs, s);
+        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_stepwise_dt<PCCL_F8E4M3>(L, ptrs, s);
+        default: return (int)hipErrorInvalidValue;
+    }
+}
+
+static int grid_for_tiles(int64_t ntiles) {
+    int64_t cap = (int64_t)current_cus() * 8;
+    return (int)(ntiles < cap ? (ntiles > 0 ? ntiles : 1) : cap);
+}
+
+int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream) {
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const char* pa = (const char*)a; const char* pb = (const char*)b; char* pc = (char*)c;
+    int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+    int grid = grid_for_tiles(((int64_t)n * es + kPrimTileBytes - 1) / kPrimTileBytes);
+    switch (dtype) {
+        case PCCL_F32: hipLaunchKernelGGL((reduce_kernel<PCCL_F32>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
+        case PCCL_F16: hipLaunchKernelGGL((reduce_kernel<PCCL_F16>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
+        case PCCL_BF16: hipLaunchKernelGGL((reduce_kernel<PCCL_BF16>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
+        case PCCL_I32: hipLaunchKernelGGL((reduce_kernel<PCCL_I32>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
+        default: return (int)hipErrorInvalidValue;
+    }
+    return (int)hipGetLastError();
+}
+
+int launch_copy_bytes(const void* src, void* dst, size_t nbytes, void* stream) {
+    if (nbytes == 0) return 0;
+    int grid = grid_for_tiles(((int64_t)nbytes + kPrimTileBytes - 1) / kPrimTileBytes);
+    hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(kThreads), 0, (hipStream_t)stream, (const char*)src, (char*)dst, (int64_t)nbytes);
+    return (int)hipGetLastError();
+}
+
+int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& off, int R, size_t bytes, void* stream) {
+    if (bytes == 0 || R <= 0) return 0;
+    int64_t ntiles = ((int64_t)bytes + kPrimTileBytes - 1) / kPrimTileBytes;
+    int64_t cap = ((int64_t)current_cus() * 8 + R - 1) / R;
+    int gx = (int)(ntiles < cap ? ntiles : cap);
+    if (gx < 1) gx = 1;
+    hipLaunchKernelGGL(stage_kernel, dim3(gx, R), dim3(kThreads), 0, (hipStream_t)stream, src, dst, off, (int64_t)bytes);
+    return (int)hipGetLastError();
+}
+
+int launch_fill_zero(void* dst, size_t nbytes, void* stream) {
+    int64_t nwords = (int64_t)(nbytes / 4);
+    if (nwords == 0) return 0;
+    int grid = (int)((nwords + kThreads - 1) / kThreads);
+    if (grid > 1024) grid = 1024;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(kThreads), 0, (hipStream_t)stream, (uint32_t*)dst, nwords);
+    return (int)hipGetLastError();
+}
+
+}  // namespace pccl_hip

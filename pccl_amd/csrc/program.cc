@@ -1,0 +1,359 @@
+// Cross-rank linker and plan builder.
+//
+// The reference runs one process per rank and lets counting semaphores order the ranks at run time
+// (csrc/plugins/cuda/cuda_executor.cu:414-445).  With all ranks in one address space the same
+// ordering can be derived once, on the host: simulate the semaphores, pair every wait with the
+// notify that releases it, and keep only the resulting dependencies between data ops.
+#include "program.h"
+
+#include <algorithm>
+#include <cstring>
+#include <deque>
+#include <map>
+#include <numeric>
+#include <set>
+
+namespace pccl_hip {
+
+namespace {
+
+struct Bitset {
+    std::vector<uint64_t> w;
+    explicit Bitset(size_t n = 0) : w((n + 63) / 64, 0) {}
+    void set(size_t i) { w[i >> 6] |= 1ull << (i & 63); }
+    bool test(size_t i) const { return w[i >> 6] >> (i & 63) & 1; }
+    void or_with(const Bitset& o) { for (size_t k = 0; k < w.size(); ++k) w[k] |= o.w[k]; }
+};
+
+struct Node {
+    int rank, pos;
+    std::vector<int> preds;  // global node ids
+};
+
+std::string op_name(const RankGraph& g, int rank, int pos) {
+    const GraphOp& o = g.ops[pos];
+    const char* k = o.kind == OpKind::Reduce ? "reduce" : o.kind == OpKind::Copy ? "copy" : o.kind == OpKind::Notify ? "notify" : o.kind == OpKind::Wait ? "wait_notify" : "noop";
+    return "rank " + std::to_string(rank) + " op " + std::to_string(o.index) + " (" + k + ")";
+}
+
+constexpr size_t kClosureLimit = 24000;   // nodes; above this the O(N^2) checks are skipped
+constexpr size_t kPairLimit = 20000000;   // access pairs examined by the race check
+
+}  // namespace
+
+Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOptions& opt) {
+    const int R = (int)graphs.size();
+    if (R <= 0 || R > PCCL_HIP_MAX_VRANKS) throw Error{PCCL_ERR_INVALID, "number of virtual ranks must be 1.." + std::to_string(PCCL_HIP_MAX_VRANKS)};
+    Program P;
+    P.R = R;
+    bool have_dtype = false;
+    std::vector<int> base(R + 1, 0);
+    for (int r = 0; r < R; ++r) {
+        if (!graphs[r]) throw Error{PCCL_ERR_LINK, "virtual rank " + std::to_string(r) + " has no registered graph"};
+        const RankGraph& g = *graphs[r];
+        base[r + 1] = base[r] + (int)g.ops.size();
+        if (g.has_dtype) {
+            if (have_dtype && g.dtype != P.dtype) throw Error{PCCL_ERR_LINK, "ranks disagree on tensor_info.dtype"};
+            P.dtype = g.dtype; have_dtype = true;
+        }
+        if (r == 0) { P.collective_type = g.collective_type; P.tensor_elems = g.tensor_elems; }
+        else if (g.collective_type != P.collective_type) throw Error{PCCL_ERR_LINK, "ranks disagree on collective_type"};
+        P.buffer_elems = std::max(P.buffer_elems, g.max_extent());
+        P.tensor_elems = std::max(P.tensor_elems, g.tensor_elems);
+    }
+    const int N = base[R];
+    P.num_all_ops = N;
+    const int es = elem_size(P.dtype);
+
+    // ---- static checks on ranks
+    for (int r = 0; r < R; ++r)
+        for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
+            const GraphOp& o = graphs[r]->ops[i];
+            bool uses_peer = o.kind == OpKind::Reduce || o.kind == OpKind::Copy || o.kind == OpKind::Notify;
+            if (uses_peer && (o.peer < 0 || o.peer >= R))
+                throw Error{PCCL_ERR_LINK, op_name(*graphs[r], r, (int)i) + " names rank " + std::to_string(o.peer) + " but only " + std::to_string(R) + " virtual ranks exist"};
+        }
+
+    // ---- simulate the semaphores (same discipline as the reference's dependency-counter runner:
+    //      per rank and channel a FIFO of ready ops, one at a time; a wait blocks its channel)
+    std::vector<Node> nodes(N);
+    for (int r = 0; r < R; ++r)
+        for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
+            Node& n = nodes[base[r] + i];
+            n.rank = r; n.pos = (int)i;
+            for (int d : graphs[r]->ops[i].deps) n.preds.push_back(base[r] + d);
+        }
+    std::vector<int> remaining(N);
+    std::vector<std::deque<int>> queues((size_t)R * PCCL_HIP_MAX_CHANNELS);
+    for (int r = 0; r < R; ++r)
+        for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
+            remaining[base[r] + i] = graphs[r]->ops[i].num_deps_declared;
+            if (remaining[base[r] + i] == 0) queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + graphs[r]->ops[i].channel].push_back((int)i);
+        }
+    // per (target rank, id): notify nodes not yet consumed, in arrival order
+    std::map<std::pair<int, int>, std::deque<int>> pending;
+    std::map<std::pair<int, int>, std::vector<int>> notify_seq, wait_seq;  // for the ambiguity check
+    std::vector<int> exec_order;
+    exec_order.reserve(N);
+    int done = 0;
+    while (done < N) {
+        bool progressed = false;
+        for (int r = 0; r < R; ++r)
+            for (int c = 0; c < PCCL_HIP_MAX_CHANNELS; ++c) {
+                auto& q = queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + c];
+                while (!q.empty()) {
+                    int i = q.front();
+                    const GraphOp& o = graphs[r]->ops[i];
+                    int id = base[r] + i;
+                    if (o.kind == OpKind::Wait) {
+                        auto key = std::make_pair(r, (int)o.off0);
+                        auto it = pending.find(key);
+                        if (it == pending.end() || it->second.empty()) break;  // blocked
+                        nodes[id].preds.push_back(it->second.front());
+                        it->second.pop_front();
+                        wait_seq[key].push_back(id);
+                    } else if (o.kind == OpKind::Notify) {
+                        auto key = std::make_pair(o.peer, (int)o.off0);
+                        pending[key].push_back(id);
+                        notify_seq[key].push_back(id);
+                    }
+                    q.pop_front();
+                    exec_order.push_back(id);
+                    ++done; progressed = true;
+                    for (int nx : o.nexts)
+                        if (--remaining[base[r] + nx] == 0)
+                            queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + graphs[r]->ops[nx].channel].push_back(nx);
+                }
+            }
+        if (!progressed) {
+            std::string blocked;
+            int shown = 0;
+            for (int r = 0; r < R && shown < 4; ++r)
+                for (int c = 0; c < PCCL_HIP_MAX_CHANNELS && shown < 4; ++c) {
+                    auto& q = queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + c];
+                    if (!q.empty()) { blocked += (shown ? "; " : "") + op_name(*graphs[r], r, q.front()) + " waits on signal " + std::to_string(graphs[r]->ops[q.front()].off0); ++shown; }
+                }
+            if (blocked.empty()) blocked = "ops with unmet dependencies (cyclic or dangling dependency lists)";
+            throw Error{PCCL_ERR_LINK, "deadlock: " + std::to_string(done) + " of " + std::to_string(N) + " ops can run; blocked: " + blocked};
+        }
+    }
+    for (auto& kv : pending) if (!kv.second.empty()) P.residual_signals++;
+
+    // ---- reachability (happens-before) over all ops, in execution order (a topological order)
+    const bool closure = (size_t)N <= kClosureLimit;
+    std::vector<Bitset> reach;  // reach[v] = nodes that happen before v
+    if (closure) {
+        reach.assign(N, Bitset(N));
+        for (int id : exec_order)
+            for (int p : nodes[id].preds) { reach[id].or_with(reach[p]); reach[id].set(p); }
+        auto ordered_seq = [&](const std::vector<int>& seq) {
+            for (size_t k = 1; k < seq.size(); ++k)
+                if (!reach[seq[k]].test(seq[k - 1])) return false;
+            return true;
+        };
+        for (auto& kv : notify_seq)
+            if (!ordered_seq(kv.second))
+                throw Error{PCCL_ERR_LINK, "signal " + std::to_string(kv.first.second) + " of rank " + std::to_string(kv.first.first) + " is notified by ops that are not ordered with each other: the pairing of notifies and waits is ambiguous"};
+        for (auto& kv : wait_seq)
+            if (!ordered_seq(kv.second))
+                throw Error{PCCL_ERR_LINK, "signal " + std::to_string(kv.first.second) + " of rank " + std::to_string(kv.first.first) + " is awaited by ops that are not ordered with each other: the pairing of notifies and waits is ambiguous"};
+    }
+
+    // ---- data ops and their nearest data predecessors
+    std::vector<int> data_of(N, -1);  // node id -> provisional data-op index
+    std::vector<int> data_nodes;
+    for (int id : exec_order) {
+        const GraphOp& o = graphs[nodes[id].rank]->ops[nodes[id].pos];
+        if (o.kind == OpKind::Reduce || o.kind == OpKind::Copy) { data_of[id] = (int)data_nodes.size(); data_nodes.push_back(id); }
+    }
+    const int D = (int)data_nodes.size();
+    // frontier[v] = set of data nodes that are the nearest data ancestors of v (through signals/noops)
+    std::vector<std::vector<int>> frontier(N);
+    for (int id : exec_order) {
+        std::vector<int>& f = frontier[id];
+        for (int p : nodes[id].preds) {
+            if (data_of[p] >= 0) f.push_back(p);
+            else f.insert(f.end(), frontier[p].begin(), frontier[p].end());
+        }
+        std::sort(f.begin(), f.end());
+        f.erase(std::unique(f.begin(), f.end()), f.end());
+        if (closure && f.size() > 1) {  // drop ancestors of other members
+            std::vector<int> keep;
+            for (int a : f) {
+                bool redundant = false;
+                for (int b : f) if (a != b && reach[b].test(a)) { redundant = true; break; }
+                if (!redundant) keep.push_back(a);
+            }
+            f.swap(keep);
+        }
+    }
+    std::vector<LinkedOp> ops(D);
+    for (int k = 0; k < D; ++k) {
+        int id = data_nodes[k];
+        const GraphOp& o = graphs[nodes[id].rank]->ops[nodes[id].pos];
+        LinkedOp& L = ops[k];
+        L.rank = nodes[id].rank; L.channel = o.channel; L.graph_pos = nodes[id].pos; L.index = o.index;
+        L.is_reduce = o.kind == OpKind::Reduce; L.redop = o.redop; L.peer = o.peer;
+        L.off0 = o.off0; L.off1 = o.off1; L.off2 = o.off2; L.size = o.size;
+        for (int p : frontier[id]) L.deps.push_back(data_of[p]);
+        int lvl = 0;
+        for (int d : L.deps) lvl = std::max(lvl, ops[d].level + 1);
+        L.level = lvl;
+        P.num_levels = std::max(P.num_levels, lvl + 1);
+        P.algorithmic_bytes += (L.is_reduce ? 3 : 2) * L.size * es;
+        // an op whose own source and destination ranges overlap without coinciding has no
+        // defined element order
+        auto partial = [&](int64_t s, int64_t d) { return s != d && s < d + L.size && d < s + L.size; };
+        if (L.size > 0) {
+            if (L.is_reduce && partial(L.off1, L.off2)) throw Error{PCCL_ERR_LINK, op_name(*graphs[L.rank], L.rank, L.graph_pos) + ": src and dst ranges overlap without coinciding"};
+            if (L.peer == L.rank && partial(L.off0, L.dst_off())) throw Error{PCCL_ERR_LINK, op_name(*graphs[L.rank], L.rank, L.graph_pos) + ": reads and writes overlapping ranges of its own buffer"};
+        }
+    }
+
+    // ---- race check: conflicting accesses to one rank buffer must be ordered
+    if (opt.check_races && closure && D > 1) {
+        struct Acc { int rank; int64_t s, e; bool write; int op; };
+        std::vector<Acc> acc;
+        for (int k = 0; k < D; ++k) {
+            const LinkedOp& L = ops[k];
+            if (L.size <= 0) continue;
+            acc.push_back({L.peer, L.off0, L.off0 + L.size, false, k});
+            if (L.is_reduce) acc.push_back({L.rank, L.off1, L.off1 + L.size, false, k});
+            acc.push_back({L.rank, L.dst_off(), L.dst_off() + L.size, true, k});
+        }
+        std::sort(acc.begin(), acc.end(), [](const Acc& a, const Acc& b) { return a.rank != b.rank ? a.rank < b.rank : a.s < b.s; });
+        size_t pairs = 0;
+        bool complete = true;
+        for (size_t i = 0; i < acc.size() && complete; ++i)
+            for (size_t j = i + 1; j < acc.size() && acc[j].rank == acc[i].rank && acc[j].s < acc[i].e; ++j) {
+                if (++pairs > kPairLimit) { complete = false; break; }
+                if (!(acc[i].write || acc[j].write) || acc[i].op == acc[j].op) continue;
+                int a = data_nodes[acc[i].op], b = data_nodes[acc[j].op];
+                if (!reach[a].test(b) && !reach[b].test(a)) {
+                    const LinkedOp &A = ops[acc[i].op], &B = ops[acc[j].op];
+                    throw Error{PCCL_ERR_LINK, "data race on rank " + std::to_string(acc[i].rank) + " elements [" + std::to_string(std::max(acc[i].s, acc[j].s)) + ", " + std::to_string(std::min(acc[i].e, acc[j].e)) + "): " +
+                                                   op_name(*graphs[A.rank], A.rank, A.graph_pos) + " and " + op_name(*graphs[B.rank], B.rank, B.graph_pos) + " are not ordered by any notify/wait chain"};
+                }
+            }
+        P.race_checked = complete;
+    }
+
+    // ---- final order: (level, rank, channel, graph position); remap deps
+    std::vector<int> perm(D);
+    std::iota(perm.begin(), perm.end(), 0);
+    std::stable_sort(perm.begin(), perm.end(), [&](int a, int b) {
+        const LinkedOp &A = ops[a], &B = ops[b];
+        if (A.level != B.level) return A.level < B.level;
+        if (A.rank != B.rank) return A.rank < B.rank;
+        if (A.channel != B.channel) return A.channel < B.channel;
+        return A.graph_pos < B.graph_pos;
+    });
+    std::vector<int> inv(D);
+    for (int k = 0; k < D; ++k) inv[perm[k]] = k;
+    P.ops.resize(D);
+    for (int k = 0; k < D; ++k) {
+        P.ops[k] = ops[perm[k]];
+        for (int& d : P.ops[k].deps) d = inv[d];
+        std::sort(P.ops[k].deps.begin(), P.ops[k].deps.end());
+    }
+
+    // ---- stepwise plan
+    P.tile_elems = std::max<int64_t>(opt.step_tile_bytes / es, 1024);
+    P.step_ops.resize(D);
+    int64_t items = 0;
+    for (int k = 0; k < D; ++k) {
+        StepOpPlan& s = P.step_ops[k];
+        s.first_item = (int)items;
+        s.ntiles = (int)((P.ops[k].size + P.tile_elems - 1) / P.tile_elems);
+        s.dep_start = (int)P.step_deps.size();
+        s.ndeps = (int)P.ops[k].deps.size();
+        for (int d : P.ops[k].deps) P.step_deps.push_back(d);
+        items += s.ntiles;
+        if (items > INT32_MAX) throw Error{PCCL_ERR_UNSUPPORTED, "program has more than 2^31 work items"};
+    }
+    P.num_items = items;
+
+    // ---- column plan
+    P.position_aligned = D > 0;
+    for (auto& L : P.ops) if (!L.position_aligned()) { P.position_aligned = false; break; }
+    if (P.position_aligned) {
+        std::vector<int64_t> cuts;
+        for (auto& L : P.ops) if (L.size > 0) { cuts.push_back(L.off0); cuts.push_back(L.off0 + L.size); }
+        std::sort(cuts.begin(), cuts.end());
+        cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+        // ops covering each elementary interval, in program order
+        std::vector<std::vector<int>> cover(cuts.size() > 0 ? cuts.size() - 1 : 0);
+        for (int k = 0; k < D; ++k) {
+            const LinkedOp& L = P.ops[k];
+            if (L.size <= 0) continue;
+            size_t a = std::lower_bound(cuts.begin(), cuts.end(), L.off0) - cuts.begin();
+            size_t b = std::lower_bound(cuts.begin(), cuts.end(), L.off0 + L.size) - cuts.begin();
+            for (size_t i = a; i < b; ++i) cover[i].push_back(k);
+        }
+        // instruction signature of an op list (what the device program depends on)
+        auto sig = [&](const std::vector<int>& v) {
+            std::vector<int> s;
+            for (int k : v) { const LinkedOp& L = P.ops[k]; s.push_back(L.rank | L.peer << 8 | (int)L.is_reduce << 16 | L.redop << 17); }
+            return s;
+        };
+        std::vector<int> prev_sig;
+        for (size_t i = 0; i < cover.size(); ++i) {
+            if (cover[i].empty()) { prev_sig.clear(); continue; }
+            std::vector<int> s = sig(cover[i]);
+            if (!P.segs.empty() && P.segs.back().end == cuts[i] && s == prev_sig) { P.segs.back().end = cuts[i + 1]; continue; }
+            prev_sig = s;
+            ColSegment seg;
+            seg.start = cuts[i]; seg.end = cuts[i + 1];
+            seg.prog_start = (int)P.col_instrs.size();
+            seg.fifo_start = (int)P.col_fifo.size();
+            // build + optimise the column program
+            std::vector<ColInstr> prog;
+            uint64_t written = 0;  // ranks an earlier instruction of this program wrote
+            for (size_t n = 0; n < cover[i].size(); ++n) {
+                const LinkedOp& L = P.ops[cover[i][n]];
+                ColInstr in{};
+                in.self = (uint8_t)L.rank; in.peer = (uint8_t)L.peer; in.redop = (uint8_t)L.redop; in.store = 1;
+                bool prev_is_peer = n > 0 && prog.back().self == in.peer;
+                bool prev_is_self = n > 0 && prog.back().self == in.self;
+                in.a_src = prev_is_peer ? SRC_ACC : SRC_MEM;
+                in.b_src = !L.is_reduce ? SRC_NONE : prev_is_self ? SRC_ACC : SRC_MEM;
+                if (in.a_src == SRC_MEM) in.a_first = !(written >> in.peer & 1);
+                if (in.b_src == SRC_MEM) in.b_first = !(written >> in.self & 1);
+                written |= 1ull << in.self;
+                prog.push_back(in);
+            }
+            // dead stores: overwritten before any later instruction reads that rank from memory
+            for (size_t n = 0; n < prog.size(); ++n) {
+                for (size_t m = n + 1; m < prog.size(); ++m) {
+                    bool reads = (prog[m].a_src != SRC_ACC && prog[m].peer == prog[n].self) ||
+                                 (prog[m].b_src == SRC_MEM && prog[m].self == prog[n].self);
+                    if (reads) break;
+                    if (prog[m].self == prog[n].self) { prog[n].store = 0; break; }
+                }
+            }
+            // first-touch loads may be issued early through the FIFO (nothing before them writes
+            // the location, so any earlier issue point reads the same value)
+            if (opt.fifo_depth > 0)
+                for (auto& in : prog) {
+                    if (in.a_src == SRC_MEM && in.a_first) { in.a_src = SRC_FIFO; P.col_fifo.push_back(in.peer); }
+                    if (in.b_src == SRC_MEM && in.b_first) { in.b_src = SRC_FIFO; P.col_fifo.push_back(in.self); }
+                }
+            seg.prog_len = (int)prog.size();
+            seg.fifo_len = (int)P.col_fifo.size() - seg.fifo_start;
+            P.col_instrs.insert(P.col_instrs.end(), prog.begin(), prog.end());
+            P.segs.push_back(seg);
+        }
+        for (auto& seg : P.segs) {
+            int64_t n = seg.end - seg.start;
+            for (int k = 0; k < seg.prog_len; ++k) {
+                const ColInstr& in = P.col_instrs[seg.prog_start + k];
+                if (in.a_src == SRC_MEM || in.a_src == SRC_FIFO) P.column_load_bytes += n * es;
+                if (in.b_src == SRC_MEM || in.b_src == SRC_FIFO) P.column_load_bytes += n * es;
+                if (in.store) P.column_store_bytes += n * es;
+            }
+        }
+    }
+    return P;
+}
+
+}  // namespace pccl_hip

@@ -1,0 +1,89 @@
+// Linked program: R per-rank graphs folded into one dependency graph of data ops, plus the two
+// execution plans derived from it (column plan and stepwise plan).
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "graph.h"
+
+namespace pccl_hip {
+
+struct LinkedOp {
+    int rank = 0, channel = 0, graph_pos = 0, index = 0;
+    bool is_reduce = false;
+    int redop = PCCL_SUM;
+    int peer = 0;
+    int64_t off0 = 0, off1 = 0, off2 = 0, size = 0;
+    int level = 0;
+    std::vector<int> deps;  // indices into Program::ops (after ordering)
+
+    int64_t dst_off() const { return is_reduce ? off2 : off1; }
+    bool position_aligned() const { return is_reduce ? (off0 == off1 && off1 == off2) : (off0 == off1); }
+};
+
+// Operand sources of a column instruction.
+enum : uint8_t { SRC_NONE = 0, SRC_MEM = 1, SRC_ACC = 2, SRC_FIFO = 3 };
+
+// One step of a segment's column program: acc = a (copy) or acc = a (op) b (reduce), then
+// optionally mem[self] = acc.  a is the peer's value, b the own value.
+struct ColInstr {
+    uint8_t self;
+    uint8_t peer;
+    uint8_t a_src;   // SRC_MEM | SRC_ACC | SRC_FIFO
+    uint8_t b_src;   // SRC_NONE (copy) | SRC_MEM | SRC_ACC | SRC_FIFO
+    uint8_t redop;
+    uint8_t store;   // 0: the write is dead (overwritten before anything reads it from memory)
+    uint8_t a_first; // 1: this load is the first access to (peer, position) in the program
+    uint8_t b_first;
+};
+static_assert(sizeof(ColInstr) == 8, "ColInstr is read as one 8-byte word on the device");
+
+struct ColSegment {
+    int64_t start = 0, end = 0;  // element positions [start, end)
+    int32_t prog_start = 0, prog_len = 0;
+    int32_t fifo_start = 0, fifo_len = 0;  // entries in Program::col_fifo (ranks, consumption order)
+};
+
+struct StepOpPlan {
+    int first_item = 0, ntiles = 0, dep_start = 0, ndeps = 0;
+};
+
+struct Program {
+    int R = 0;
+    int dtype = PCCL_F32;
+    std::string collective_type;
+    int64_t tensor_elems = 0;
+    std::vector<LinkedOp> ops;  // topological order: (level, rank, channel, position)
+    int num_all_ops = 0;
+    int num_levels = 0;
+    int residual_signals = 0;
+    int64_t buffer_elems = 0;
+    int64_t algorithmic_bytes = 0;
+    bool race_checked = false;
+
+    // column plan (valid when position_aligned)
+    bool position_aligned = false;
+    std::vector<ColSegment> segs;
+    std::vector<ColInstr> col_instrs;
+    std::vector<uint8_t> col_fifo;
+    int64_t column_load_bytes = 0, column_store_bytes = 0;
+
+    // stepwise plan
+    int64_t tile_elems = 0;
+    std::vector<StepOpPlan> step_ops;
+    std::vector<int32_t> step_deps;
+    int64_t num_items = 0;
+};
+
+struct LinkOptions {
+    bool check_races = true;
+    int fifo_depth = 0;            // 0: every first-touch load is SRC_MEM
+    int64_t step_tile_bytes = 128 * 1024;
+};
+
+// Throws Error (PCCL_ERR_LINK for deadlock, ambiguous signal pairing, races, bad ranks).
+Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOptions& opt);
+
+}  // namespace pccl_hip

@@ -7,8 +7,9 @@ step opens with a "my earlier ops are done" notify, and only the last doubling s
 acknowledged so all semaphores return to zero.
 
 Extension: ``num_channels > 1`` (the reference always emits channel 0).  Channel ``c`` runs the
-same schedule on the slice ``[c*seg/C, (c+1)*seg/C)`` of every segment, on stream ``ch{c}`` with
-signal ids ``c*1000 + sender`` (the ring templates' id convention).
+whole schedule on its own slice ``[c*N/C, (c+1)*N/C)`` of the tensor (halving that slice step by
+step), on stream ``ch{c}`` with signal ids ``c*1000 + sender`` (the ring templates' id
+convention), so channels never touch each other's positions.
 """
 from __future__ import annotations
 
@@ -26,34 +27,30 @@ class RecursiveHalvingDoubling(CollectiveAlgorithm):
                         num_channels=1, reduce_op="sum", cuts=None) -> Graph:
         log_n = require_power_of_two("RecursiveHalvingDoubling", world_size)
 
+        per_ch = tensor_size // num_channels
+
         def region_start(k: int) -> int:
-            return sum(tensor_size >> (j + 1) for j in range(k) if rank >> j & 1)
+            return sum(per_ch >> (j + 1) for j in range(k) if rank >> j & 1)
 
         with CommunicationOp(name=f"rhd_ar_{executor}_rank{rank}") as op:
             op.tensor(dtype=dtype, shape=(tensor_size,))
             em = _Emit(op, executor, reduce_op, cuts)
             for c in range(num_channels):
-                sig = c * 1000
+                sig, base = c * 1000, c * per_ch
                 with Stream("main" if num_channels == 1 else f"ch{c}"):
                     op.set_channel(c)
-
-                    def sub(off: int, seg: int):
-                        lo = c * seg // num_channels
-                        hi = (c + 1) * seg // num_channels
-                        return off + lo, hi - lo
-
                     for k in range(log_n):
-                        partner, seg = rank ^ (1 << k), tensor_size >> (k + 1)
-                        keep = region_start(k) + (seg if rank >> k & 1 else 0)
+                        partner, seg = rank ^ (1 << k), per_ch >> (k + 1)
+                        keep = base + region_start(k) + (seg if rank >> k & 1 else 0)
                         op.notify(signal_id=sig + rank, target_rank=partner)
                         op.wait_notify(signal_id=sig + partner, source_rank=partner)
-                        em.reduce(partner, *sub(keep, seg))
+                        em.reduce(partner, keep, seg)
                     for k in range(log_n - 1, -1, -1):
-                        partner, seg = rank ^ (1 << k), tensor_size >> (k + 1)
-                        fetch = region_start(k) + (0 if rank >> k & 1 else seg)
+                        partner, seg = rank ^ (1 << k), per_ch >> (k + 1)
+                        fetch = base + region_start(k) + (0 if rank >> k & 1 else seg)
                         op.notify(signal_id=sig + rank, target_rank=partner)
                         op.wait_notify(signal_id=sig + partner, source_rank=partner)
-                        em.copy(partner, *sub(fetch, seg))
+                        em.copy(partner, fetch, seg)
                         if k == 0:
                             op.notify(signal_id=sig + rank, target_rank=partner)
                     op.wait_notify(signal_id=sig + (rank ^ 1), source_rank=rank ^ 1)

@@ -1,0 +1,240 @@
+"""Engine facade: the reference's ``pccl.engine`` call surface over the HIP executor.
+
+Reference (pccl/engine.py:11-71): ``register_operation(name, filename) -> bool``,
+``execute_operation(name, input, output=None) -> Tensor`` (allocates ``empty_like`` and
+synchronises), ``execute_operation_async`` (no sync), ``sync_operation(name)``,
+``reset_signals(name)``, ``get_engine()``.  There every process is one rank and ``RANK`` comes from
+the environment.  Here one process holds all R ranks of a schedule as *virtual ranks* on one GPU:
+
+* collective form: ``engine.execute_operation(name, [in_0 .. in_{R-1}], [out_0 ..])`` — lists (or an
+  ``[R, N]`` tensor) instead of one tensor;
+* per-rank form, for code written against the reference: ``engine.rank(r)`` returns a view with the
+  reference's exact single-rank signatures; ``execute_operation_async`` posts that rank's tensors and
+  the launch happens when the last rank has posted (``execute_operation`` on a view is only legal
+  once every other rank has posted, because it synchronises).
+
+All work is enqueued on the current PyTorch stream, like the reference
+(csrc/plugins/cuda/cuda_device.cc:245-248,301).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from . import _lib
+from ._lib import PcclError
+
+TensorList = Union[Sequence[torch.Tensor], torch.Tensor]
+
+
+def _current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class Engine:
+    def __init__(self, num_vranks: Optional[int] = None, device: int = 0):
+        if num_vranks is None:
+            num_vranks = int(os.environ.get("PCCL_VRANKS", "0"))
+        if num_vranks <= 0:
+            raise RuntimeError("number of virtual ranks not given: pass num_vranks or set PCCL_VRANKS")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible: the HIP executor has no CPU fallback")
+        self.num_vranks = num_vranks
+        self.device = torch.device("cuda", device)
+        self._L = _lib.lib()
+        h = ctypes.c_void_p()
+        _lib.check(self._L.pccl_hip_create(ctypes.byref(h), device, num_vranks))
+        self._h = h
+        self._posted: Dict[str, Dict[int, tuple]] = {}
+        self._views = [RankView(self, r) for r in range(num_vranks)]
+
+    def close(self) -> None:
+        if getattr(self, "_h", None):
+            self._L.pccl_hip_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- registration -------------------------------------------------------------------------
+    def register_operation(self, name: str, filename: str, rank: Optional[int] = None) -> bool:
+        """Register rank ``rank``'s graph file; with ``rank=None`` ``filename`` must contain
+        ``{rank}`` and all virtual ranks are registered.  Returns False when a file cannot be
+        loaded (like the reference's ``regOp``); a bad primitive or dtype raises."""
+        ranks = [rank] if rank is not None else list(range(self.num_vranks))
+        if rank is None and "{rank}" not in filename:
+            raise ValueError("register_operation without rank needs a '{rank}' placeholder in filename")
+        for r in ranks:
+            path = filename.format(rank=r) if "{rank}" in filename else filename
+            rc = self._L.pccl_hip_register_file(self._h, name.encode(), r, path.encode())
+            if rc in (_lib.ERR_NOT_FOUND,):
+                return False
+            if rc == _lib.ERR_PARSE and "lacks index/executor/primitive" in self.last_error() or \
+               rc == _lib.ERR_PARSE and "no 'operations'" in self.last_error():
+                return False
+            _lib.check(rc)
+        return True
+
+    def register_operation_json(self, name: str, text: str, rank: int) -> bool:
+        data = text.encode()
+        _lib.check(self._L.pccl_hip_register_json(self._h, name.encode(), rank, data, len(data)))
+        return True
+
+    def last_error(self) -> str:
+        return self._L.pccl_hip_last_error().decode(errors="replace")
+
+    def set_option(self, key: str, value) -> None:
+        _lib.check(self._L.pccl_hip_set_option(self._h, key.encode(), str(value).encode()))
+
+    # -- execution ----------------------------------------------------------------------------
+    def _as_list(self, t: TensorList, what: str) -> List[torch.Tensor]:
+        ts = list(t.unbind(0)) if isinstance(t, torch.Tensor) else list(t)
+        if len(ts) != self.num_vranks:
+            raise ValueError(f"{what}: expected {self.num_vranks} tensors, got {len(ts)}")
+        for x in ts:
+            if not x.is_cuda:
+                raise ValueError(f"{what}: tensors must live on the GPU")
+            if not x.is_contiguous():
+                raise ValueError(f"{what}: tensors must be contiguous")
+        return ts
+
+    def _ptrs(self, ts: List[torch.Tensor]):
+        return (ctypes.c_void_p * len(ts))(*[x.data_ptr() for x in ts])
+
+    def _launch(self, name: str, inputs: List[torch.Tensor], outputs: List[torch.Tensor], sync: bool):
+        nb_in, nb_out = inputs[0].nbytes, outputs[0].nbytes
+        if any(x.nbytes != nb_in for x in inputs) or any(x.nbytes != nb_out for x in outputs):
+            raise ValueError("all ranks must pass tensors of the same size")
+        _lib.check(self._L.pccl_hip_execute(self._h, name.encode(), self._ptrs(inputs), self._ptrs(outputs),
+                                            nb_in, nb_out, _current_stream_ptr(self.device), int(sync)))
+
+    def execute_operation(self, name: str, inputs: TensorList, outputs: Optional[TensorList] = None):
+        ins = self._as_list(inputs, "inputs")
+        outs = [torch.empty_like(x) for x in ins] if outputs is None else self._as_list(outputs, "outputs")
+        self._launch(name, ins, outs, True)
+        return outs
+
+    def execute_operation_async(self, name: str, inputs: TensorList, outputs: Optional[TensorList] = None):
+        ins = self._as_list(inputs, "inputs")
+        outs = [torch.empty_like(x) for x in ins] if outputs is None else self._as_list(outputs, "outputs")
+        self._launch(name, ins, outs, False)
+        return outs
+
+    def execute_inplace(self, name: str, bufs: TensorList, sync: bool = False):
+        """Zero-copy execution: ``bufs[r]`` is rank ``r``'s buffer and is updated in place."""
+        bs = self._as_list(bufs, "bufs")
+        _lib.check(self._L.pccl_hip_execute_inplace(self._h, name.encode(), self._ptrs(bs), bs[0].nbytes,
+                                                    _current_stream_ptr(self.device), int(sync)))
+        return bs
+
+    def sync_operation(self, name: str) -> None:
+        _lib.check(self._L.pccl_hip_sync(self._h, name.encode()))
+
+    def reset_signals(self, name: str) -> None:
+        _lib.check(self._L.pccl_hip_reset_signals(self._h, name.encode()))
+
+    def op_info(self, name: str) -> dict:
+        out = _lib.ProgramInfo()
+        _lib.check(self._L.pccl_hip_op_info(self._h, name.encode(), ctypes.byref(out)))
+        return out.as_dict()
+
+    def last_kernel_ms(self, name: str) -> float:
+        ms = ctypes.c_float()
+        _lib.check(self._L.pccl_hip_last_kernel_ms(self._h, name.encode(), ctypes.byref(ms)))
+        return ms.value
+
+    # -- per-rank views -----------------------------------------------------------------------
+    def rank(self, r: int) -> "RankView":
+        return self._views[r]
+
+    def _post(self, name: str, r: int, inp: torch.Tensor, out: torch.Tensor, sync: bool):
+        slot = self._posted.setdefault(name, {})
+        if r in slot:
+            raise RuntimeError(f"rank {r} posted '{name}' twice before the other ranks arrived")
+        slot[r] = (inp, out)
+        if len(slot) < self.num_vranks:
+            if sync:
+                del slot[r]
+                raise RuntimeError(
+                    f"execute_operation('{name}') on rank {r} would block: only {len(slot) + 1} of "
+                    f"{self.num_vranks} virtual ranks have posted; post the others with "
+                    "execute_operation_async first")
+            return
+        ins = self._as_list([slot[i][0] for i in range(self.num_vranks)], "inputs")
+        outs = self._as_list([slot[i][1] for i in range(self.num_vranks)], "outputs")
+        del self._posted[name]
+        self._launch(name, ins, outs, sync)
+
+
+class RankView:
+    """The reference's single-rank API for one virtual rank."""
+
+    def __init__(self, engine: Engine, rank: int):
+        self.engine, self.rank = engine, rank
+
+    def register_operation(self, name: str, filename: str) -> bool:
+        return self.engine.register_operation(name, filename, rank=self.rank)
+
+    def execute_operation(self, name, input_tensor, output_tensor=None):
+        if output_tensor is None:
+            output_tensor = torch.empty_like(input_tensor)
+        self.engine._post(name, self.rank, input_tensor, output_tensor, True)
+        return output_tensor
+
+    def execute_operation_async(self, name, input_tensor, output_tensor=None):
+        if output_tensor is None:
+            output_tensor = torch.empty_like(input_tensor)
+        self.engine._post(name, self.rank, input_tensor, output_tensor, False)
+        return output_tensor
+
+    def sync_operation(self, name):
+        self.engine.sync_operation(name)
+
+    def reset_signals(self, name):
+        self.engine.reset_signals(name)
+
+
+_engine_instance: Optional[Engine] = None
+
+
+def initialize_engine(num_vranks: Optional[int] = None, device: int = 0) -> Engine:
+    """Create the process-wide engine (the reference's ``initialize_engine(group)`` exchanges
+    endpoints between processes; with virtual ranks there is nothing to exchange)."""
+    global _engine_instance
+    if _engine_instance is not None:
+        _engine_instance.close()
+    _engine_instance = Engine(num_vranks, device)
+    return _engine_instance
+
+
+def get_engine() -> Engine:
+    global _engine_instance
+    if _engine_instance is None:
+        _engine_instance = Engine()
+    return _engine_instance
+
+
+def register_operation(name, filename, rank=None):
+    return get_engine().register_operation(name, filename, rank)
+
+
+def execute_operation(name, input_tensor, output_tensor=None):
+    return get_engine().execute_operation(name, input_tensor, output_tensor)
+
+
+def execute_operation_async(name, input_tensor, output_tensor=None):
+    return get_engine().execute_operation_async(name, input_tensor, output_tensor)
+
+
+def sync_operation(name):
+    return get_engine().sync_operation(name)
+
+
+def reset_signals(name):
+    return get_engine().reset_signals(name)

@@ -1,0 +1,107 @@
+"""Shared test utilities: graph generation, seeded inputs, and the oracle leg.
+
+The oracle (oracle/) is imported here and only here on the test side; the product package never
+sees it.
+"""
+from __future__ import annotations
+
+import json
+import os
+import sys
+from typing import List, Sequence
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from oracle import oracle  # noqa: E402
+from pccl_amd.dsl import ALGORITHMS, compile_to_json_string  # noqa: E402
+
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+TORCH_DTYPE = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16,
+               "int32": torch.int32}
+RAW_NP = {"float32": np.float32, "float16": np.uint16, "bfloat16": np.uint16, "int32": np.int32}
+
+
+def graph_jsons(alg: str, method: str, world: int, n: int, dtype: str, executor: str = "sm",
+                channels: int = 1, **ext) -> List[str]:
+    a = ALGORITHMS[alg]()
+    return [compile_to_json_string(getattr(a, method)(r, world, n, dtype=dtype, executor=executor,
+                                                      num_channels=channels, **ext))
+            for r in range(world)]
+
+
+def to_raw(t: torch.Tensor) -> np.ndarray:
+    """CPU tensor -> numpy array of its storage bits (bf16/f16 as uint16)."""
+    t = t.contiguous()
+    if t.dtype in (torch.bfloat16, torch.float16):
+        return t.view(torch.int16).numpy().view(np.uint16).copy()
+    return t.numpy().copy()
+
+
+def from_raw(a: np.ndarray, dtype: str) -> torch.Tensor:
+    if dtype in ("bfloat16", "float16"):
+        return torch.from_numpy(a.view(np.int16).copy()).view(TORCH_DTYPE[dtype])
+    return torch.from_numpy(a.copy())
+
+
+def seeded_inputs(kind: str, world: int, n: int, dtype: str, seed: int = 0) -> List[torch.Tensor]:
+    """CPU-generator inputs, one row per rank, as the configurations prescribe."""
+    g = torch.Generator().manual_seed(seed)
+    if kind == "randn":
+        x = torch.randn(world, n, generator=g)
+    elif kind == "uniform":
+        x = torch.rand(world, n, generator=g) * 2 - 1
+    elif kind == "randn0.1":
+        x = torch.randn(world, n, generator=g) * 0.1
+    elif kind == "randint":
+        x = torch.randint(-1000, 1000, (world, n), generator=g)
+    elif kind == "rank+1":
+        x = torch.arange(1, world + 1).view(world, 1).expand(world, n).float()
+    else:
+        raise ValueError(kind)
+    return [x[r].to(TORCH_DTYPE[dtype]).contiguous() for r in range(world)]
+
+
+def oracle_buffers(jsons: Sequence[str], inputs: Sequence[torch.Tensor], dtype: str,
+                   sched_seed: int = 0, buffer_elems: int = 0, place=None,
+                   threads: int = 0) -> List[torch.Tensor]:
+    """Run the graphs on the CPU oracle.  Rank r's buffer starts as zeros with inputs[r] copied in
+    at element offset place(r) (default 0); returns the final buffers."""
+    graphs = [oracle.Graph(json.loads(j)) for j in jsons]
+    n = max(buffer_elems, max(len(x) + (place(r) if place else 0) for r, x in enumerate(inputs)))
+    bufs = []
+    for r, x in enumerate(inputs):
+        raw = np.zeros(n, dtype=RAW_NP[dtype])
+        off = place(r) if place else 0
+        raw[off:off + len(x)] = to_raw(x)
+        bufs.append(raw)
+    oracle.run(graphs, bufs, sched_seed=sched_seed, threads=threads)
+    return [from_raw(b, dtype) for b in bufs]
+
+
+def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
+    a, b = a.cpu().contiguous(), b.cpu().contiguous()
+    if a.dtype in (torch.bfloat16, torch.float16):
+        return torch.equal(a.view(torch.int16), b.view(torch.int16))
+    if a.dtype == torch.float32:
+        return torch.equal(a.view(torch.int32), b.view(torch.int32))
+    return torch.equal(a, b)
+
+
+def mismatch_report(a: torch.Tensor, b: torch.Tensor) -> str:
+    a, b = a.cpu(), b.cpu()
+    if a.dtype in (torch.bfloat16, torch.float16):
+        ne = (a.view(torch.int16) != b.view(torch.int16)).nonzero().flatten()
+    elif a.dtype == torch.float32:
+        ne = (a.view(torch.int32) != b.view(torch.int32)).nonzero().flatten()
+    else:
+        ne = (a != b).nonzero().flatten()
+    if len(ne) == 0:
+        return "equal"
+    i = int(ne[0])
+    return f"{len(ne)} of {a.numel()} differ; first at {i}: got {a[i].item()} expected {b[i].item()}"

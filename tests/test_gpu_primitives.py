@@ -1,0 +1,101 @@
+"""GPU parity of the two data primitives on their own (reduce, copy) against the CPU oracle.
+
+Reference: executeReduce / executeCopy -> vector_add / vector_copy
+(csrc/plugins/cuda/cuda_executor.cu:60-101, kernel/compute.h:21-102).  Bit-exact for every dtype;
+sizes and offsets that are not multiples of 16 bytes are included (the reference drops such tails;
+here they are processed, see the oracle header).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import TORCH_DTYPE, bits_equal, from_raw, mismatch_report, oracle, to_raw
+from pccl_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+
+def gpu_reduce(dtype, redop, a, b, c_out):
+    L = _lib.lib()
+    n = a.numel()
+    _lib.check(L.pccl_hip_reduce(_lib.DTYPE_ID[dtype], _lib.REDOP_ID[redop], a.data_ptr(), b.data_ptr(),
+                                 c_out.data_ptr(), n, None))
+    torch.cuda.synchronize()
+
+
+def make(dtype, n, seed, special=False):
+    g = torch.Generator().manual_seed(seed)
+    if dtype == "int32":
+        x = torch.randint(-2**31, 2**31 - 1, (n,), generator=g, dtype=torch.int64).to(torch.int32)
+    else:
+        x = (torch.randn(n, generator=g) * 3).to(TORCH_DTYPE[dtype])
+        if special and n >= 16:
+            vals = torch.tensor([float("inf"), float("-inf"), float("nan"), 0.0, -0.0, 65504.0, -65504.0,
+                                 1e-8, -1e-8, 3.0e38, -3.0e38, 6e-5, 1e-40, 1.0, -1.0, 0.5]).to(TORCH_DTYPE[dtype])
+            x[:16] = vals
+    return x
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16", "int32"])
+@pytest.mark.parametrize("redop", ["sum", "max", "min"])
+@pytest.mark.parametrize("n", [1, 7, 64, 4099, 1 << 20])
+def test_reduce_matches_oracle(dtype, redop, n):
+    a, b = make(dtype, n, 1, special=True), make(dtype, n, 2, special=True)
+    if n >= 16:
+        b[:16] = a[:16].flip(0)   # inf + -inf, nan with anything, +0 with -0 ...
+    want = from_raw(oracle.reduce(dtype, redop, to_raw(a), to_raw(b)), dtype)
+    da, db = a.cuda(), b.cuda()
+    dc = torch.empty_like(da)
+    gpu_reduce(dtype, redop, da, db, dc)
+    assert bits_equal(dc, want), mismatch_report(dc, want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shift", [(0, 0, 0), (1, 1, 1), (3, 3, 3), (1, 2, 3), (0, 1, 0)])
+def test_reduce_unaligned_offsets(dtype, shift):
+    """Element offsets that break 16-byte alignment, equal and unequal between the operands."""
+    n = 10007
+    a, b = make(dtype, n + 8, 3), make(dtype, n + 8, 4)
+    sa, sb, sc = shift
+    want = from_raw(oracle.reduce(dtype, "sum", to_raw(a[sa:sa + n]), to_raw(b[sb:sb + n])), dtype)
+    da, db = a.cuda(), b.cuda()
+    dc = torch.zeros(n + 8, dtype=TORCH_DTYPE[dtype], device="cuda")
+    gpu_reduce(dtype, "sum", da[sa:sa + n], db[sb:sb + n], dc[sc:sc + n])
+    assert bits_equal(dc[sc:sc + n], want), mismatch_report(dc[sc:sc + n], want)
+    assert torch.all(dc[:sc] == 0) and torch.all(dc[sc + n:] == 0), "wrote outside the range"
+
+
+def test_reduce_in_place_aliasing():
+    """c aliases b, as every schedule of the reference uses it (off1 == off2)."""
+    n = 1 << 16
+    a, b = make("bfloat16", n, 5), make("bfloat16", n, 6)
+    want = from_raw(oracle.reduce("bfloat16", "sum", to_raw(a), to_raw(b)), "bfloat16")
+    da, db = a.cuda(), b.cuda()
+    gpu_reduce("bfloat16", "sum", da, db, db)
+    assert bits_equal(db, want)
+
+
+@pytest.mark.parametrize("nbytes", [1, 15, 16, 17, 4096, 65537, 1 << 22])
+@pytest.mark.parametrize("shift", [(0, 0), (1, 1), (5, 5), (1, 2)])
+def test_copy_bytes(nbytes, shift):
+    L = _lib.lib()
+    src = torch.randint(0, 256, (nbytes + 16,), dtype=torch.uint8)
+    dsrc = src.cuda()
+    ddst = torch.zeros(nbytes + 16, dtype=torch.uint8, device="cuda")
+    s, d = shift
+    _lib.check(L.pccl_hip_copy(_lib.DTYPE_ID["float8_e4m3"], dsrc[s:].data_ptr(), ddst[d:].data_ptr(), nbytes, None))
+    torch.cuda.synchronize()
+    out = ddst.cpu()
+    assert torch.equal(out[d:d + nbytes], src[s:s + nbytes])
+    assert torch.all(out[:d] == 0) and torch.all(out[d + nbytes:] == 0)
+
+
+def test_bad_arguments_are_errors():
+    L = _lib.lib()
+    x = torch.zeros(16, device="cuda")
+    assert L.pccl_hip_reduce(3, 0, x.data_ptr(), x.data_ptr(), x.data_ptr(), 4, None) == _lib.ERR_UNSUPPORTED
+    assert L.pccl_hip_reduce(0, 9, x.data_ptr(), x.data_ptr(), x.data_ptr(), 4, None) == _lib.ERR_INVALID
+    assert L.pccl_hip_reduce(0, 0, None, x.data_ptr(), x.data_ptr(), 4, None) == _lib.ERR_INVALID
+    assert b"null" in L.pccl_hip_last_error()
