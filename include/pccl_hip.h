@@ -184,9 +184,10 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
                                const char* collective_type);
 
 /* Options, the counterpart of the reference's environment switches (csrc/plugins/cuda/cuda_device.cc:
- * 289-298, csrc/engine_c.cc:351): key "mode" = "auto" | "column" | "stepwise";
- * "num_blocks" = workgroups of the persistent launch (0 = fill the device);
- * "check_races" = "0" | "1". */
+ * 289-298, csrc/engine_c.cc:351): key "mode" = "auto" | "column" | "stepwise" | "persistent";
+ * "num_blocks" = workgroup cap of a launch (0 = sized to the device); "check_races" = "0" | "1";
+ * "timing" = "0" | "1" (record HIP events around the program); "vecs_per_thread" = 1 | 2 | 4;
+ * "step_tile_bytes"; "spin_limit" (polls before a wait of the persistent runner gives up). */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
 
 /* Engine::exeOp / exeOpAsync (reference csrc/engine_c.cc:269-560): for every virtual rank r copy

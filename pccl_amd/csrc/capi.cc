@@ -204,6 +204,8 @@ struct OpEntry {
     int vecs_per_thread = 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool timed = false;
+    bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
+    std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
     void release() {
         segs.release(); instrs.release(); fifo.release(); step_ops.release(); step_deps.release();
         item_op.release(); state.release();
@@ -214,7 +216,7 @@ struct OpEntry {
     }
 };
 
-enum class Mode { Auto, Column, Stepwise };
+enum class Mode { Auto, Column, Stepwise, Persistent };
 
 }  // namespace
 
@@ -232,6 +234,7 @@ struct pccl_hip_ctx {
     bool timing = false;
     int fifo_depth = 0;
     int64_t step_tile_bytes = 128 * 1024;
+    int spin_limit = 1 << 22;             // polls (~0.1 us sleep each) before a persistent wait gives up
     hipStream_t last_stream = nullptr;
 };
 
@@ -301,6 +304,10 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
             if (d.ndeps > 256) throw Error{PCCL_ERR_UNSUPPORTED, "a data op with more than 256 direct predecessors"};
             for (int t = 0; t < d.ntiles; ++t) item_op[(size_t)d.first_item + t] = (int32_t)k;
         }
+        e.level_item_begin.clear();
+        for (size_t k = 0; k < P.ops.size(); ++k)
+            if (k == 0 || P.ops[k].level != P.ops[k - 1].level) e.level_item_begin.push_back(P.step_ops[k].first_item);
+        e.level_item_begin.push_back((int)P.num_items);
         e.step_ops.upload(so.data(), so.size() * sizeof(DevStepOp));
         e.step_deps.upload(P.step_deps.data(), P.step_deps.size() * sizeof(int32_t));
         e.item_op.upload(item_op.data(), item_op.size() * sizeof(int32_t));
@@ -336,7 +343,7 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
         ptrs.p[PCCL_HIP_MAX_VRANKS + r] = rank_bufs[r];
     }
     bool column = P.position_aligned && aligned16;
-    if (ctx->mode == Mode::Stepwise) column = false;
+    if (ctx->mode == Mode::Stepwise || ctx->mode == Mode::Persistent) column = false;
     if (ctx->mode == Mode::Column && !column)
         throw Error{PCCL_ERR_UNSUPPORTED, P.position_aligned ? "column mode needs 16-byte aligned rank buffers" : "column mode needs every data op to read and write the same element positions"};
     if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
@@ -353,11 +360,35 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
         L.ops = (const DevStepOp*)e.step_ops.p; L.num_ops = (int)P.ops.size();
         L.deps = (const int32_t*)e.step_deps.p; L.item_op = (const int32_t*)e.item_op.p;
         L.num_items = (int)P.num_items; L.tile_elems = P.tile_elems; L.state = (StepState*)e.state.p;
-        L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
-        rc = launch_stepwise(L, ptrs, stream);
+        L.dtype = P.dtype; L.num_blocks = ctx->num_blocks; L.spin_limit = ctx->spin_limit;
+        if (ctx->mode == Mode::Persistent) {
+            rc = launch_persistent(L, ptrs, stream);
+            e.ran_persistent = true;
+        } else {
+            rc = 0;
+            for (size_t l = 0; l + 1 < e.level_item_begin.size() && rc == 0; ++l)
+                rc = launch_level(L, e.level_item_begin[l], e.level_item_begin[l + 1], ptrs, stream);
+        }
     }
     if (rc != 0) throw Error{PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)};
     if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, stream)); e.timed = true; }
+}
+
+// After the stream has drained: did a bounded wait of the persistent runner expire?
+void check_stall(OpEntry& e, const std::string& name) {
+    if (!e.ran_persistent || !e.state.p) return;
+    e.ran_persistent = false;
+    StepState st;
+    HIP_TRY(hipMemcpy(&st, e.state.p, sizeof(st), hipMemcpyDeviceToHost));
+    if (st.error_op == 0) return;
+    std::vector<char> zeros(e.state.bytes, 0);
+    HIP_TRY(hipMemcpy(e.state.p, zeros.data(), zeros.size(), hipMemcpyHostToDevice));
+    const LinkedOp& a = e.prog.ops[st.error_op - 1];
+    const LinkedOp& b = e.prog.ops[st.error_dep - 1];
+    throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting: data op " + std::to_string(st.error_op - 1) +
+                                  " (rank " + std::to_string(a.rank) + ", level " + std::to_string(a.level) + ") never saw its predecessor " +
+                                  std::to_string(st.error_dep - 1) + " (rank " + std::to_string(b.rank) + ", level " + std::to_string(b.level) +
+                                  ") complete; rank buffers are partially updated"};
 }
 
 int register_graph(pccl_hip_ctx* ctx, const char* name, int vrank, RankGraph&& g) {
@@ -436,9 +467,18 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             if (v == "auto") ctx->mode = Mode::Auto;
             else if (v == "column") ctx->mode = Mode::Column;
             else if (v == "stepwise") ctx->mode = Mode::Stepwise;
-            else return fail(PCCL_ERR_INVALID, "mode must be auto, column or stepwise");
+            else if (v == "persistent") {
+                // The single-launch flag-ordered runner stopped making progress on MI355X in its
+                // first runs and the cause has not been established; until it is, the mode is
+                // refused rather than launched.  PCCL_ENABLE_PERSISTENT=1 is for developers only.
+                if (!std::getenv("PCCL_ENABLE_PERSISTENT"))
+                    return fail(PCCL_ERR_UNSUPPORTED, "mode 'persistent' is switched off: the flag-ordered single-launch runner hangs on MI355X (cause not yet established); use 'stepwise' or 'column'");
+                ctx->mode = Mode::Persistent;
+            }
+            else return fail(PCCL_ERR_INVALID, "mode must be auto, column, stepwise or persistent");
         } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
         else if (k == "timing") ctx->timing = std::atoi(value) != 0;
+        else if (k == "spin_limit") { ctx->spin_limit = std::atoi(value); if (ctx->spin_limit < 1) ctx->spin_limit = 1; }
         else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
         else if (k == "vecs_per_thread") {
             int u = std::atoi(value);
@@ -517,7 +557,7 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
         }
         if (rc) return fail(PCCL_ERR_HIP, std::string("output staging: ") + hipGetErrorString((hipError_t)rc));
         ctx->last_stream = s;
-        if (sync) HIP_TRY(hipStreamSynchronize(s));
+        if (sync) { HIP_TRY(hipStreamSynchronize(s)); check_stall(e, name); }
         return 0;
     });
 }
@@ -533,7 +573,7 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
         hipStream_t s = (hipStream_t)stream;
         run_program(ctx, e, (char* const*)bufs, buf_bytes, s);
         ctx->last_stream = s;
-        if (sync) HIP_TRY(hipStreamSynchronize(s));
+        if (sync) { HIP_TRY(hipStreamSynchronize(s)); check_stall(e, name); }
         return 0;
     });
 }
@@ -542,9 +582,11 @@ int pccl_hip_sync(pccl_hip_ctx* ctx, const char* name) {
     return guarded([&] {
         if (!ctx) return fail(PCCL_ERR_INVALID, "null argument");
         std::lock_guard<std::mutex> lock(ctx->mu);
-        if (ctx->ops.find(name ? name : "") == ctx->ops.end()) return 0;  // the reference returns silently
+        auto it = ctx->ops.find(name ? name : "");
+        if (it == ctx->ops.end()) return 0;  // the reference returns silently
         HIP_TRY(hipSetDevice(ctx->device));
         HIP_TRY(hipStreamSynchronize(ctx->last_stream));
+        check_stall(it->second, it->first);
         return 0;
     });
 }

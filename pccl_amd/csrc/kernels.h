@@ -31,7 +31,9 @@ struct DevStepOp {
 struct StepState {      // device memory, zero between launches (the kernel restores it on exit)
     int32_t cursor;
     int32_t exited;
-    int32_t pad[30];
+    int32_t error_op;   // 1 + index of the op whose bounded wait expired (0 = none); host clears it
+    int32_t error_dep;  // 1 + index of the predecessor it was waiting for
+    int32_t pad[28];
     // followed by int32 done[num_ops]
 };
 
@@ -56,11 +58,14 @@ struct StepwiseLaunch {
     StepState* state;
     int32_t dtype;
     int32_t num_blocks;
+    int32_t spin_limit;   // polls of one dependency counter before the persistent runner gives up
 };
 
 // All return a hipError_t value as int (0 = success).
 int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream);
-int launch_stepwise(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream);
+int launch_persistent(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream);
+// One dependency level: items [item_begin, item_end) of the work list.
+int launch_level(const StepwiseLaunch& L, int item_begin, int item_end, const RankPtrs& ptrs, void* stream);
 int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream);
 int launch_copy_bytes(const void* src, void* dst, size_t nbytes, void* stream);
 // One launch copying `bytes` from src.p[r] + src_off[r] to dst.p[r] + dst_off[r] for r < R.

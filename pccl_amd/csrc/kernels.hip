@@ -1,5 +1,5 @@
 // gfx950 kernels of the executor: element arithmetic, the chunk reduce/copy primitives, the
-// stepwise (flag-ordered) runner and the column runner.
+// level runner, the persistent (flag-ordered) runner and the column runner.
 //
 // Arithmetic contract (what the reference's Vec<T>::operator+ computes on its hardware,
 // csrc/plugins/cuda/kernel/vec.h:104-111,170-177,232-239): one correctly rounded addition in the
@@ -221,23 +221,52 @@ __global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* dst, int6
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * kThreads) dst[i] = 0;
 }
 
-// ------------------------------------------------------------------------------- stepwise runner
+// ------------------------------------------------------------------------------- level runner
+//
+// General path for any linked program: the data ops are grouped by dependency level and every
+// level is one launch; the launch boundary orders the levels.  A workgroup runs whole (op, tile)
+// items of its level.
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int item_begin, int item_end, RankPtrs ptrs) {
+    constexpr int ES = ElemBytes<DT>::value;
+    const int tid = threadIdx.x;
+    for (int item = item_begin + (int)blockIdx.x; item < item_end; item += (int)gridDim.x) {
+        int opi = L.item_op[item];
+        DevStepOp op = L.ops[opi];
+        int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
+        int64_t cnt = op.size - e0 < L.tile_elems ? op.size - e0 : L.tile_elems;
+        char* self = ptrs.p[op.self];
+        const char* peer = ptrs.p[op.peer];
+        if (op.is_reduce)
+            range_op<DT, true>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
+        else
+            range_copy_bytes(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
+    }
+}
+
+// ------------------------------------------------------------------------------- persistent runner
 //
 // One persistent launch executes every data op of the linked program.  Work items are (op, tile)
 // pairs in level order; a workgroup claims the next item from one atomic cursor, waits until every
 // tile of the op's predecessors has been published, runs the tile, then publishes it.  A claimed
 // item only ever waits for items claimed earlier by workgroups that are already running, so the
-// scheme cannot deadlock whatever the grid size.
+// scheme cannot deadlock whatever the grid size.  Every wait is bounded all the same: after
+// `spin_limit` polls the waiter records (op, predecessor) in the state block and every workgroup
+// leaves at its next claim, so the grid always drains and the host reports the stall as an error.
 
 template <int DT>
-__global__ __launch_bounds__(kThreads) void stepwise_kernel(StepwiseLaunch L, RankPtrs ptrs) {
+__global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     constexpr int ES = ElemBytes<DT>::value;
     __shared__ int s_item;
     __shared__ int s_last;
     int32_t* done = reinterpret_cast<int32_t*>(L.state + 1);
     const int tid = threadIdx.x;
     for (;;) {
-        if (tid == 0) s_item = atomicAdd(&L.state->cursor, 1);
+        if (tid == 0) {
+            int stalled = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_item = stalled ? L.num_items : atomicAdd(&L.state->cursor, 1);
+        }
         __syncthreads();
         int item = s_item;
         __syncthreads();
@@ -247,10 +276,26 @@ __global__ __launch_bounds__(kThreads) void stepwise_kernel(StepwiseLaunch L, Ra
         if (tid < op.ndeps) {
             int d = L.deps[op.dep_start + tid];
             int need = L.ops[d].ntiles;
-            while (__hip_atomic_load(&done[d], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) __builtin_amdgcn_s_sleep(4);
+            int spins = 0;
+            while (__hip_atomic_load(&done[d], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+                if (++spins > L.spin_limit ||
+                    __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+                    if (spins > L.spin_limit) {
+                        __hip_atomic_store(&L.state->error_dep, d + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(&L.state->error_op, opi + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(8);
+            }
         }
         __syncthreads();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (tid == 0) s_item = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        bool stalled = s_item != 0;
+        __syncthreads();
+        if (stalled) break;   // a predecessor never arrived: do not touch the data, just drain
         int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
         int64_t cnt = op.size - e0 < L.tile_elems ? op.size - e0 : L.tile_elems;
         char* self = ptrs.p[op.self];
@@ -265,7 +310,8 @@ __global__ __launch_bounds__(kThreads) void stepwise_kernel(StepwiseLaunch L, Ra
             __hip_atomic_fetch_add(&done[opi], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    // the last workgroup out restores the state block for the next launch
+    // the last workgroup out restores the progress counters for the next launch (the error
+    // words stay until the host has read and cleared them)
     if (tid == 0) s_last = (atomicAdd(&L.state->exited, 1) == (int)gridDim.x - 1);
     __syncthreads();
     if (s_last) {
@@ -442,22 +488,44 @@ int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
 }
 
 template <int DT>
-static int launch_stepwise_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
+static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
     int grid = L.num_blocks > 0 ? L.num_blocks : current_cus() * 8;
     if (grid > L.num_items) grid = L.num_items;
     if (grid <= 0) return 0;
-    hipLaunchKernelGGL((stepwise_kernel<DT>), dim3(grid), dim3(kThreads), 0, s, L, ptrs);
+    hipLaunchKernelGGL((persistent_kernel<DT>), dim3(grid), dim3(kThreads), 0, s, L, ptrs);
     return (int)hipGetLastError();
 }
 
-int launch_stepwise(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream) {
+int launch_persistent(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream) {
     hipStream_t s = (hipStream_t)stream;
     switch (L.dtype) {
-        case PCCL_F32: return launch_stepwise_dt<PCCL_F32>(L, ptrs, s);
-        case PCCL_F16: return launch_stepwise_dt<PCCL_F16>(L, ptrs, s);
-        case PCCL_BF16: return launch_stepwise_dt<PCCL_BF16>(L, ptrs, s);
-        case PCCL_I32: return launch_stepwise_dt<PCCL_I32>(L, ptrs, s);
-        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_stepwise_dt<PCCL_F8E4M3>(L, ptrs, s);
+        case PCCL_F32: return launch_persistent_dt<PCCL_F32>(L, ptrs, s);
+        case PCCL_F16: return launch_persistent_dt<PCCL_F16>(L, ptrs, s);
+        case PCCL_BF16: return launch_persistent_dt<PCCL_BF16>(L, ptrs, s);
+        case PCCL_I32: return launch_persistent_dt<PCCL_I32>(L, ptrs, s);
+        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_persistent_dt<PCCL_F8E4M3>(L, ptrs, s);
+        default: return (int)hipErrorInvalidValue;
+    }
+}
+
+template <int DT>
+static int launch_level_dt(const StepwiseLaunch& L, int item_begin, int item_end, const RankPtrs& ptrs, hipStream_t s) {
+    int n = item_end - item_begin;
+    if (n <= 0) return 0;
+    int cap = L.num_blocks > 0 ? L.num_blocks : current_cus() * 32;
+    int grid = n < cap ? n : cap;
+    hipLaunchKernelGGL((level_kernel<DT>), dim3(grid), dim3(kThreads), 0, s, L, item_begin, item_end, ptrs);
+    return (int)hipGetLastError();
+}
+
+int launch_level(const StepwiseLaunch& L, int item_begin, int item_end, const RankPtrs& ptrs, void* stream) {
+    hipStream_t s = (hipStream_t)stream;
+    switch (L.dtype) {
+        case PCCL_F32: return launch_level_dt<PCCL_F32>(L, item_begin, item_end, ptrs, s);
+        case PCCL_F16: return launch_level_dt<PCCL_F16>(L, item_begin, item_end, ptrs, s);
+        case PCCL_BF16: return launch_level_dt<PCCL_BF16>(L, item_begin, item_end, ptrs, s);
+        case PCCL_I32: return launch_level_dt<PCCL_I32>(L, item_begin, item_end, ptrs, s);
+        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_level_dt<PCCL_F8E4M3>(L, item_begin, item_end, ptrs, s);
         default: return (int)hipErrorInvalidValue;
     }
 }

@@ -1,7 +1,9 @@
 """GPU parity: the HIP executor against the CPU oracle, bit for bit, through the C ABI.
 
-Every case runs in both execution modes (column and stepwise) and, where stated, staged
-(separate input/output tensors, the reference's call shape) and in place.
+Every case runs in the three execution modes — column (position-decomposed, no inter-workgroup
+ordering), stepwise (one launch per dependency level) and persistent (one launch, device-side
+flags with bounded waits) — in place on the caller's buffers and staged (separate input/output
+tensors, the reference's call shape).
 """
 import pytest
 import torch
@@ -44,24 +46,32 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("mode", ["column", "stepwise"])
+PERSISTENT_OFF = pytest.mark.skip(reason="the persistent flag-ordered runner hung on MI355X (wait for a "
+                                   "predecessor's tile counter never returned); the mode is refused "
+                                   "by the library until the cause is found")
+MODES = ["column", "stepwise", pytest.param("persistent", marks=PERSISTENT_OFF)]
+
+
 @pytest.mark.parametrize("alg,world,n,dtype,channels,kind", CASES)
+@pytest.mark.parametrize("mode", MODES)
 def test_allreduce_matches_oracle(engine_factory, alg, world, n, dtype, channels, kind, mode):
+    print(f"case {alg} R={world} n={n} {dtype} ch={channels} mode={mode}", flush=True)
     jsons = graph_jsons(alg, "build_allreduce", world, n, dtype, "sm", channels)
     inputs = seeded_inputs(kind, world, n, dtype)
     expect = oracle_buffers(jsons, inputs, dtype)
     engine = engine_factory(world)
-    got, info = run_gpu(engine, jsons, inputs, mode)
+    print("  in place", flush=True)
+    got, info = run_gpu(engine, jsons, inputs, mode, inplace=True)
     assert info["residual_signals"] == 0
     for r in range(world):
-        assert bits_equal(got[r], expect[r]), f"rank {r}: {mismatch_report(got[r], expect[r])}"
-    # and in place on the caller's buffers
-    got2, _ = run_gpu(engine, jsons, inputs, mode, inplace=True)
+        assert bits_equal(got[r], expect[r]), f"in place, rank {r}: {mismatch_report(got[r], expect[r])}"
+    print("  staged", flush=True)
+    got2, _ = run_gpu(engine, jsons, inputs, mode)
     for r in range(world):
-        assert bits_equal(got2[r], expect[r]), f"in place, rank {r}: {mismatch_report(got2[r], expect[r])}"
+        assert bits_equal(got2[r], expect[r]), f"staged, rank {r}: {mismatch_report(got2[r], expect[r])}"
 
 
-@pytest.mark.parametrize("mode", ["column", "stepwise"])
+@pytest.mark.parametrize("mode", MODES)
 def test_closed_form_rank_plus_one(engine_factory, mode):
     """Input rank+1 everywhere -> allreduce = R(R+1)/2, exact in bf16
     (reference tests/test_correctness.py:142,170-171)."""
@@ -73,7 +83,7 @@ def test_closed_form_rank_plus_one(engine_factory, mode):
         assert torch.all(got[r].float() == world * (world + 1) / 2)
 
 
-@pytest.mark.parametrize("mode", ["column", "stepwise"])
+@pytest.mark.parametrize("mode", MODES)
 def test_reduce_scatter_and_allgather(engine_factory, mode):
     """reference tests/test_correctness.py:196-241: reduce_scatter output is one chunk of sums;
     allgather input is one chunk, output the concatenation."""
@@ -95,7 +105,7 @@ def test_reduce_scatter_and_allgather(engine_factory, mode):
         assert bits_equal(got[r], whole), f"rank {r}: {mismatch_report(got[r], whole)}"
 
 
-@pytest.mark.parametrize("mode", ["stepwise"])
+@pytest.mark.parametrize("mode", ["stepwise", pytest.param("persistent", marks=PERSISTENT_OFF)])
 def test_alltoall(engine_factory, mode):
     """reference tests/test_correctness.py:243-272: out[i] chunk = chunk r of rank i's input."""
     world, n = 4, 1 << 12
@@ -108,3 +118,12 @@ def test_alltoall(engine_factory, mode):
     for r in range(world):
         want = torch.cat([torch.full((chunk,), i * 100 + r, dtype=torch.bfloat16) for i in range(world)])
         assert bits_equal(got[r], want), mismatch_report(got[r], want)
+
+
+def test_persistent_mode_is_refused(engine_factory):
+    from pccl_amd._lib import PcclError, ERR_UNSUPPORTED
+    engine = engine_factory(2)
+    with pytest.raises(PcclError) as e:
+        engine.set_option("mode", "persistent")
+    assert e.value.code == ERR_UNSUPPORTED
+    engine.set_option("mode", "auto")
