@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Headline benchmark: the 8-virtual-rank, 512 MB-per-rank bf16 ring-allreduce graph on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode auto|column|stepwise]
+
+A step is one execution of the compiled graph (448 data ops over 8 rank buffers resident in HBM),
+in place on the rank buffers, one launch of the column runner.  Prints ONE JSON line.
+
+* value     algorithmic schedule bytes (reduce 3*n*esize, copy 2*n*esize, summed over the linked
+            program = 5*(R-1)*S) times K, divided by the wall time of the K timed steps
+* roofline  the same bytes divided by the average kernel duration measured with HIP events on the
+            launch stream (torch's current stream, which is the stream the C ABI launches on),
+            against the 8 TB/s HBM peak; `traffic` is the measured HBM bytes per launch from the
+            committed rocprofv3 counter summary when present
+* cpu_baseline  the CPU oracle (oracle/, OpenMP) executing the same graph shape on a bounded sample
+            on this box's host cores; a reported baseline, not the target
+
+Inputs: one CPU generator seeded 0; for rank r = 0..7, for slice s = 0..7, draw
+torch.randn(N/8) and cast to bf16 (rank-major, slice-major) — N(0,1) values as the configuration
+prescribes, generated in slices to bound host memory.  The first execution is verified at full size
+before anything is timed: all ranks must hold bit-identical results and those must equal the
+ring's per-element reduction order evaluated with plain torch bf16 adds.
+"""
+from __future__ import annotations
+
+import argparse
+import hashlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+R = 8
+N = 268_435_456          # bf16 elements per rank = 512 MiB
+CHANNELS = 4
+DTYPE = "bfloat16"
+PEAK_GBPS = 8000.0
+WORKLOAD = "ring_allreduce_sum_R8_bf16_512MiB_per_rank_4ch"
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def build_graphs(n: int, channels: int):
+    from pccl_amd.dsl import RingAllreduce, compile_to_json_string
+    return [compile_to_json_string(RingAllreduce().build_allreduce(r, R, n, dtype=DTYPE, executor="sm",
+                                                                   num_channels=channels))
+            for r in range(R)]
+
+
+def make_inputs(n: int, device):
+    import torch
+    g = torch.Generator().manual_seed(0)
+    slices = 8
+    per = n // slices
+    bufs = []
+    for r in range(R):
+        buf = torch.empty(n, dtype=torch.bfloat16, device=device)
+        for s in range(slices):
+            buf[s * per:(s + 1) * per] = torch.randn(per, generator=g).to(torch.bfloat16).to(device)
+        bufs.append(buf)
+    return bufs
+
+
+def ring_expected(inputs, n: int, channels: int):
+    """Ring order (chunk c of channel ch: acc = x_c; acc = x_(c+k) + acc, k = 1..R-1), each add
+    rounded to bf16, evaluated with torch's own bf16 add on the GPU."""
+    import torch
+    per_ch = n // channels
+    per_rank = per_ch // R
+    out = torch.empty_like(inputs[0])
+    for ch in range(channels):
+        for c in range(R):
+            lo = ch * per_ch + c * per_rank
+            acc = inputs[c][lo:lo + per_rank].clone()
+            for k in range(1, R):
+                acc = inputs[(c + k) % R][lo:lo + per_rank] + acc
+            out[lo:lo + per_rank] = acc
+    return out
+
+
+def sha256_of(t) -> str:
+    import torch
+    h = hashlib.sha256()
+    flat = t.view(torch.int16)
+    step = 1 << 26
+    for i in range(0, flat.numel(), step):
+        h.update(flat[i:i + step].cpu().numpy().tobytes())
+    return h.hexdigest()
+
+
+def cpu_baseline(sample_elems: int, channels: int, reps: int = 3):
+    """Time the CPU oracle on the same graph shape at `sample_elems` elements per rank."""
+    import numpy as np
+    from oracle import oracle
+    graphs = [oracle.Graph(json.loads(j)) for j in build_graphs(sample_elems, channels)]
+    rng = np.random.default_rng(0)
+    threads = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        threads = int(env)
+    # first touch by filling; bf16 bit patterns of N(0,1)-like magnitudes
+    bufs = [(rng.integers(0x3C00, 0x4000, sample_elems, dtype=np.uint16)) for _ in range(R)]
+    stats = oracle.run(graphs, bufs, threads=threads)      # warm-up
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        stats = oracle.run(graphs, bufs, threads=threads)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(stats.bytes / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"same ring graph (R={R}, {channels} channels, bf16) at {sample_elems} elements "
+                      f"per rank ({sample_elems * 2 >> 20} MiB), {stats.bytes} algorithmic bytes, median of "
+                      f"{reps} runs after 1 warm-up, {med * 1e3:.1f} ms"}
+
+
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel from the committed rocprofv3 counter summary."""
+    path = os.path.join(ROOT, "profiles", "column_kernel_ring_allreduce_R8_bf16_512MiB.traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--mode", default="auto")
+    ap.add_argument("--elems", type=int, default=N, help="elements per rank (default: the headline size)")
+    ap.add_argument("--channels", type=int, default=CHANNELS)
+    ap.add_argument("--vecs-per-thread", type=int, default=0)
+    ap.add_argument("--num-blocks", type=int, default=-1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--cpu-sample-elems", type=int, default=N)
+    ap.add_argument("--cpu-reps", type=int, default=20)
+    ap.add_argument("--calibrate-copy-bytes", type=int, default=0,
+                    help="also launch the library's plain copy kernel on this many bytes (3 times): a "
+                         "known-traffic reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU: the R ranks are virtual ranks resident in one "
+              "MI355X's HBM and no multi-GPU path exists; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the executor has no CPU fallback", file=sys.stderr)
+        return 1
+    from pccl_amd.engine import Engine
+
+    n, channels = args.elems, args.channels
+    dev = torch.device("cuda", 0)
+    eng = Engine(R, 0)
+    for r, text in enumerate(build_graphs(n, channels)):
+        eng.register_operation_json("bench", text, r)
+    eng.set_option("mode", args.mode)
+    if args.vecs_per_thread:
+        eng.set_option("vecs_per_thread", args.vecs_per_thread)
+    if args.num_blocks >= 0:
+        eng.set_option("num_blocks", args.num_blocks)
+    info = eng.op_info("bench")
+    alg_bytes = info["algorithmic_bytes"]
+    log(f"program: {info}")
+
+    t0 = time.perf_counter()
+    pristine = make_inputs(n, dev)
+    log(f"inputs generated in {time.perf_counter() - t0:.1f} s")
+    bufs = [p.clone() for p in pristine]
+
+    verify = {}
+    if not args.no_verify:
+        eng.execute_inplace("bench", bufs, sync=True)
+        same = all(torch.equal(bufs[0].view(torch.int16), b.view(torch.int16)) for b in bufs[1:])
+        want = ring_expected(pristine, n, channels)
+        exact = torch.equal(want.view(torch.int16), bufs[0].view(torch.int16))
+        ref32 = sum(p[:1 << 20].float() for p in pristine)
+        rel = ((bufs[0][:1 << 20].float() - ref32).abs() / ref32.abs().clamp_min(1.0)).max().item()
+        verify = {"ranks_identical": bool(same), "matches_ring_order_bf16": bool(exact),
+                  "max_rel_err_vs_fp32_sum_first_1Mi": round(rel, 5), "output_sha256": sha256_of(bufs[0])}
+        log(f"verify: {verify}")
+        del want
+        if not (same and exact):
+            print(json.dumps({"error": "verification failed", **verify}))
+            return 1
+        for b, p in zip(bufs, pristine):
+            b.copy_(p)
+
+    if args.calibrate_copy_bytes:
+        from pccl_amd import _lib
+        src = torch.empty(args.calibrate_copy_bytes, dtype=torch.uint8, device=dev).random_(0, 256)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(_lib.lib().pccl_hip_copy(3, src.data_ptr(), dst.data_ptr(), src.numel(), None))
+        torch.cuda.synchronize()
+        del src, dst
+
+    for _ in range(args.warmup):
+        eng.execute_inplace("bench", bufs)
+    torch.cuda.synchronize()
+    ev0 = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ev1 = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ev0[i].record()
+        eng.execute_inplace("bench", bufs)
+        ev1[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = [a.elapsed_time(b) for a, b in zip(ev0, ev1)]
+    avg_ms = sum(kern_ms) / len(kern_ms)
+    ms_per_step = wall * 1e3 / args.steps
+    value = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = alg_bytes / (avg_ms * 1e-3) / 1e9
+
+    # end to end the reference's way: input and output staging copies included
+    outs = [torch.empty_like(p) for p in pristine]
+    eng.execute_operation("bench", pristine, outs)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    reps = max(3, args.steps // 4)
+    for _ in range(reps):
+        eng.execute_operation_async("bench", pristine, outs)
+    e1.record()
+    torch.cuda.synchronize()
+    staged_ms = e0.elapsed_time(e1) / reps
+    del outs
+
+    traffic = measured_traffic() if (n == N and channels == CHANNELS) else None
+    result = {
+        "metric": "HBM GB/s (algorithmic schedule bytes read+written per second), 8-vrank 512MB bf16 ring allreduce graph",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": WORKLOAD if (n == N and channels == CHANNELS) else
+                   f"ring_allreduce_sum_R8_bf16_{n}elems_per_rank_{channels}ch",
+                   "virtual_ranks": R, "bytes_per_rank": n * 2, "channels": channels, "data_ops": info["num_data_ops"],
+                   "algorithmic_bytes_per_step": alg_bytes, "mode": args.mode, "in_place": True},
+        "pct_of_hbm_peak": round(100 * value / PEAK_GBPS, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_GBPS, 4), "traffic": traffic,
+                     "kernel_ms_avg": round(avg_ms, 4), "kernel_ms_min": round(min(kern_ms), 4),
+                     "planned_load_bytes": info["column_load_bytes"], "planned_store_bytes": info["column_store_bytes"]},
+        "end_to_end_staged": {"ms_per_call": round(staged_ms, 4), "GB/s": round(alg_bytes / (staged_ms * 1e-3) / 1e9, 1),
+                              "note": "input and output staging copies included, the reference's own timing method"},
+        "verify": verify,
+    }
+    if traffic:
+        result["roofline"]["hbm_frac"] = round(traffic / (avg_ms * 1e-3) / 1e9 / PEAK_GBPS, 4)
+    if not args.no_cpu_baseline:
+        del bufs, pristine
+        torch.cuda.empty_cache()
+        result["cpu_baseline"] = cpu_baseline(min(args.cpu_sample_elems, n), channels, args.cpu_reps)
+    print(json.dumps(result))
+    eng.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -90,6 +90,11 @@ def lib() -> ctypes.CDLL:
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `python -m pccl_amd.build` (hipcc, gfx950). "
             "The executor has no CPU or PyTorch fallback.")
+    # PyTorch-ROCm ships its own HIP runtime (libamdhip64.so.7).  It must be in the process before
+    # this library is, so that the dynamic loader binds this library to that same runtime; loaded
+    # the other way round the process ends up with two HIP runtimes and neither sees the other's
+    # device state.
+    import torch  # noqa: F401
     L = ctypes.CDLL(LIB_PATH)
     vp, cp, i32, i64, sz = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
     P = ctypes.POINTER
