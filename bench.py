@@ -141,6 +141,8 @@ def main() -> int:
     ap.add_argument("--num-blocks", type=int, default=-1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--gpu-inputs", action="store_true",
+                    help="draw the inputs with the GPU generator (tuning sweeps only; not the prescribed inputs)")
     ap.add_argument("--cpu-sample-elems", type=int, default=N)
     ap.add_argument("--cpu-reps", type=int, default=20)
     ap.add_argument("--calibrate-copy-bytes", type=int, default=0,
@@ -173,7 +175,11 @@ def main() -> int:
     log(f"program: {info}")
 
     t0 = time.perf_counter()
-    pristine = make_inputs(n, dev)
+    if args.gpu_inputs:
+        torch.manual_seed(0)
+        pristine = [torch.randn(n, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(R)]
+    else:
+        pristine = make_inputs(n, dev)
     log(f"inputs generated in {time.perf_counter() - t0:.1f} s")
     bufs = [p.clone() for p in pristine]
 
@@ -256,6 +262,8 @@ def main() -> int:
                               "note": "input and output staging copies included, the reference's own timing method"},
         "verify": verify,
     }
+    if args.gpu_inputs:
+        result["data"] = "synthetic (GPU generator: tuning run)"
     if traffic:
         result["roofline"]["hbm_frac"] = round(traffic / (avg_ms * 1e-3) / 1e9 / PEAK_GBPS, 4)
     if not args.no_cpu_baseline:
