@@ -199,15 +199,15 @@ struct OpEntry {
     std::vector<std::unique_ptr<RankGraph>> graphs;
     bool linked = false;
     Program prog;
-    DevBuf segs, instrs, fifo, step_ops, step_deps, item_op, state;
-    int64_t total_tiles = 0;
+    DevBuf segs, direct_segs, instrs, fifo, step_ops, step_deps, item_op, state;
+    int64_t total_tiles = 0, direct_tiles = 0;
     int vecs_per_thread = 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool timed = false;
     bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
     std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
     void release() {
-        segs.release(); instrs.release(); fifo.release(); step_ops.release(); step_deps.release();
+        segs.release(); direct_segs.release(); instrs.release(); fifo.release(); step_ops.release(); step_deps.release();
         item_op.release(); state.release();
         if (ev0) (void)hipEventDestroy(ev0);
         if (ev1) (void)hipEventDestroy(ev1);
@@ -234,6 +234,7 @@ struct pccl_hip_ctx {
     bool timing = false;
     int fifo_depth = 0;
     int64_t step_tile_bytes = 128 * 1024;
+    bool fuse_staging = true;             // run staged calls on the caller's tensors when possible
     int spin_limit = 1 << 22;             // polls (~0.1 us sleep each) before a persistent wait gives up
     hipStream_t last_stream = nullptr;
 };
@@ -269,24 +270,37 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
     const int ve = 16 / es;
     e.vecs_per_thread = ctx->vecs_per_thread;
 
-    // column plan
+    // column plans (in place, and direct = staging fused into the program)
     if (P.position_aligned) {
-        std::vector<DevColSegment> ds(P.segs.size());
-        int64_t tiles = 0;
         const int64_t tile_v = 256 * (int64_t)e.vecs_per_thread;
-        for (size_t i = 0; i < P.segs.size(); ++i) {
-            const ColSegment& s = P.segs[i];
-            DevColSegment& d = ds[i];
-            d.start = s.start; d.end = s.end;
-            d.first_vec = s.start / ve;
-            int64_t last_vec = (s.end - 1) / ve;
-            d.first_tile = tiles;
-            tiles += (last_vec - d.first_vec + 1 + tile_v - 1) / tile_v;
-            d.prog_start = s.prog_start; d.prog_len = s.prog_len;
-            d.fifo_start = s.fifo_start; d.fifo_len = s.fifo_len;
-        }
-        e.total_tiles = tiles;
+        auto device_segments = [&](const std::vector<ColSegment>& segs, int64_t* total) {
+            std::vector<DevColSegment> ds(segs.size());
+            int64_t tiles = 0;
+            for (size_t i = 0; i < segs.size(); ++i) {
+                const ColSegment& s = segs[i];
+                DevColSegment& d = ds[i];
+                d.start = s.start; d.end = s.end;
+                d.first_vec = s.start / ve;
+                int64_t last_vec = (s.end - 1) / ve;
+                d.first_tile = tiles;
+                tiles += (last_vec - d.first_vec + 1 + tile_v - 1) / tile_v;
+                d.prog_start = s.prog_start; d.prog_len = s.prog_len;
+                d.fifo_start = s.fifo_start; d.fifo_len = s.fifo_len;
+                d.streaming = 1; d.pad_ = 0;
+                for (int k = 0; k < s.prog_len; ++k) {
+                    const ColInstr& in = P.col_instrs[s.prog_start + k];
+                    if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || in.store == 1) d.streaming = 0;
+                }
+            }
+            *total = tiles;
+            return ds;
+        };
+        auto ds = device_segments(P.segs, &e.total_tiles);
         e.segs.upload(ds.data(), ds.size() * sizeof(DevColSegment));
+        if (!P.direct_segs.empty()) {
+            auto dd = device_segments(P.direct_segs, &e.direct_tiles);
+            e.direct_segs.upload(dd.data(), dd.size() * sizeof(DevColSegment));
+        }
         e.instrs.upload(P.col_instrs.data(), P.col_instrs.size() * sizeof(ColInstr));
         e.fifo.upload(P.col_fifo.data(), P.col_fifo.size());
     }
@@ -372,6 +386,43 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
     }
     if (rc != 0) throw Error{PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)};
     if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, stream)); e.timed = true; }
+}
+
+// Staged semantics without staging copies: first-touch loads read the caller's inputs, every store
+// goes to the caller's outputs.  Returns false when the call does not qualify (the caller then
+// stages through the engine's rank buffers).
+bool run_direct(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* const* outputs,
+                size_t in_bytes, size_t out_bytes, hipStream_t stream) {
+    const Program& P = e.prog;
+    if (!ctx->fuse_staging || ctx->mode == Mode::Stepwise || ctx->mode == Mode::Persistent) return false;
+    if (!P.position_aligned || P.direct_segs.empty() || !e.direct_segs.p) return false;
+    if (!(P.collective_type.empty() || P.collective_type == "allreduce")) return false;
+    const size_t es = elem_size(P.dtype);
+    if (in_bytes != out_bytes || in_bytes != (size_t)P.tensor_elems * es) return false;
+    RankPtrs ptrs;
+    std::memset(&ptrs, 0, sizeof(ptrs));
+    for (int r = 0; r < ctx->R; ++r) {
+        uintptr_t in = (uintptr_t)inputs[r], out = (uintptr_t)outputs[r];
+        if ((in | out) & 15) return false;
+        if (in != out && in < out + out_bytes && out < in + in_bytes) return false;  // partial overlap
+        for (int q = 0; q < r; ++q) {  // an output must not alias another rank's tensors
+            uintptr_t oq = (uintptr_t)outputs[q], iq = (uintptr_t)inputs[q];
+            if ((out < oq + out_bytes && oq < out + out_bytes) || (out < iq + in_bytes && iq < out + out_bytes) ||
+                (oq < in + in_bytes && in < oq + out_bytes)) return false;
+        }
+        ptrs.p[r] = (char*)outputs[r];
+        ptrs.p[PCCL_HIP_MAX_VRANKS + r] = (char*)inputs[r];
+    }
+    if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
+    ColumnLaunch L{};
+    L.segs = (const DevColSegment*)e.direct_segs.p; L.num_segs = (int)P.direct_segs.size();
+    L.instrs = (const uint64_t*)e.instrs.p; L.fifo = (const uint8_t*)e.fifo.p;
+    L.total_tiles = e.direct_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
+    L.num_blocks = ctx->num_blocks;
+    int rc = launch_column(L, ptrs, stream);
+    if (rc != 0) throw Error{PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)};
+    if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, stream)); e.timed = true; }
+    return true;
 }
 
 // After the stream has drained: did a bounded wait of the persistent runner expire?
@@ -478,6 +529,7 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             else return fail(PCCL_ERR_INVALID, "mode must be auto, column, stepwise or persistent");
         } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
         else if (k == "timing") ctx->timing = std::atoi(value) != 0;
+        else if (k == "fuse_staging") ctx->fuse_staging = std::atoi(value) != 0;
         else if (k == "spin_limit") { ctx->spin_limit = std::atoi(value); if (ctx->spin_limit < 1) ctx->spin_limit = 1; }
         else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
         else if (k == "vecs_per_thread") {
@@ -514,6 +566,12 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
         hipStream_t s = (hipStream_t)stream;
         for (int r = 0; r < R; ++r)
             if (!inputs[r] || !outputs[r]) return fail(PCCL_ERR_INVALID, "null tensor for virtual rank " + std::to_string(r));
+
+        if (run_direct(ctx, e, inputs, outputs, in_bytes, out_bytes, s)) {
+            ctx->last_stream = s;
+            if (sync) HIP_TRY(hipStreamSynchronize(s));
+            return 0;
+        }
 
         // layout of the staged data inside a rank buffer (reference engine_c.cc:468-548)
         size_t need = (size_t)P.buffer_elems * es;

@@ -20,6 +20,8 @@ struct DevColSegment {
     int64_t first_tile;      // prefix sum of tiles
     int32_t prog_start, prog_len;
     int32_t fifo_start, fifo_len;
+    int32_t streaming;       // 1: every load is a first touch and every live store is final
+    int32_t pad_;
 };
 
 struct DevStepOp {

@@ -331,6 +331,15 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                     if (prog[m].self == prog[n].self) { prog[n].store = 0; break; }
                 }
             }
+            // a store nothing in this program reads back from memory is final: mark it streaming
+            for (size_t n = 0; n < prog.size(); ++n) {
+                if (!prog[n].store) continue;
+                bool reread = false;
+                for (size_t m = n + 1; m < prog.size() && !reread; ++m)
+                    reread = (prog[m].a_src != SRC_ACC && prog[m].peer == prog[n].self) ||
+                             (prog[m].b_src == SRC_MEM && prog[m].self == prog[n].self);
+                if (!reread) prog[n].store = 2;
+            }
             // first-touch loads may be issued early through the FIFO (nothing before them writes
             // the location, so any earlier issue point reads the same value)
             if (opt.fifo_depth > 0)
@@ -350,6 +359,59 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                 if (in.a_src == SRC_MEM || in.a_src == SRC_FIFO) P.column_load_bytes += n * es;
                 if (in.b_src == SRC_MEM || in.b_src == SRC_FIFO) P.column_load_bytes += n * es;
                 if (in.store) P.column_store_bytes += n * es;
+            }
+        }
+
+        // ---- direct plan: the same programs with the caller's input tensors as the source of
+        // every first-touch load and the output tensors as the destination of every store, so
+        // that no staging copy is needed.  For the output to equal "input copied in, program
+        // run, buffer copied out", a (rank, position) the program never writes must be passed
+        // through from input to output: one copy instruction (peer = self, first touch) per
+        // unwritten rank of a segment, and whole pass-through segments over the uncovered gaps.
+        if (P.tensor_elems >= P.buffer_elems && P.tensor_elems > 0) {
+            auto passthrough = [&](uint64_t written) {
+                for (int r = 0; r < R; ++r)
+                    if (!(written >> r & 1)) {
+                        ColInstr in{};
+                        in.self = in.peer = (uint8_t)r; in.a_src = SRC_MEM; in.b_src = SRC_NONE;
+                        in.a_first = 1; in.store = 2;
+                        P.col_instrs.push_back(in);
+                    }
+            };
+            auto gap_segment = [&](int64_t a, int64_t b) {
+                if (a >= b) return;
+                ColSegment g;
+                g.start = a; g.end = b; g.prog_start = (int)P.col_instrs.size();
+                passthrough(0);
+                g.prog_len = (int)P.col_instrs.size() - g.prog_start;
+                P.direct_segs.push_back(g);
+            };
+            int64_t cursor = 0;
+            const std::vector<ColSegment> base_segs = P.segs;
+            for (const ColSegment& seg : base_segs) {
+                gap_segment(cursor, seg.start);
+                ColSegment d = seg;
+                d.prog_start = (int)P.col_instrs.size();
+                uint64_t written = 0;
+                for (int k = 0; k < seg.prog_len; ++k) {
+                    ColInstr in = P.col_instrs[seg.prog_start + k];
+                    written |= 1ull << in.self;
+                    P.col_instrs.push_back(in);
+                }
+                passthrough(written);
+                d.prog_len = (int)P.col_instrs.size() - d.prog_start;
+                P.direct_segs.push_back(d);
+                cursor = seg.end;
+            }
+            gap_segment(cursor, P.tensor_elems);
+            for (auto& seg : P.direct_segs) {
+                int64_t n = seg.end - seg.start;
+                for (int k = 0; k < seg.prog_len; ++k) {
+                    const ColInstr& in = P.col_instrs[seg.prog_start + k];
+                    if (in.a_src == SRC_MEM || in.a_src == SRC_FIFO) P.direct_load_bytes += n * es;
+                    if (in.b_src == SRC_MEM || in.b_src == SRC_FIFO) P.direct_load_bytes += n * es;
+                    if (in.store) P.direct_store_bytes += n * es;
+                }
             }
         }
     }

@@ -34,7 +34,8 @@ struct ColInstr {
     uint8_t a_src;   // SRC_MEM | SRC_ACC | SRC_FIFO
     uint8_t b_src;   // SRC_NONE (copy) | SRC_MEM | SRC_ACC | SRC_FIFO
     uint8_t redop;
-    uint8_t store;   // 0: the write is dead (overwritten before anything reads it from memory)
+    uint8_t store;   // 0: the write is dead (overwritten before anything reads it from memory),
+                     // 1: written and read back later by this program, 2: final value (streaming store)
     uint8_t a_first; // 1: this load is the first access to (peer, position) in the program
     uint8_t b_first;
 };
@@ -69,6 +70,9 @@ struct Program {
     std::vector<ColInstr> col_instrs;
     std::vector<uint8_t> col_fifo;
     int64_t column_load_bytes = 0, column_store_bytes = 0;
+    // direct plan (staging fused into the program; valid when non-empty): covers [0, tensor_elems)
+    std::vector<ColSegment> direct_segs;
+    int64_t direct_load_bytes = 0, direct_store_bytes = 0;
 
     // stepwise plan
     int64_t tile_elems = 0;

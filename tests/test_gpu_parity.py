@@ -127,3 +127,95 @@ def test_persistent_mode_is_refused(engine_factory):
         engine.set_option("mode", "persistent")
     assert e.value.code == ERR_UNSUPPORTED
     engine.set_option("mode", "auto")
+
+
+# ---------------------------------------------------------------------------------------------
+# Staged calls: fused into the program (default) and through the engine's rank buffers.
+
+def _ring_partial(kind, rank, world, n):
+    """The reference's reduce-only / copy-only ring graphs (tests/test_correctness.py:46-90):
+    no collective_type, so the engine stages them like an allreduce."""
+    from pccl_amd.dsl import CommunicationOp, compile_to_json_string
+    chunk = n // world
+    prev, nxt = (rank - 1) % world, (rank + 1) % world
+    with CommunicationOp(name=f"test_{kind}_rank{rank}") as op:
+        op.tensor(dtype="bfloat16", shape=(n,))
+        op.notify(signal_id=100, target_rank=nxt)
+        op.wait_notify(signal_id=100, source_rank=prev)
+        for step in range(world - 1):
+            c = (rank - step - 1) % world if kind == "reduce" else (rank - step) % world
+            if step > 0:
+                op.wait_notify(signal_id=0, source_rank=prev)
+            if kind == "reduce":
+                op.tma_reduce(reduce_op="sum", source_rank=prev, src_offset=c * chunk, dst_offset=c * chunk,
+                              remote_offset=c * chunk, count=chunk)
+            else:
+                op.tma_copy(source_rank=prev, src_offset=c * chunk, dst_offset=c * chunk, size=chunk)
+            op.notify(signal_id=0, target_rank=nxt)
+        op.wait_notify(signal_id=0, source_rank=prev)
+    return compile_to_json_string(op.get_graph())
+
+
+@pytest.mark.parametrize("fuse", [1, 0])
+@pytest.mark.parametrize("kind", ["reduce", "copy"])
+def test_partial_ring_graphs_pass_untouched_chunks_through(engine_factory, kind, fuse):
+    """Chunks a graph never writes must come out as they went in, whichever way the call is staged
+    (closed forms of reference tests/test_correctness.py:150-161,180-189)."""
+    world, n = 4, 1 << 14
+    jsons = [_ring_partial(kind, r, world, n) for r in range(world)]
+    inputs = seeded_inputs("randn", world, n, "bfloat16", seed=3)
+    expect = oracle_buffers(jsons, inputs, "bfloat16")
+    engine = engine_factory(world)
+    engine.set_option("fuse_staging", fuse)
+    try:
+        got, info = run_gpu(engine, jsons, inputs, "column")
+    finally:
+        engine.set_option("fuse_staging", 1)
+    for r in range(world):
+        assert bits_equal(got[r], expect[r]), f"rank {r}: {mismatch_report(got[r], expect[r])}"
+
+
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_staged_call_with_output_aliasing_input(engine_factory, fuse):
+    world, n = 8, 1 << 15
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 2)
+    inputs = seeded_inputs("randn", world, n, "float32", seed=5)
+    expect = oracle_buffers(jsons, inputs, "float32")
+    engine = engine_factory(world)
+    engine.set_option("fuse_staging", fuse)
+    engine.set_option("mode", "auto")
+    try:
+        for r, j in enumerate(jsons):
+            engine.register_operation_json("alias", j, r)
+        dev = [x.cuda() for x in inputs]
+        outs = engine.execute_operation("alias", dev, dev)
+    finally:
+        engine.set_option("fuse_staging", 1)
+    for r in range(world):
+        assert bits_equal(outs[r], expect[r]), mismatch_report(outs[r], expect[r])
+
+
+def test_fused_staging_covers_positions_outside_every_op(engine_factory):
+    """A graph that touches only the middle of the tensor: head and tail are passed through."""
+    from pccl_amd.dsl import CommunicationOp, compile_to_json_string
+    world, n = 2, 4099
+    jsons = []
+    for rank in range(world):
+        other = 1 - rank
+        with CommunicationOp(name=f"mid{rank}") as op:
+            op.tensor(dtype="float32", shape=(n,))
+            op.notify(signal_id=rank, target_rank=other)
+            op.wait_notify(signal_id=other, source_rank=other)
+            if rank == 0:
+                op.sm_reduce(source_rank=1, src_offset=1001, dst_offset=1001, remote_offset=1001, count=2003)
+            op.notify(signal_id=10 + rank, target_rank=other)
+            op.wait_notify(signal_id=10 + other, source_rank=other)
+        g = op.get_graph()
+        g.collective_type = "allreduce"
+        jsons.append(compile_to_json_string(g))
+    inputs = seeded_inputs("randn", world, n, "float32", seed=9)
+    expect = oracle_buffers(jsons, inputs, "float32")
+    got, info = run_gpu(engine_factory(world), jsons, inputs, "column")
+    assert info["num_segments"] == 1
+    for r in range(world):
+        assert bits_equal(got[r], expect[r]), mismatch_report(got[r], expect[r])
