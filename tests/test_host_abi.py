@@ -1,0 +1,277 @@
+"""Host-side behaviour of the C ABI (no GPU): the library loads and exports what the header
+declares, graphs load with the reference's field mapping and error behaviour, fused steps group
+like the reference's descriptor builder, and the cross-rank linker finds deadlocks and races.
+"""
+import ctypes
+import json
+import os
+import re
+
+import pytest
+
+from helpers import ROOT, graph_jsons, oracle
+from pccl_amd import _lib
+from pccl_amd._lib import (ERR_INVALID, ERR_LINK, ERR_NOT_FOUND, ERR_PARSE, ERR_UNSUPPORTED, HostGraph,
+                           HostProgram, PcclError)
+from pccl_amd.dsl import CommunicationOp, compile_to_json_string
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "pccl_hip.h")).read()
+    declared = set(re.findall(r"\b(pccl_(?:hip|graph|program)_\w+)\s*\(", header))
+    assert len(declared) >= 30
+    L = _lib.lib()
+    missing = [n for n in sorted(declared) if not hasattr(L, n)]
+    assert not missing, missing
+    assert declared == set(_lib.EXPORTS)
+    assert b"gfx950" in L.pccl_hip_version()
+
+
+def test_struct_layouts_match_the_reference():
+    """sizes / offsets of the reference structs (proxy_trigger.h:8-16, primitive.h:8-17, fused_step.h:7-22)."""
+    assert ctypes.sizeof(_lib.Trigger) == 32
+    assert [getattr(_lib.Trigger, f).offset for f in ("primitive_type", "op_index", "peer_rank", "offset_0",
+                                                      "offset_1", "offset_2", "size")] == [0, 4, 8, 12, 16, 20, 24]
+    assert ctypes.sizeof(_lib.PrimitiveMeta) == 88
+    assert ctypes.sizeof(_lib.FusedStep) == 44
+
+
+def test_no_device_means_error_not_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    h = ctypes.c_void_p()
+    rc = _lib.lib().pccl_hip_create(ctypes.byref(h), 0, 8)
+    assert rc == _lib.ERR_HIP
+    assert b"no CPU fallback" in _lib.lib().pccl_hip_last_error()
+    from pccl_amd.engine import Engine
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        Engine(8, 0)
+
+
+# ------------------------------------------------------------------------------- graph loading
+
+def test_trigger_fields_agree_with_an_independent_parse():
+    """The product's C++ loader against the oracle's Python loader (both follow sm_channel.h /
+    tma_channel.h) on every golden graph."""
+    idx = json.load(open(os.path.join(ROOT, "tests/golden/graphs/index.json")))
+    kinds = {1: "reduce", 2: "copy", 3: "notify", 4: "wait"}
+    for case in idx:
+        for rank in range(case["world_size"]):
+            path = os.path.join(ROOT, "tests/golden/graphs", f"{case['stem']}_rank{rank}.json")
+            g = HostGraph.from_file(path)
+            o = oracle.Graph.from_file(path)
+            trig, n = g.triggers()
+            meta, _ = g.meta()
+            assert n == o.n and g.collective_type == o.collective_type
+            assert g.dtype == o.dtype and g.tensor_elems == case["tensor_size"]
+            for i in range(n):
+                t, m, q = trig[i], meta[i], o.table[i]
+                assert (t.op_index, t.peer_rank, m.channel, m.num_dependencies, m.num_next_ops) == \
+                       (q.index, q.peer, q.channel, q.ndeps, q.nnext)
+                pt = t.primitive_type
+                if kinds[q.kind] == "reduce":
+                    assert pt in (1 + o.dtype, 33 + o.dtype)
+                    assert (t.offset_0, t.offset_1, t.offset_2, t.size) == (q.off0, q.off1, q.off2, q.size)
+                elif kinds[q.kind] == "copy":
+                    assert pt in (6 + o.dtype, 28 + o.dtype)
+                    assert (t.offset_0, t.offset_1, t.size) == (q.off0, q.off1, q.size)
+                else:
+                    assert pt == (22 if kinds[q.kind] == "notify" else 21) and t.offset_0 == q.off0
+                assert list(m.next_primitive_index)[:m.num_next_ops] == list(q.next)[:q.nnext]
+
+
+def test_primitive_ids_distinguish_sm_and_tma():
+    sm = HostGraph.from_json(graph_jsons("ring", "build_allreduce", 2, 2048, "bfloat16", "sm")[0]).triggers()[0]
+    tma = HostGraph.from_json(graph_jsons("ring", "build_allreduce", 2, 2048, "bfloat16", "tma")[0]).triggers()[0]
+    assert sm[2].primitive_type == 3 and sm[5].primitive_type == 8        # cuda_reduce_bf16, cuda_copy_bf16
+    assert tma[2].primitive_type == 35 and tma[5].primitive_type == 30    # cuda_tma_reduce_bf16, cuda_tma_copy_bf16
+
+
+def _doc(**over):
+    doc = json.loads(graph_jsons("ring", "build_allreduce", 2, 2048, "float32", "sm")[0])
+    doc.update(over)
+    return doc
+
+
+def _load_err(doc_or_text):
+    text = doc_or_text if isinstance(doc_or_text, str) else json.dumps(doc_or_text)
+    with pytest.raises(PcclError) as e:
+        HostGraph.from_json(text)
+    return e.value
+
+
+def test_load_errors():
+    with pytest.raises(PcclError) as e:
+        HostGraph.from_file("/nonexistent/graph.json")
+    assert e.value.code == ERR_NOT_FOUND                       # reference: regOp returns false
+    d = _doc(); del d["operations"]
+    assert _load_err(d).code == ERR_PARSE                       # reference: returns false
+    d = _doc(); del d["operations"][3]["primitive"]
+    assert "index/executor/primitive" in str(_load_err(d))
+    d = _doc(); d["operations"][2]["primitive"] = "sm.scatter"
+    assert "unknown primitive" in str(_load_err(d))             # reference: throws
+    d = _doc(); d["tensor_info"]["dtype"] = "float64"
+    assert "Unsupported dtype" in str(_load_err(d))             # reference: throws (sm_channel.h:71)
+    d = _doc(); d["tensor_info"]["dtype"] = "float8_e4m3"
+    assert _load_err(d).code == ERR_UNSUPPORTED                 # fp8 reduce is not implemented here
+    d = _doc(); d["operations"][2]["executor"] = "cuda_ce"
+    assert _load_err(d).code == ERR_UNSUPPORTED
+    d = _doc(); d["operations"][2]["params"]["reduce_op"] = "avg"
+    assert _load_err(d).code == ERR_UNSUPPORTED
+    d = _doc(); del d["operations"][2]["params"]["count"]
+    assert "params.count" in str(_load_err(d))
+    d = _doc(); d["operations"][0]["params"]["signal_id"] = 4096
+    assert "signal_id" in str(_load_err(d))
+    d = _doc(); d["operations"][1]["dependencies"] = [99]
+    assert "unknown operation index" in str(_load_err(d))
+    assert _load_err("{not json").code == ERR_PARSE
+    assert _load_err('{"operations": [1, 2').code == ERR_PARSE
+
+
+def test_int32_and_max_are_accepted_as_extensions():
+    g = HostGraph.from_json(graph_jsons("tree", "build_allreduce", 4, 1024, "int32", "sm", reduce_op="max")[0])
+    trig, n = g.triggers()
+    red = [trig[i] for i in range(n) if trig[i].primitive_type == 64]
+    assert red and all(t.redop == 1 for t in red)
+    assert g.dtype == 5
+
+
+def test_graph_from_triggers_round_trip():
+    text = graph_jsons("ring", "build_allreduce", 4, 4096, "float16", "tma", 2)[1]
+    g = HostGraph.from_json(text)
+    trig, n = g.triggers()
+    meta, _ = g.meta()
+    g2 = HostGraph.from_triggers(trig, meta, g.collective_type)
+    t2, n2 = g2.triggers()
+    assert n2 == n and g2.dtype == g.dtype and g2.collective_type == "allreduce"
+    for i in range(n):
+        assert bytes(trig[i])[:28] == bytes(t2[i])[:28]
+
+
+# ------------------------------------------------------------------------------- fused steps
+
+def test_fused_steps_two_rank_ring():
+    """The worked example: notify/wait/data grouping of reference graph_builder.cc:236-311."""
+    g = HostGraph.from_file(os.path.join(ROOT, "tests/golden/graphs/ring_ar_sm_w2_n2048_bf16_c1_rank0.json"))
+    steps, offs = g.fused_steps()
+    assert offs == [0, 3]
+    s0, s1, s2 = steps
+    assert (s0.has_notify, s0.notify_peer_rank, s0.notify_signal_id, s0.has_wait, s0.wait_signal_id) == (1, 1, 100, 1, 100)
+    assert (s0.primitive_type, s0.peer_rank, s0.offset_0, s0.offset_1, s0.offset_2, s0.size) == (3, 1, 1024, 1024, 1024, 1024)
+    assert (s1.has_notify, s1.notify_signal_id, s1.has_wait, s1.primitive_type, s1.offset_0, s1.size) == (1, 0, 1, 8, 0, 1024)
+    assert (s2.has_notify, s2.has_wait, s2.primitive_type) == (1, 1, 0)
+
+
+def test_fused_steps_counts():
+    g = HostGraph.from_json(graph_jsons("ring", "build_allreduce", 8, 8192 * 4, "bfloat16", "sm", 4)[0])
+    steps, offs = g.fused_steps()
+    assert offs == [0, 15, 30, 45, 60]                       # 7 reduce + 7 copy + 1 signal-only per channel
+    assert sum(1 for s in steps if 1 <= s.primitive_type <= 5) == 28
+    g = HostGraph.from_json(graph_jsons("rhd", "build_allreduce", 16, 4096, "float32", "sm")[3])
+    assert len(g.fused_steps()[0]) == 9
+
+
+def test_fused_steps_fall_back_like_the_reference():
+    # alltoall: a data op directly follows a data op -> not a fused chain
+    g = HostGraph.from_json(graph_jsons("ring", "build_alltoall", 4, 4096, "bfloat16")[0])
+    with pytest.raises(PcclError) as e:
+        g.fused_steps()
+    assert e.value.code == ERR_UNSUPPORTED
+    # ring with 32 ranks and 4 channels needs 252 > 128 steps
+    g = HostGraph.from_json(graph_jsons("ring", "build_allreduce", 32, 4096 * 32, "bfloat16", "sm", 4)[0])
+    with pytest.raises(PcclError):
+        g.fused_steps()
+
+
+# ------------------------------------------------------------------------------- linker
+
+def _link(jsons):
+    return HostProgram([HostGraph.from_json(j) for j in jsons])
+
+
+def test_program_info_closed_forms():
+    world, n = 8, 8192 * 4
+    info = _link(graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 4)).info()
+    S = n * 2
+    assert info["num_data_ops"] == 448 and info["num_ops"] == 8 * 176
+    assert info["num_levels"] == 2 * (world - 1)
+    assert info["algorithmic_bytes"] == 5 * (world - 1) * S
+    assert info["position_aligned"] == 1 and info["num_segments"] == 32
+    # column plan: every rank buffer read once and written once
+    assert info["column_load_bytes"] == world * S and info["column_store_bytes"] == world * S
+    assert info["residual_signals"] == 0 and info["buffer_elems"] == n
+    info = _link(graph_jsons("rhd", "build_allreduce", 16, 4096, "float32", "sm")).info()
+    assert info["num_levels"] == 8 and info["algorithmic_bytes"] == 5 * 15 * 4096 * 4
+    info = _link(graph_jsons("tree", "build_allreduce", 32, 4096, "float32", "sm")).info()
+    assert info["num_levels"] == 10 and info["num_data_ops"] == 62
+    info = _link(graph_jsons("ring", "build_alltoall", 4, 4096, "bfloat16")).info()
+    assert info["position_aligned"] == 0 and info["buffer_elems"] == 2 * 4096
+
+
+def test_linked_dependencies_of_the_ring():
+    world, n = 4, 4096
+    ops = _link(graph_jsons("ring", "build_allreduce", world, n, "float32", "sm")).ops()
+    by = {(o.rank, o.level): (k, o) for k, o in enumerate(ops)}
+    for (rank, level), (k, o) in by.items():
+        deps = sorted(list(o.deps)[:o.num_deps])
+        if level == 0:
+            assert deps == []
+        else:   # own previous op and the previous rank's previous op
+            assert deps == sorted([by[(rank, level - 1)][0], by[((rank - 1) % world, level - 1)][0]])
+        assert o.peer_rank == (rank - 1) % world
+        assert o.is_reduce == (1 if level < world - 1 else 0)
+
+
+def _two_rank(build):
+    out = []
+    for rank in range(2):
+        with CommunicationOp(name=f"g{rank}") as op:
+            op.tensor(dtype="float32", shape=(64,))
+            build(op, rank, 1 - rank)
+        out.append(compile_to_json_string(op.get_graph()))
+    return out
+
+
+def _link_err(jsons):
+    with pytest.raises(PcclError) as e:
+        _link(jsons)
+    assert e.value.code == ERR_LINK
+    return str(e.value)
+
+
+def test_linker_reports_deadlock():
+    msg = _link_err(_two_rank(lambda op, me, other: (op.wait_notify(signal_id=3, source_rank=other),
+                                                     op.sm_copy(source_rank=other, src_offset=0, dst_offset=0, size=64))))
+    assert "deadlock" in msg and "signal 3" in msg
+
+
+def test_linker_reports_unordered_conflicting_accesses():
+    # both ranks copy from the other into the range the other is reading, with no ordering at all
+    msg = _link_err(_two_rank(lambda op, me, other: op.sm_copy(source_rank=other, src_offset=0, dst_offset=0, size=64)))
+    assert "data race" in msg
+    # the same exchange made safe: disjoint halves
+    jsons = _two_rank(lambda op, me, other: op.sm_copy(source_rank=other, src_offset=32 * other, dst_offset=32 * other, size=32))
+    assert _link(jsons).info()["num_data_ops"] == 2
+
+
+def test_linker_rejects_bad_ranks_and_mixed_types():
+    msg = _link_err(_two_rank(lambda op, me, other: op.sm_copy(source_rank=5, src_offset=0, dst_offset=0, size=8)))
+    assert "names rank 5" in msg
+    a = graph_jsons("ring", "build_allreduce", 2, 2048, "float32", "sm")
+    b = graph_jsons("ring", "build_allreduce", 2, 2048, "bfloat16", "sm")
+    assert "dtype" in _link_err([a[0], b[1]])
+    c = graph_jsons("ring", "build_reduce_scatter", 2, 2048, "float32", "sm")
+    assert "collective_type" in _link_err([a[0], c[1]])
+
+
+def test_linker_rejects_partially_overlapping_in_place_op():
+    msg = _link_err(_two_rank(lambda op, me, other: op.sm_reduce(source_rank=other, src_offset=0, dst_offset=8,
+                                                                 remote_offset=0, count=32) if me == 0 else
+                              op.notify(signal_id=1, target_rank=other)))
+    assert "overlap" in msg
+
+
+def test_residual_signals_are_counted():
+    jsons = _two_rank(lambda op, me, other: op.notify(signal_id=9, target_rank=other))   # never awaited
+    assert _link(jsons).info()["residual_signals"] == 2
