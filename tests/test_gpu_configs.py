@@ -1,0 +1,161 @@
+"""The benchmark configurations at their full sizes, checked through size-independent properties
+evaluated with plain torch on the GPU (the CPU oracle covers the same graphs at small sizes in
+test_gpu_parity.py):
+
+* ring / RHD / tree results must equal the schedule's per-element reduction order written with
+  torch adds in the storage dtype (bit-exact), and all ranks must hold identical bits;
+* int32 SUM and float MAX must equal torch.stack(x).sum(0) / .amax(0) (order-insensitive);
+* reduce_scatter and allgather must satisfy their definitions chunk by chunk.
+"""
+import pytest
+import torch
+
+from helpers import TORCH_DTYPE, graph_jsons
+from pccl_amd.dsl import ragged_cuts
+
+pytestmark = pytest.mark.gpu
+
+
+def dev_inputs(kind, world, n, dtype, seed=0):
+    """Seeded inputs generated on the GPU (full-size inputs from the CPU generator take minutes)."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    outs = []
+    for _ in range(world):
+        if kind == "randn":
+            x = torch.randn(n, generator=g, device="cuda")
+        elif kind == "uniform":
+            x = torch.rand(n, generator=g, device="cuda") * 2 - 1
+        elif kind == "randn0.1":
+            x = torch.randn(n, generator=g, device="cuda") * 0.1
+        else:
+            x = torch.randint(-1000, 1000, (n,), generator=g, device="cuda")
+        outs.append(x.to(TORCH_DTYPE[dtype]))
+    return outs
+
+
+def same_bits(a, b):
+    if a.dtype in (torch.float16, torch.bfloat16):
+        return torch.equal(a.view(torch.int16), b.view(torch.int16))
+    if a.dtype == torch.float32:
+        return torch.equal(a.view(torch.int32), b.view(torch.int32))
+    return torch.equal(a, b)
+
+
+def register(engine, name, jsons, mode):
+    for r, j in enumerate(jsons):
+        engine.register_operation_json(name, j, r)
+    engine.set_option("mode", mode)
+
+
+def rhd_expected(x, world, lo, n):
+    v = [t[lo:lo + n].clone() for t in x]
+    k = 1
+    while k < world:
+        v = [v[r ^ k] + v[r] for r in range(world)]
+        k <<= 1
+    return v[0]
+
+
+@pytest.mark.parametrize("mode", ["column", "stepwise"])
+def test_config3_rhd_16_ranks_64mb_f32_two_channels(engine_factory, mode):
+    world, n = 16, 16_777_216
+    print(f"config 3: RHD R={world} n={n} f32 2 channels, mode={mode}", flush=True)
+    jsons = graph_jsons("rhd", "build_allreduce", world, n, "float32", "sm", 2)
+    x = dev_inputs("uniform", world, n, "float32")
+    engine = engine_factory(world)
+    register(engine, f"c3_{mode}", jsons, mode)
+    bufs = [t.clone() for t in x]
+    engine.execute_inplace(f"c3_{mode}", bufs, sync=True)
+    want = rhd_expected(x, world, 0, n)
+    assert same_bits(bufs[0], want)
+    for r in range(1, world):
+        assert same_bits(bufs[r], bufs[0]), f"rank {r} differs from rank 0"
+    exact = sum(t.double() for t in x)
+    assert torch.all((bufs[0].double() - exact).abs() <= 1e-6 * world * exact.abs().clamp_min(1.0))
+    info = engine.op_info(f"c3_{mode}")
+    assert info["algorithmic_bytes"] == 75 * n * 4        # 5 (1 - 1/R) R S
+
+
+@pytest.mark.parametrize("mode", ["column", "stepwise"])
+@pytest.mark.parametrize("dtype,redop,kind", [("int32", "sum", "randint"), ("float32", "max", "randn")])
+def test_config5_tree_32_ranks_96mb_ragged(engine_factory, dtype, redop, kind, mode):
+    world, n = 32, 25_165_824
+    print(f"config 5: tree R={world} n={n} {dtype} {redop} ragged, mode={mode}", flush=True)
+    cuts = ragged_cuts(n, 8, seed=0)
+    assert all(c % 4 for c in cuts)
+    jsons = graph_jsons("tree", "build_allreduce", world, n, dtype, "sm", 1, reduce_op=redop, cuts=cuts)
+    x = dev_inputs(kind, world, n, dtype)
+    engine = engine_factory(world)
+    name = f"c5_{dtype}_{mode}"
+    register(engine, name, jsons, mode)
+    bufs = [t.clone() for t in x]
+    engine.execute_inplace(name, bufs, sync=True)
+    if redop == "sum":
+        want = x[0].clone()
+        for t in x[1:]:
+            want += t                                    # int32 wraps; any order gives the same bits
+    else:
+        want = torch.stack(x).amax(0)
+    for r in range(world):
+        assert same_bits(bufs[r], want), f"rank {r}"
+    info = engine.op_info(name)
+    assert info["algorithmic_bytes"] == 155 * n * 4      # 5 (R-1) S
+    assert info["num_data_ops"] == 62 * 8                # every tree op cut into 8 ragged pieces
+
+
+@pytest.mark.parametrize("mode", ["column", "stepwise"])
+@pytest.mark.parametrize("nbytes", [4096, 65536, 1 << 20, 16 << 20, 256 << 20, 512 << 20])
+def test_config4_reduce_scatter_allgather_fp16(engine_factory, nbytes, mode):
+    world = 8
+    n = nbytes // 2
+    chunk = n // world
+    print(f"config 4: RS/AG R={world} {nbytes} B per rank fp16, mode={mode}", flush=True)
+    engine = engine_factory(world)
+    x = dev_inputs("randn0.1", world, n, "float16")
+    # reduce_scatter: chunk r of the ring-ordered sum lands on rank r
+    name = f"rs_{nbytes}_{mode}"
+    register(engine, name, graph_jsons("ring", "build_reduce_scatter", world, n, "float16", "sm", 1), mode)
+    outs = engine.execute_operation(name, x, [torch.zeros(chunk, dtype=torch.float16, device="cuda") for _ in range(world)])
+    for c in range(world):
+        lo = c * chunk
+        # chunk c travels c+1 -> c+2 -> ... -> c: acc = x_{c+1}; acc = x_{c+1+k} + acc
+        acc = x[(c + 1) % world][lo:lo + chunk].clone()
+        for k in range(1, world):
+            acc = x[(c + 1 + k) % world][lo:lo + chunk] + acc
+        assert same_bits(outs[c], acc), f"reduce_scatter chunk {c}"
+    del outs
+    # allgather: rank r contributes chunk r
+    name = f"ag_{nbytes}_{mode}"
+    register(engine, name, graph_jsons("ring", "build_allgather", world, n, "float16", "sm", 1), mode)
+    parts = [t[:chunk].contiguous() for t in x]
+    outs = engine.execute_operation(name, parts, [torch.zeros(n, dtype=torch.float16, device="cuda") for _ in range(world)])
+    whole = torch.cat(parts)
+    for r in range(world):
+        assert same_bits(outs[r], whole), f"allgather rank {r}"
+
+
+def test_config2_headline_shape_in_both_modes_agree(engine_factory):
+    """512 MiB per rank, bf16, 4 channels: column and stepwise runners must produce the same bits."""
+    world, n = 8, 268_435_456
+    print("config 2: ring R=8 512 MiB bf16 4 channels, column vs stepwise", flush=True)
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 4)
+    x = dev_inputs("randn", world, n, "bfloat16")
+    engine = engine_factory(world)
+    results = {}
+    for mode in ("column", "stepwise"):
+        register(engine, f"c2_{mode}", jsons, mode)
+        bufs = [t.clone() for t in x]
+        engine.execute_inplace(f"c2_{mode}", bufs, sync=True)
+        for r in range(1, world):
+            assert same_bits(bufs[r], bufs[0])
+        results[mode] = bufs[0]
+        del bufs
+    assert same_bits(results["column"], results["stepwise"])
+    per_ch, per_rank = n // 4, n // 32
+    for ch in (0, 3):
+        for c in (0, 5):
+            lo = ch * per_ch + c * per_rank
+            acc = x[c][lo:lo + per_rank].clone()
+            for k in range(1, world):
+                acc = x[(c + k) % world][lo:lo + per_rank] + acc
+            assert same_bits(results["column"][lo:lo + per_rank], acc)
