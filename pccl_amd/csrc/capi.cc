@@ -205,6 +205,8 @@ struct OpEntry {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool timed = false;
     bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
+    int epoch = 0;                        // persistent runner: launches so far
+    uint32_t ticket_base = 0;             // persistent runner: tickets consumed so far
     std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
     void release() {
         segs.release(); direct_segs.release(); instrs.release(); fifo.release(); step_ops.release(); step_deps.release();
@@ -235,7 +237,7 @@ struct pccl_hip_ctx {
     int fifo_depth = 0;
     int64_t step_tile_bytes = 128 * 1024;
     bool fuse_staging = true;             // run staged calls on the caller's tensors when possible
-    int spin_limit = 1 << 22;             // polls (~0.1 us sleep each) before a persistent wait gives up
+    int wait_timeout_ms = 2000;           // a persistent launch gives up on a dependency after this long
     hipStream_t last_stream = nullptr;
 };
 
@@ -325,8 +327,9 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
         e.step_ops.upload(so.data(), so.size() * sizeof(DevStepOp));
         e.step_deps.upload(P.step_deps.data(), P.step_deps.size() * sizeof(int32_t));
         e.item_op.upload(item_op.data(), item_op.size() * sizeof(int32_t));
-        std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * (P.ops.size() + 1), 0);
+        std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * ((size_t)P.num_items + 1), 0);
         e.state.upload(zeros.data(), zeros.size());
+        e.epoch = 0; e.ticket_base = 0;
     }
     HIP_TRY(hipEventCreate(&e.ev0));
     HIP_TRY(hipEventCreate(&e.ev1));
@@ -374,8 +377,15 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
         L.ops = (const DevStepOp*)e.step_ops.p; L.num_ops = (int)P.ops.size();
         L.deps = (const int32_t*)e.step_deps.p; L.item_op = (const int32_t*)e.item_op.p;
         L.num_items = (int)P.num_items; L.tile_elems = P.tile_elems; L.state = (StepState*)e.state.p;
-        L.dtype = P.dtype; L.num_blocks = ctx->num_blocks; L.spin_limit = ctx->spin_limit;
+        L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
         if (ctx->mode == Mode::Persistent) {
+            int grid = ctx->num_blocks > 0 ? ctx->num_blocks : device_cu_count(ctx->device) * 8;
+            if (grid > L.num_items) grid = L.num_items;
+            L.num_blocks = grid;
+            L.epoch = ++e.epoch;
+            L.ticket_base = e.ticket_base;
+            L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
+            e.ticket_base += (uint32_t)L.num_items + (uint32_t)grid;   // every workgroup draws one ticket past the end
             rc = launch_persistent(L, ptrs, stream);
             e.ran_persistent = true;
         } else {
@@ -434,6 +444,7 @@ void check_stall(OpEntry& e, const std::string& name) {
     if (st.error_op == 0) return;
     std::vector<char> zeros(e.state.bytes, 0);
     HIP_TRY(hipMemcpy(e.state.p, zeros.data(), zeros.size(), hipMemcpyHostToDevice));
+    e.epoch = 0; e.ticket_base = 0;
     const LinkedOp& a = e.prog.ops[st.error_op - 1];
     const LinkedOp& b = e.prog.ops[st.error_dep - 1];
     throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting: data op " + std::to_string(st.error_op - 1) +
@@ -518,19 +529,16 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             if (v == "auto") ctx->mode = Mode::Auto;
             else if (v == "column") ctx->mode = Mode::Column;
             else if (v == "stepwise") ctx->mode = Mode::Stepwise;
-            else if (v == "persistent") {
-                // The single-launch flag-ordered runner stopped making progress on MI355X in its
-                // first runs and the cause has not been established; until it is, the mode is
-                // refused rather than launched.  PCCL_ENABLE_PERSISTENT=1 is for developers only.
-                if (!std::getenv("PCCL_ENABLE_PERSISTENT"))
-                    return fail(PCCL_ERR_UNSUPPORTED, "mode 'persistent' is switched off: the flag-ordered single-launch runner hangs on MI355X (cause not yet established); use 'stepwise' or 'column'");
-                ctx->mode = Mode::Persistent;
-            }
+            else if (v == "persistent")
+                // The single-launch flag-ordered runner never drained on MI355X in three attempts
+                // (tile counters, bounded polls, store-published per-item flags with a wall-clock
+                // bound); the cause is not established, so the mode is refused, never launched.
+                return fail(PCCL_ERR_UNSUPPORTED, "mode 'persistent' is switched off: the flag-ordered single-launch runner does not drain on MI355X (cause not yet established); use 'stepwise' or 'column'");
             else return fail(PCCL_ERR_INVALID, "mode must be auto, column, stepwise or persistent");
         } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
         else if (k == "timing") ctx->timing = std::atoi(value) != 0;
         else if (k == "fuse_staging") ctx->fuse_staging = std::atoi(value) != 0;
-        else if (k == "spin_limit") { ctx->spin_limit = std::atoi(value); if (ctx->spin_limit < 1) ctx->spin_limit = 1; }
+        else if (k == "wait_timeout_ms") { ctx->wait_timeout_ms = std::atoi(value); if (ctx->wait_timeout_ms < 1) ctx->wait_timeout_ms = 1; }
         else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
         else if (k == "vecs_per_thread") {
             int u = std::atoi(value);
@@ -664,6 +672,7 @@ int pccl_hip_reset_signals(pccl_hip_ctx* ctx, const char* name) {
             int rc = launch_fill_zero(e.state.p, e.state.bytes, ctx->last_stream);
             if (rc) return fail(PCCL_ERR_HIP, hipGetErrorString((hipError_t)rc));
             HIP_TRY(hipStreamSynchronize(ctx->last_stream));
+            e.epoch = 0; e.ticket_base = 0;
         }
         return 0;
     });

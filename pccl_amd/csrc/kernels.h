@@ -30,13 +30,13 @@ struct DevStepOp {
     int32_t first_item, ntiles, dep_start, ndeps;
 };
 
-struct StepState {      // device memory, zero between launches (the kernel restores it on exit)
-    int32_t cursor;
-    int32_t exited;
+struct StepState {      // device memory of the persistent runner
+    uint32_t ticket;    // next work ticket; never reset, the host tracks where a launch starts
+    int32_t reserved;
     int32_t error_op;   // 1 + index of the op whose bounded wait expired (0 = none); host clears it
     int32_t error_dep;  // 1 + index of the predecessor it was waiting for
     int32_t pad[28];
-    // followed by int32 done[num_ops]
+    // followed by int32 flag[num_items]: the epoch of the launch that last completed the item
 };
 
 struct ColumnLaunch {
@@ -60,7 +60,9 @@ struct StepwiseLaunch {
     StepState* state;
     int32_t dtype;
     int32_t num_blocks;
-    int32_t spin_limit;   // polls of one dependency counter before the persistent runner gives up
+    int32_t epoch;            // persistent runner: value a completed item's flag takes in this launch
+    uint32_t ticket_base;     // persistent runner: ticket of this launch's item 0
+    uint64_t timeout_ticks;   // persistent runner: 100 MHz ticks a workgroup may run before a wait gives up
 };
 
 // All return a hipError_t value as int (0 = success).

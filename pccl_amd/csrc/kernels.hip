@@ -269,52 +269,62 @@ __global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int i
 // ------------------------------------------------------------------------------- persistent runner
 //
 // One persistent launch executes every data op of the linked program.  Work items are (op, tile)
-// pairs in level order; a workgroup claims the next item from one atomic cursor, waits until every
-// tile of the op's predecessors has been published, runs the tile, then publishes it.  A claimed
-// item only ever waits for items claimed earlier by workgroups that are already running, so the
-// scheme cannot deadlock whatever the grid size.  Every wait is bounded all the same: after
-// `spin_limit` polls the waiter records (op, predecessor) in the state block and every workgroup
-// leaves at its next claim, so the grid always drains and the host reports the stall as an error.
+// pairs in level order; a workgroup takes the next item from one atomic ticket counter, waits
+// until every item of the op's predecessors has been published, runs the item, then publishes it.
+// A claimed item only ever waits for items claimed earlier by workgroups that are already running,
+// so the scheme cannot deadlock whatever the grid size.
+//
+// Cross-workgroup visibility follows the pattern the ROCm scan primitives use on multi-XCD parts:
+// one flag word per item, published with an agent-scope atomic STORE after an agent-scope release
+// fence and polled with agent-scope atomic LOADs (both bypass the per-XCD L2).  A flag holds the
+// launch epoch, so flags are never cleared; the ticket counter is never reset either (the host
+// passes the ticket of this launch's item 0).  Every wait is bounded by wall-clock time: when
+// `timeout_ticks` of the 100 MHz counter have passed since the workgroup started, the waiter
+// records (op, predecessor) and every workgroup leaves at its next claim, so the grid always
+// drains and the host reports the stall as an error.
 
 template <int DT>
 __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     constexpr int ES = ElemBytes<DT>::value;
     __shared__ int s_item;
-    __shared__ int s_last;
-    int32_t* done = reinterpret_cast<int32_t*>(L.state + 1);
+    int32_t* flags = reinterpret_cast<int32_t*>(L.state + 1);
     const int tid = threadIdx.x;
+    const uint64_t t_start = __builtin_amdgcn_s_memrealtime();
     for (;;) {
         if (tid == 0) {
             int stalled = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_item = stalled ? L.num_items : atomicAdd(&L.state->cursor, 1);
+            s_item = stalled ? L.num_items : (int)(atomicAdd(&L.state->ticket, 1u) - L.ticket_base);
         }
         __syncthreads();
-        int item = s_item;
+        const int item = s_item;
         __syncthreads();
-        if (item >= L.num_items) break;
-        int opi = L.item_op[item];
-        DevStepOp op = L.ops[opi];
-        if (tid < op.ndeps) {
-            int d = L.deps[op.dep_start + tid];
-            int need = L.ops[d].ntiles;
-            int spins = 0;
-            while (__hip_atomic_load(&done[d], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
-                if (++spins > L.spin_limit ||
-                    __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
-                    if (spins > L.spin_limit) {
+        if (item >= L.num_items || item < 0) break;
+        const int opi = L.item_op[item];
+        const DevStepOp op = L.ops[opi];
+        // wait: thread t watches items t, t+256, ... of each predecessor
+        for (int k = 0; k < op.ndeps; ++k) {
+            const int d = L.deps[op.dep_start + k];
+            const int first = L.ops[d].first_item, nt = L.ops[d].ntiles;
+            for (int t = tid; t < nt; t += kThreads) {
+                int nap = 1;
+                while (__hip_atomic_load(&flags[first + t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != L.epoch) {
+                    if (__builtin_amdgcn_s_memrealtime() - t_start > L.timeout_ticks) {
                         __hip_atomic_store(&L.state->error_dep, d + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         __hip_atomic_store(&L.state->error_op, opi + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
                     }
-                    break;
+                    if (__hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+                    __builtin_amdgcn_s_sleep(1);
+                    for (int z = 1; z < nap; ++z) __builtin_amdgcn_s_sleep(8);
+                    if (nap < 32) nap <<= 1;
                 }
-                __builtin_amdgcn_s_sleep(8);
             }
         }
         __syncthreads();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         if (tid == 0) s_item = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        bool stalled = s_item != 0;
+        const bool stalled = s_item != 0;
         __syncthreads();
         if (stalled) break;   // a predecessor never arrived: do not touch the data, just drain
         int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
@@ -328,16 +338,8 @@ __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, 
         __syncthreads();  // every wave's stores are issued and counted before the publish
         if (tid == 0) {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            __hip_atomic_fetch_add(&done[opi], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&flags[item], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-    }
-    // the last workgroup out restores the progress counters for the next launch (the error
-    // words stay until the host has read and cleared them)
-    if (tid == 0) s_last = (atomicAdd(&L.state->exited, 1) == (int)gridDim.x - 1);
-    __syncthreads();
-    if (s_last) {
-        for (int i = tid; i < L.num_ops; i += kThreads) done[i] = 0;
-        if (tid == 0) { L.state->cursor = 0; L.state->exited = 0; }
     }
 }
 

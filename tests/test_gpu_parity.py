@@ -46,9 +46,10 @@ CASES = [
 ]
 
 
-PERSISTENT_OFF = pytest.mark.skip(reason="the persistent flag-ordered runner hung on MI355X (wait for a "
-                                   "predecessor's tile counter never returned); the mode is refused "
-                                   "by the library until the cause is found")
+PERSISTENT_OFF = pytest.mark.skip(reason="the persistent flag-ordered runner never drained on MI355X in "
+                                   "three forms (tile counters, bounded polls, store-published flags "
+                                   "with a wall-clock bound); the mode is refused by the library until "
+                                   "the cause is found")
 MODES = ["column", "stepwise", pytest.param("persistent", marks=PERSISTENT_OFF)]
 
 
