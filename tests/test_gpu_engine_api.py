@@ -1,0 +1,187 @@
+"""Engine facade on the GPU: the reference's call shapes (pccl/engine.py:11-71,
+tests/test_correctness.py:92-104) and the error behaviour of the boundary."""
+import json
+import os
+
+import pytest
+import torch
+
+from helpers import bits_equal, graph_jsons, oracle_buffers, seeded_inputs
+from pccl_amd import engine as engine_mod
+from pccl_amd._lib import ERR_INVALID, ERR_LINK, ERR_NOT_FOUND, ERR_UNSUPPORTED, PcclError
+
+pytestmark = pytest.mark.gpu
+
+
+def write_graphs(tmp_path, stem, jsons):
+    for r, j in enumerate(jsons):
+        (tmp_path / f"{stem}_rank{r}.json").write_text(j)
+    return str(tmp_path / (stem + "_rank{rank}.json"))
+
+
+def test_reference_style_per_rank_flow(engine_factory, tmp_path):
+    """register per rank from files, post execute_operation_async per rank, sync, compare."""
+    world, n = 4, 1 << 14
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "tma", 1)
+    pattern = write_graphs(tmp_path, "ar", jsons)
+    eng = engine_factory(world)
+    for r in range(world):
+        assert eng.rank(r).register_operation("test_allreduce", pattern.format(rank=r)) is True
+    inp = [torch.ones(n, dtype=torch.bfloat16, device="cuda") * (r + 1) for r in range(world)]
+    out = [torch.zeros_like(t) for t in inp]
+    for r in range(world):
+        eng.rank(r).execute_operation_async("test_allreduce", inp[r], out[r])
+    eng.sync_operation("test_allreduce")
+    torch.cuda.synchronize()
+    for r in range(world):
+        assert (out[r] != world * (world + 1) / 2).sum().item() == 0
+    eng.reset_signals("test_allreduce")            # a no-op here, must not fail
+    # a second round reuses the registration; the last rank may use the synchronising form
+    for r in range(world - 1):
+        eng.rank(r).execute_operation_async("test_allreduce", inp[r], out[r])
+    res = eng.rank(world - 1).execute_operation("test_allreduce", inp[world - 1], out[world - 1])
+    assert res is out[world - 1] and (res != 10).sum().item() == 0
+    # a synchronising call before the others have posted cannot complete
+    with pytest.raises(RuntimeError, match="would block"):
+        eng.rank(0).execute_operation("test_allreduce", inp[0], out[0])
+
+
+def test_collective_form_with_placeholder_and_stacked_tensor(engine_factory, tmp_path):
+    world, n = 4, 4096
+    jsons = graph_jsons("rhd", "build_allreduce", world, n, "float32", "sm", 1)
+    eng = engine_factory(world)
+    assert eng.register_operation("rhd", write_graphs(tmp_path, "rhd", jsons)) is True
+    x = seeded_inputs("randn", world, n, "float32", seed=21)
+    want = oracle_buffers(jsons, x, "float32")
+    outs = eng.execute_operation("rhd", torch.stack(x).cuda())     # [R, N] tensor, outputs allocated
+    for r in range(world):
+        assert bits_equal(outs[r], want[r])
+    outs = eng.execute_operation_async("rhd", [t.cuda() for t in x])
+    eng.sync_operation("rhd")
+    assert bits_equal(outs[2], want[2])
+    info = eng.op_info("rhd")
+    assert info["num_vranks"] == world and info["num_levels"] == 4
+
+
+def test_module_level_api(tmp_path):
+    world, n = 2, 2048
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float16", "sm", 1)
+    pattern = write_graphs(tmp_path, "m", jsons)
+    engine_mod.initialize_engine(num_vranks=world)
+    try:
+        assert engine_mod.register_operation("m", pattern) is True
+        x = [torch.full((n,), float(r + 1), dtype=torch.float16, device="cuda") for r in range(world)]
+        outs = engine_mod.execute_operation("m", x)
+        assert all(torch.all(o == 3) for o in outs)
+        engine_mod.sync_operation("m")
+        engine_mod.reset_signals("m")
+    finally:
+        engine_mod.get_engine().close()
+        engine_mod._engine_instance = None
+
+
+def test_registration_and_lookup_errors(engine_factory, tmp_path):
+    eng = engine_factory(2)
+    assert eng.register_operation("nofile", str(tmp_path / "missing_rank{rank}.json")) is False   # reference: regOp -> false
+    (tmp_path / "bad_rank0.json").write_text('{"version": 2}')
+    assert eng.register_operation("bad", str(tmp_path / "bad_rank0.json"), rank=0) is False
+    doc = json.loads(graph_jsons("ring", "build_allreduce", 2, 2048, "float32", "sm")[0])
+    doc["operations"][2]["primitive"] = "sm.scatter"
+    (tmp_path / "prim_rank0.json").write_text(json.dumps(doc))
+    with pytest.raises(PcclError, match="unknown primitive"):
+        eng.register_operation("prim", str(tmp_path / "prim_rank0.json"), rank=0)
+    with pytest.raises(PcclError) as e:
+        eng.register_operation_json("x", "{}", 7)
+    assert e.value.code == ERR_INVALID or "operations" in str(e.value)
+    x = [torch.zeros(16, device="cuda") for _ in range(2)]
+    with pytest.raises(PcclError, match="Unknown operation") as e:
+        eng.execute_operation("never_registered", x)
+    assert e.value.code == ERR_NOT_FOUND
+    eng.sync_operation("never_registered")                    # the reference returns silently
+    with pytest.raises(ValueError, match="expected 2 tensors"):
+        eng.execute_operation("never_registered", x[:1])
+    with pytest.raises(ValueError, match="GPU"):
+        eng.execute_operation("never_registered", [t.cpu() for t in x])
+    with pytest.raises(PcclError):
+        eng.set_option("mode", "warp-speed")
+
+
+def test_link_errors_surface_at_first_execution(engine_factory):
+    from pccl_amd.dsl import CommunicationOp, compile_to_json_string
+    eng = engine_factory(2)
+    # only one of two ranks registered
+    eng.register_operation_json("half", graph_jsons("ring", "build_allreduce", 2, 2048, "float32", "sm")[0], 0)
+    x = [torch.zeros(2048, device="cuda") for _ in range(2)]
+    with pytest.raises(PcclError, match="no registered graph") as e:
+        eng.execute_operation("half", x)
+    assert e.value.code == ERR_LINK
+    # a wait nobody releases: reported, not hung
+    for rank in range(2):
+        with CommunicationOp(name=f"dl{rank}") as op:
+            op.tensor(dtype="float32", shape=(2048,))
+            op.wait_notify(signal_id=5, source_rank=1 - rank)
+            op.sm_copy(source_rank=1 - rank, src_offset=0, dst_offset=0, size=2048)
+        eng.register_operation_json("deadlock", compile_to_json_string(op.get_graph()), rank)
+    with pytest.raises(PcclError, match="deadlock"):
+        eng.execute_operation("deadlock", x)
+
+
+def test_buffer_checks_and_mode_selection(engine_factory):
+    world, n = 2, 4096
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm")
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("ar", j, r)
+    x = seeded_inputs("randn", world, n, "float32", seed=4)
+    want = oracle_buffers(jsons, x, "float32")
+    small = [torch.zeros(n // 2, device="cuda") for _ in range(world)]
+    with pytest.raises(PcclError, match="smaller than"):
+        eng.execute_inplace("ar", small, sync=True)
+    # buffers that are only 4-byte aligned: auto falls back to the level runner, column refuses
+    base = [torch.zeros(n + 4, device="cuda") for _ in range(world)]
+    shifted = [b[1:n + 1] for b in base]
+    for s, t in zip(shifted, x):
+        s.copy_(t)
+    eng.set_option("mode", "auto")
+    eng.execute_inplace("ar", shifted, sync=True)
+    for r in range(world):
+        assert bits_equal(shifted[r], want[r])
+    eng.set_option("mode", "column")
+    with pytest.raises(PcclError, match="16-byte aligned") as e:
+        eng.execute_inplace("ar", shifted, sync=True)
+    assert e.value.code == ERR_UNSUPPORTED
+    eng.set_option("mode", "auto")
+    # staged call on the same misaligned tensors (direct plan does not apply, staging does)
+    for s, t in zip(shifted, x):
+        s.copy_(t)
+    outs = eng.execute_operation("ar", shifted)
+    for r in range(world):
+        assert bits_equal(outs[r], want[r])
+
+
+def test_column_mode_refuses_graphs_that_are_not_position_aligned(engine_factory):
+    world, n = 4, 4096
+    eng = engine_factory(world)
+    for r, j in enumerate(graph_jsons("ring", "build_alltoall", world, n, "bfloat16")):
+        eng.register_operation_json("a2a", j, r)
+    eng.set_option("mode", "column")
+    x = [torch.zeros(n, dtype=torch.bfloat16, device="cuda") for _ in range(world)]
+    with pytest.raises(PcclError, match="same element positions"):
+        eng.execute_operation("a2a", x)
+    eng.set_option("mode", "auto")
+    eng.execute_operation("a2a", x)
+
+
+def test_kernel_timing_option(engine_factory):
+    world, n = 8, 1 << 20
+    eng = engine_factory(world)
+    for r, j in enumerate(graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 4)):
+        eng.register_operation_json("t", j, r)
+    bufs = [torch.zeros(n, dtype=torch.bfloat16, device="cuda") for _ in range(world)]
+    with pytest.raises(PcclError, match="timing"):
+        eng.last_kernel_ms("t")
+    eng.set_option("timing", 1)
+    eng.execute_inplace("t", bufs, sync=True)
+    ms = eng.last_kernel_ms("t")
+    eng.set_option("timing", 0)
+    assert 0.0 < ms < 50.0
