@@ -406,22 +406,28 @@ bool run_direct(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
     const Program& P = e.prog;
     if (!ctx->fuse_staging || ctx->mode == Mode::Stepwise || ctx->mode == Mode::Persistent) return false;
     if (!P.position_aligned || P.direct_segs.empty() || !e.direct_segs.p) return false;
-    if (!(P.collective_type.empty() || P.collective_type == "allreduce")) return false;
     const size_t es = elem_size(P.dtype);
-    if (in_bytes != out_bytes || in_bytes != (size_t)P.tensor_elems * es) return false;
+    // the tensors must be exactly the windows the plan was built for
+    const size_t want_in = (size_t)(P.direct_in_end[0] - P.direct_in_start[0]) * es;
+    const size_t want_out = (size_t)(P.direct_out_end[0] - P.direct_out_start[0]) * es;
+    if (in_bytes != want_in || out_bytes < want_out) return false;
+    const bool same_windows = P.direct_in_start == P.direct_out_start && P.direct_in_end == P.direct_out_end;
     RankPtrs ptrs;
     std::memset(&ptrs, 0, sizeof(ptrs));
     for (int r = 0; r < ctx->R; ++r) {
         uintptr_t in = (uintptr_t)inputs[r], out = (uintptr_t)outputs[r];
-        if ((in | out) & 15) return false;
-        if (in != out && in < out + out_bytes && out < in + in_bytes) return false;  // partial overlap
+        // position p of rank r lives at base + p*es: shift the bases by the window starts
+        uintptr_t in_base = in - (uintptr_t)P.direct_in_start[r] * es, out_base = out - (uintptr_t)P.direct_out_start[r] * es;
+        if ((in_base | out_base) & 15) return false;
+        bool aliased = in == out && same_windows;   // in place: every position read before it is written
+        if (!aliased && in < out + want_out && out < in + in_bytes) return false;
         for (int q = 0; q < r; ++q) {  // an output must not alias another rank's tensors
             uintptr_t oq = (uintptr_t)outputs[q], iq = (uintptr_t)inputs[q];
-            if ((out < oq + out_bytes && oq < out + out_bytes) || (out < iq + in_bytes && iq < out + out_bytes) ||
-                (oq < in + in_bytes && in < oq + out_bytes)) return false;
+            if ((out < oq + want_out && oq < out + want_out) || (out < iq + in_bytes && iq < out + want_out) ||
+                (oq < in + in_bytes && in < oq + want_out)) return false;
         }
-        ptrs.p[r] = (char*)outputs[r];
-        ptrs.p[PCCL_HIP_MAX_VRANKS + r] = (char*)inputs[r];
+        ptrs.p[r] = (char*)out_base;
+        ptrs.p[PCCL_HIP_MAX_VRANKS + r] = (char*)in_base;
     }
     if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
     ColumnLaunch L{};

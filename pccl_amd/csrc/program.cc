@@ -238,6 +238,42 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
         P.race_checked = complete;
     }
 
+    // ---- keep only the orderings that matter: B must follow A exactly when A happens before B
+    //      AND they touch overlapping memory with at least one write.  Chain order between ops on
+    //      disjoint ranges (e.g. the ragged pieces of one schedule step) is not a dependency, so
+    //      such ops share a level and run in one launch.  Any execution that respects these edges
+    //      gives the results of every order the notify/wait chains allow.
+    if (opt.conflict_deps && closure && D > 1 && D <= 8192) {
+        auto overlaps = [](int64_t s0, int64_t n0, int64_t s1, int64_t n1) { return s0 < s1 + n1 && s1 < s0 + n0; };
+        auto conflict = [&](const LinkedOp& A, const LinkedOp& B) {
+            if (A.size <= 0 || B.size <= 0) return false;
+            // writes of A against every access of B, and writes of B against reads of A
+            if (A.rank == B.rank && overlaps(A.dst_off(), A.size, B.dst_off(), B.size)) return true;
+            if (A.rank == B.peer && overlaps(A.dst_off(), A.size, B.off0, B.size)) return true;
+            if (B.is_reduce && A.rank == B.rank && overlaps(A.dst_off(), A.size, B.off1, B.size)) return true;
+            if (B.rank == A.peer && overlaps(B.dst_off(), B.size, A.off0, A.size)) return true;
+            if (A.is_reduce && A.rank == B.rank && overlaps(B.dst_off(), B.size, A.off1, A.size)) return true;
+            return false;
+        };
+        std::vector<Bitset> kept(D, Bitset(D));   // data ops ordered before k through kept edges
+        P.num_levels = 0;
+        for (int k = 0; k < D; ++k) {             // ops[] is in execution (topological) order
+            LinkedOp& B = ops[k];
+            B.deps.clear();
+            for (int a = k - 1; a >= 0; --a) {    // latest first, so covered ancestors are skipped
+                if (kept[k].test(a)) continue;
+                if (!reach[data_nodes[k]].test(data_nodes[a]) || !conflict(ops[a], B)) continue;
+                B.deps.push_back(a);
+                kept[k].or_with(kept[a]);
+                kept[k].set(a);
+            }
+            int lvl = 0;
+            for (int d : B.deps) lvl = std::max(lvl, ops[d].level + 1);
+            B.level = lvl;
+            P.num_levels = std::max(P.num_levels, lvl + 1);
+        }
+    }
+
     // ---- final order: (level, rank, channel, graph position); remap deps
     std::vector<int> perm(D);
     std::iota(perm.begin(), perm.end(), 0);
@@ -364,53 +400,93 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
 
         // ---- direct plan: the same programs with the caller's input tensors as the source of
         // every first-touch load and the output tensors as the destination of every store, so
-        // that no staging copy is needed.  For the output to equal "input copied in, program
-        // run, buffer copied out", a (rank, position) the program never writes must be passed
-        // through from input to output: one copy instruction (peer = self, first touch) per
-        // unwritten rank of a segment, and whole pass-through segments over the uncovered gaps.
-        if (P.tensor_elems >= P.buffer_elems && P.tensor_elems > 0) {
-            auto passthrough = [&](uint64_t written) {
-                for (int r = 0; r < R; ++r)
-                    if (!(written >> r & 1)) {
+        // that no staging copy is needed.  The staged semantics are "place input r in buffer r at
+        // its window, run, hand back the output window of buffer r" (reference engine_c.cc:468-548):
+        //   allreduce / untyped   in [0,n)                out [0,n)
+        //   reduce_scatter        in [0,n)                out [r*n/R, (r+1)*n/R)
+        //   allgather             in [r*n/R, (r+1)*n/R)   out [0,n)
+        // For the result to be identical, a (rank, position) inside the output window that the
+        // program never writes is passed through from the input (one copy instruction with
+        // peer = self), a final store outside the output window is dropped (nobody can observe
+        // it), and the plan is abandoned (staging is used instead) if any access would need
+        // memory outside the windows: a first touch outside the input window, or a value that is
+        // written outside the output window and read back later.
+        const int64_t n = P.tensor_elems;
+        const std::string& ct = P.collective_type;
+        const bool ar = ct.empty() || ct == "allreduce";
+        const bool rs = ct == "reduce_scatter", ag = ct == "allgather";
+        if ((ar || rs || ag) && n >= P.buffer_elems && n > 0 && (ar || n % R == 0)) {
+            const int64_t chunk = n / R;
+            P.direct_in_start.assign(R, 0); P.direct_in_end.assign(R, n);
+            P.direct_out_start.assign(R, 0); P.direct_out_end.assign(R, n);
+            for (int r = 0; r < R; ++r) {
+                if (rs) { P.direct_out_start[r] = r * chunk; P.direct_out_end[r] = (r + 1) * chunk; }
+                if (ag) { P.direct_in_start[r] = r * chunk; P.direct_in_end[r] = (r + 1) * chunk; }
+            }
+            std::vector<int64_t> cuts2 = {0, n};
+            for (auto& sg : P.segs) { cuts2.push_back(sg.start); cuts2.push_back(sg.end); }
+            if (!ar) for (int r = 0; r <= R; ++r) cuts2.push_back(r * chunk);
+            std::sort(cuts2.begin(), cuts2.end());
+            cuts2.erase(std::unique(cuts2.begin(), cuts2.end()), cuts2.end());
+            bool valid = true;
+            std::vector<ColInstr> prev_prog;
+            const std::vector<ColSegment> base_segs = P.segs;
+            size_t si = 0;
+            for (size_t i = 0; i + 1 < cuts2.size() && valid; ++i) {
+                const int64_t a = cuts2[i], b = cuts2[i + 1];
+                if (a < 0 || b > n) continue;
+                while (si < base_segs.size() && base_segs[si].end <= a) ++si;
+                const ColSegment* base = (si < base_segs.size() && base_segs[si].start <= a && b <= base_segs[si].end) ? &base_segs[si] : nullptr;
+                auto in_window = [&](int r) { return P.direct_in_start[r] <= a && b <= P.direct_in_end[r]; };
+                auto out_window = [&](int r) { return P.direct_out_start[r] <= a && b <= P.direct_out_end[r]; };
+                std::vector<ColInstr> prog;
+                uint64_t written = 0;
+                if (base)
+                    for (int k = 0; k < base->prog_len && valid; ++k) {
+                        ColInstr in = P.col_instrs[base->prog_start + k];
+                        if (in.a_src == SRC_MEM) valid = in.a_first ? in_window(in.peer) : out_window(in.peer);
+                        if (valid && in.b_src == SRC_MEM) valid = in.b_first ? in_window(in.self) : out_window(in.self);
+                        if (in.store && !out_window(in.self)) {
+                            if (in.store == 1) valid = false;   // written outside the window and read back
+                            in.store = 0;
+                        }
+                        if (in.store) written |= 1ull << in.self;
+                        prog.push_back(in);
+                    }
+                for (int r = 0; r < R && valid; ++r)
+                    if (out_window(r) && !(written >> r & 1)) {
+                        if (!in_window(r)) { valid = false; break; }   // the reference would hand back stale buffer contents
                         ColInstr in{};
                         in.self = in.peer = (uint8_t)r; in.a_src = SRC_MEM; in.b_src = SRC_NONE;
                         in.a_first = 1; in.store = 2;
-                        P.col_instrs.push_back(in);
+                        prog.push_back(in);
                     }
-            };
-            auto gap_segment = [&](int64_t a, int64_t b) {
-                if (a >= b) return;
-                ColSegment g;
-                g.start = a; g.end = b; g.prog_start = (int)P.col_instrs.size();
-                passthrough(0);
-                g.prog_len = (int)P.col_instrs.size() - g.prog_start;
-                P.direct_segs.push_back(g);
-            };
-            int64_t cursor = 0;
-            const std::vector<ColSegment> base_segs = P.segs;
-            for (const ColSegment& seg : base_segs) {
-                gap_segment(cursor, seg.start);
-                ColSegment d = seg;
-                d.prog_start = (int)P.col_instrs.size();
-                uint64_t written = 0;
-                for (int k = 0; k < seg.prog_len; ++k) {
-                    ColInstr in = P.col_instrs[seg.prog_start + k];
-                    written |= 1ull << in.self;
-                    P.col_instrs.push_back(in);
+                if (!valid) break;
+                // an instruction that neither stores nor feeds a later one can go
+                while (!prog.empty() && !prog.back().store) prog.pop_back();
+                if (prog.empty()) { prev_prog.clear(); continue; }
+                auto same = [&](const std::vector<ColInstr>& x, const std::vector<ColInstr>& y) {
+                    return x.size() == y.size() && std::memcmp(x.data(), y.data(), x.size() * sizeof(ColInstr)) == 0;
+                };
+                if (!P.direct_segs.empty() && P.direct_segs.back().end == a && same(prog, prev_prog)) {
+                    P.direct_segs.back().end = b;
+                    continue;
                 }
-                passthrough(written);
-                d.prog_len = (int)P.col_instrs.size() - d.prog_start;
+                ColSegment d;
+                d.start = a; d.end = b;
+                d.prog_start = (int)P.col_instrs.size(); d.prog_len = (int)prog.size();
+                P.col_instrs.insert(P.col_instrs.end(), prog.begin(), prog.end());
                 P.direct_segs.push_back(d);
-                cursor = seg.end;
+                prev_prog.swap(prog);
             }
-            gap_segment(cursor, P.tensor_elems);
+            if (!valid) P.direct_segs.clear();
             for (auto& seg : P.direct_segs) {
-                int64_t n = seg.end - seg.start;
+                int64_t len = seg.end - seg.start;
                 for (int k = 0; k < seg.prog_len; ++k) {
                     const ColInstr& in = P.col_instrs[seg.prog_start + k];
-                    if (in.a_src == SRC_MEM || in.a_src == SRC_FIFO) P.direct_load_bytes += n * es;
-                    if (in.b_src == SRC_MEM || in.b_src == SRC_FIFO) P.direct_load_bytes += n * es;
-                    if (in.store) P.direct_store_bytes += n * es;
+                    if (in.a_src == SRC_MEM || in.a_src == SRC_FIFO) P.direct_load_bytes += len * es;
+                    if (in.b_src == SRC_MEM || in.b_src == SRC_FIFO) P.direct_load_bytes += len * es;
+                    if (in.store) P.direct_store_bytes += len * es;
                 }
             }
         }

@@ -73,6 +73,7 @@ struct Program {
     // direct plan (staging fused into the program; valid when non-empty): covers [0, tensor_elems)
     std::vector<ColSegment> direct_segs;
     int64_t direct_load_bytes = 0, direct_store_bytes = 0;
+    std::vector<int64_t> direct_in_start, direct_in_end, direct_out_start, direct_out_end;  // windows per rank
 
     // stepwise plan
     int64_t tile_elems = 0;
@@ -83,6 +84,7 @@ struct Program {
 
 struct LinkOptions {
     bool check_races = true;
+    bool conflict_deps = true;     // order data ops by memory conflicts instead of raw chain order
     int fifo_depth = 0;            // 0: every first-touch load is SRC_MEM
     int64_t step_tile_bytes = 128 * 1024;
 };

@@ -205,6 +205,10 @@ def test_program_info_closed_forms():
     assert info["num_levels"] == 8 and info["algorithmic_bytes"] == 5 * 15 * 4096 * 4
     info = _link(graph_jsons("tree", "build_allreduce", 32, 4096, "float32", "sm")).info()
     assert info["num_levels"] == 10 and info["num_data_ops"] == 62
+    # ragged pieces of one schedule step touch disjoint ranges: they share a level
+    from pccl_amd.dsl import ragged_cuts
+    info = _link(graph_jsons("tree", "build_allreduce", 32, 4099, "int32", "sm", cuts=ragged_cuts(4099, 8))).info()
+    assert info["num_levels"] == 10 and info["num_data_ops"] == 62 * 8
     info = _link(graph_jsons("ring", "build_alltoall", 4, 4096, "bfloat16")).info()
     assert info["position_aligned"] == 0 and info["buffer_elems"] == 2 * 4096
 
@@ -217,8 +221,10 @@ def test_linked_dependencies_of_the_ring():
         deps = sorted(list(o.deps)[:o.num_deps])
         if level == 0:
             assert deps == []
-        else:   # own previous op and the previous rank's previous op
-            assert deps == sorted([by[(rank, level - 1)][0], by[((rank - 1) % world, level - 1)][0]])
+        else:   # the producer of the chunk this op pulls: the previous rank's previous op.  (The own
+                # previous op works on another chunk: chain order, but no memory conflict.)
+            assert by[((rank - 1) % world, level - 1)][0] in deps
+            assert all(ops[d].level < level for d in deps)
         assert o.peer_rank == (rank - 1) % world
         assert o.is_reduce == (1 if level < world - 1 else 0)
 
