@@ -231,7 +231,7 @@ struct pccl_hip_ctx {
     size_t buf_bytes = 0;
     Mode mode = Mode::Auto;
     int num_blocks = 0;
-    int vecs_per_thread = 2;
+    int vecs_per_thread = 1;
     bool check_races = true;
     bool timing = false;
     int fifo_depth = 0;

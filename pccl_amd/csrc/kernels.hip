@@ -15,6 +15,22 @@ namespace pccl_hip {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 
+// Every pointer the kernels see is device memory: say so, so that global_* (not flat_*)
+// instructions are selected.
+#define PCCL_GLOBAL __attribute__((address_space(1)))
+// Plan tables never change while a kernel runs: reading them through the constant address space
+// lets uniform accesses become scalar loads (scalar cache, no vector-memory slot, no readfirstlane).
+#define PCCL_CONST __attribute__((address_space(4)))
+template <class T> __device__ __forceinline__ const PCCL_CONST T* as_const(const T* p) { return (const PCCL_CONST T*)p; }
+template <class T> __device__ __forceinline__ T load_const(const T* p) {   // whole table record, 8 bytes at a time
+    static_assert(sizeof(T) % 8 == 0, "table records are multiples of 8 bytes");
+    T out;
+    const PCCL_CONST uint64_t* w = (const PCCL_CONST uint64_t*)p;
+    uint64_t* o = reinterpret_cast<uint64_t*>(&out);
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(T) / 8; ++i) o[i] = w[i];
+    return out;
+}
 constexpr int kThreads = 256;
 constexpr int kMaxR = PCCL_HIP_MAX_VRANKS;
 
@@ -98,16 +114,16 @@ __device__ __forceinline__ u32x4 vec_op(u32x4 a, u32x4 b, int redop) {
 template <int DT>
 __device__ __forceinline__ uint32_t load_elem(const char* p) {
     constexpr int ES = ElemBytes<DT>::value;
-    if constexpr (ES == 4) return *reinterpret_cast<const uint32_t*>(p);
-    else if constexpr (ES == 2) return *reinterpret_cast<const uint16_t*>(p);
-    else return *reinterpret_cast<const uint8_t*>(p);
+    if constexpr (ES == 4) return *(const PCCL_GLOBAL uint32_t*)(p);
+    else if constexpr (ES == 2) return *(const PCCL_GLOBAL uint16_t*)(p);
+    else return *(const PCCL_GLOBAL uint8_t*)(p);
 }
 template <int DT>
 __device__ __forceinline__ void store_elem(char* p, uint32_t v) {
     constexpr int ES = ElemBytes<DT>::value;
-    if constexpr (ES == 4) *reinterpret_cast<uint32_t*>(p) = v;
-    else if constexpr (ES == 2) *reinterpret_cast<uint16_t*>(p) = (uint16_t)v;
-    else *reinterpret_cast<uint8_t*>(p) = (uint8_t)v;
+    if constexpr (ES == 4) *(PCCL_GLOBAL uint32_t*)(p) = v;
+    else if constexpr (ES == 2) *(PCCL_GLOBAL uint16_t*)(p) = (uint16_t)v;
+    else *(PCCL_GLOBAL uint8_t*)(p) = (uint8_t)v;
 }
 template <int DT>
 __device__ __forceinline__ uint32_t elem_op(uint32_t a, uint32_t b, int redop) {
@@ -115,9 +131,6 @@ __device__ __forceinline__ uint32_t elem_op(uint32_t a, uint32_t b, int redop) {
     return word_op<DT>(a, b, redop);
 }
 
-// Every pointer the kernels see is device memory: say so, so that global_* (not flat_*)
-// instructions are selected.
-#define PCCL_GLOBAL __attribute__((address_space(1)))
 typedef const PCCL_GLOBAL u32x4* gvec_cptr;
 typedef PCCL_GLOBAL u32x4* gvec_ptr;
 __device__ __forceinline__ u32x4 ldv(const char* p) { return *(gvec_cptr)(p); }
@@ -249,8 +262,8 @@ __global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int i
     for (int64_t w = blockIdx.x; w < total; w += gridDim.x) {
         int item = item_begin + (int)(w / subs);
         int64_t sub = w % subs;
-        int opi = L.item_op[item];
-        DevStepOp op = L.ops[opi];
+        int opi = as_const(L.item_op)[item];
+        DevStepOp op = load_const(L.ops + opi);
         int64_t t0 = (int64_t)(item - op.first_item) * L.tile_elems;
         int64_t tcnt = op.size - t0 < L.tile_elems ? op.size - t0 : L.tile_elems;
         int64_t e0 = t0 + sub * SUB_ELEMS;
@@ -299,12 +312,12 @@ __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, 
         const int item = s_item;
         __syncthreads();
         if (item >= L.num_items || item < 0) break;
-        const int opi = L.item_op[item];
-        const DevStepOp op = L.ops[opi];
+        const int opi = as_const(L.item_op)[item];
+        const DevStepOp op = load_const(L.ops + opi);
         // wait: thread t watches items t, t+256, ... of each predecessor
         for (int k = 0; k < op.ndeps; ++k) {
-            const int d = L.deps[op.dep_start + k];
-            const int first = L.ops[d].first_item, nt = L.ops[d].ntiles;
+            const int d = as_const(L.deps)[op.dep_start + k];
+            const int first = as_const(L.ops)[d].first_item, nt = as_const(L.ops)[d].ntiles;
             for (int t = tid; t < nt; t += kThreads) {
                 int nap = 1;
                 while (__hip_atomic_load(&flags[first + t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != L.epoch) {
@@ -365,7 +378,8 @@ __device__ __forceinline__ ColInstrDev unpack_instr(uint64_t w) {
 }
 
 template <int DT, int U, bool NT>
-__device__ __forceinline__ void column_tile(const uint64_t* prog, int prog_len, char* const* s_ptr, int64_t vfirst, int tid) {
+__device__ __forceinline__ void column_tile(const PCCL_CONST uint64_t* prog, int prog_len, const RankPtrs& s_ptr_tab, int64_t vfirst, int tid) {
+    char* const* s_ptr = s_ptr_tab.p;   // kernel arguments: uniform indices become scalar loads
     int64_t off[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) off[u] = (vfirst + (int64_t)u * kThreads + tid) * 16;
@@ -412,10 +426,8 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
     constexpr int64_t TILE_V = (int64_t)kThreads * U;
-    __shared__ char* s_ptr[2 * kMaxR];
+    char* const* s_ptr = ptrs.p;   // read straight from the kernel-argument segment (scalar loads)
     const int tid = threadIdx.x;
-    if (tid < 2 * kMaxR) s_ptr[tid] = ptrs.p[tid];
-    __syncthreads();
 
     // Workgroup b runs on XCD b % 8 (round-robin dispatch): give every XCD one contiguous slab of
     // the tile space so that its L2 and TLBs stream through neighbouring addresses.
@@ -428,18 +440,18 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
         int lo = 0, hi = L.num_segs;
         while (hi - lo > 1) {
             int mid = (lo + hi) >> 1;
-            if (L.segs[mid].first_tile <= tile) lo = mid; else hi = mid;
+            if (as_const(L.segs)[mid].first_tile <= tile) lo = mid; else hi = mid;
         }
-        const DevColSegment seg = L.segs[lo];
+        const DevColSegment seg = load_const(L.segs + lo);
         const int64_t vfirst = seg.first_vec + (tile - seg.first_tile) * TILE_V;
-        const uint64_t* prog = L.instrs + seg.prog_start;
+        const PCCL_CONST uint64_t* prog = as_const(L.instrs) + seg.prog_start;
         const bool interior = vfirst * VE >= seg.start && (vfirst + TILE_V) * VE <= seg.end;
         if (interior) {
             // A segment whose every load is a first touch and whose every live store is final is
             // pure streaming: run it with non-temporal accesses throughout (a separate loop
             // instance, so the cache-policy hints cannot be merged away with the cached forms).
-            if (seg.streaming) column_tile<DT, U, true>(prog, seg.prog_len, s_ptr, vfirst, tid);
-            else column_tile<DT, U, false>(prog, seg.prog_len, s_ptr, vfirst, tid);
+            if (seg.streaming) column_tile<DT, U, true>(prog, seg.prog_len, ptrs, vfirst, tid);
+            else column_tile<DT, U, false>(prog, seg.prog_len, ptrs, vfirst, tid);
         } else {
             // edge tile: vectors may be cut by the segment boundary or lie outside it
             for (int64_t v = vfirst + tid; v < vfirst + TILE_V; v += kThreads) {
