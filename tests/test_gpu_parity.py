@@ -112,10 +112,9 @@ def test_reduce_scatter_and_allgather(engine_factory, mode, channels, fuse):
             if channels == 1:
                 assert bits_equal(got[r], torch.cat(parts)), f"rank {r}"
             else:
-                # with two channels the graph gathers per-channel pieces of the staged buffer, parts of
-                # which were never written by anyone: compare only what the oracle's zero-initialised
-                # buffers define identically, i.e. everything (the engine's buffers start zeroed too
-                # only when fresh), so restrict to positions some rank contributed
+                # with two channels the graph gathers, per channel, piece q from rank q; only where
+                # that piece lies inside the chunk rank q staged is its content defined by the
+                # inputs (elsewhere it is whatever the rank buffer held), so compare those pieces
                 per_ch, per_rank = n // channels, n // channels // world
                 for c in range(channels):
                     for q in range(world):
