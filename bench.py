@@ -145,6 +145,8 @@ def main() -> int:
     ap.add_argument("--channels", type=int, default=CHANNELS)
     ap.add_argument("--vecs-per-thread", type=int, default=0)
     ap.add_argument("--num-blocks", type=int, default=-1)
+    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
+                    help="engine option to set before the run (e.g. lds_slots=0, slot_threads=128); repeatable")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--gpu-inputs", action="store_true",
@@ -176,6 +178,9 @@ def main() -> int:
         eng.set_option("vecs_per_thread", args.vecs_per_thread)
     if args.num_blocks >= 0:
         eng.set_option("num_blocks", args.num_blocks)
+    for kv in args.option:
+        key, _, val = kv.partition("=")
+        eng.set_option(key, val)
     info = eng.op_info("bench")
     alg_bytes = info["algorithmic_bytes"]
     log(f"program: {info}")

@@ -189,7 +189,10 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * "timing" = "0" | "1" (record HIP events around the program); "vecs_per_thread" = 1 | 2 | 4;
  * "step_tile_bytes"; "wait_timeout_ms" (how long a persistent launch waits for a predecessor);
  * "fuse_staging" = "1" | "0" (allreduce-type calls in column mode read the input tensors and write
- * the output tensors directly instead of staging through the engine's rank buffers). */
+ * the output tensors directly instead of staging through the engine's rank buffers);
+ * "lds_slots" = "1" | "0" (column runner keeps values it re-reads in per-thread LDS slots, so each
+ * rank buffer is read and written at most once per position; "0" re-reads them through memory);
+ * "slot_threads" = 0 | 64 | 128 | 256 (workgroup size of that runner, 0 = from the rank count). */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
 
 /* Engine::exeOp / exeOpAsync (reference csrc/engine_c.cc:269-560): for every virtual rank r copy

@@ -199,9 +199,10 @@ struct OpEntry {
     std::vector<std::unique_ptr<RankGraph>> graphs;
     bool linked = false;
     Program prog;
-    DevBuf segs, direct_segs, instrs, fifo, step_ops, step_deps, item_op, state;
+    DevBuf segs, direct_segs, instrs, pre, step_ops, step_deps, item_op, state;
     int64_t total_tiles = 0, direct_tiles = 0;
     int vecs_per_thread = 0;
+    int slot_threads = 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool timed = false;
     bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
@@ -209,7 +210,7 @@ struct OpEntry {
     uint32_t ticket_base = 0;             // persistent runner: tickets consumed so far
     std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
     void release() {
-        segs.release(); direct_segs.release(); instrs.release(); fifo.release(); step_ops.release(); step_deps.release();
+        segs.release(); direct_segs.release(); instrs.release(); pre.release(); step_ops.release(); step_deps.release();
         item_op.release(); state.release();
         if (ev0) (void)hipEventDestroy(ev0);
         if (ev1) (void)hipEventDestroy(ev1);
@@ -234,7 +235,9 @@ struct pccl_hip_ctx {
     int vecs_per_thread = 1;
     bool check_races = true;
     bool timing = false;
-    int fifo_depth = 0;
+    bool lds_slots = true;                // column runner keeps re-read values in LDS slots
+    int slot_threads = 0;                 // slot runner workgroup size (0: chosen from the rank count)
+    bool slot_direct = true;              // slot runner fetches first touches straight into LDS
     int64_t step_tile_bytes = 128 * 1024;
     bool fuse_staging = true;             // run staged calls on the caller's tensors when possible
     int wait_timeout_ms = 2000;           // a persistent launch gives up on a dependency after this long
@@ -264,7 +267,6 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
     for (int r = 0; r < ctx->R; ++r) gs.push_back(e.graphs[r].get());
     LinkOptions opt;
     opt.check_races = ctx->check_races;
-    opt.fifo_depth = ctx->fifo_depth;
     opt.step_tile_bytes = ctx->step_tile_bytes;
     e.prog = link_program(gs, opt);
     const Program& P = e.prog;
@@ -274,7 +276,11 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
 
     // column plans (in place, and direct = staging fused into the program)
     if (P.position_aligned) {
-        const int64_t tile_v = 256 * (int64_t)e.vecs_per_thread;
+        // slot runner: one vector per thread and R 16-byte slots per thread; keep a workgroup's
+        // slots within 32 KiB so that several workgroups share a CU
+        e.slot_threads = 0;
+        if (ctx->lds_slots) e.slot_threads = ctx->slot_threads > 0 ? ctx->slot_threads : ctx->R <= 8 ? 256 : ctx->R <= 16 ? 128 : 64;
+        const int64_t tile_v = e.slot_threads > 0 ? e.slot_threads : 256 * (int64_t)e.vecs_per_thread;
         auto device_segments = [&](const std::vector<ColSegment>& segs, int64_t* total) {
             std::vector<DevColSegment> ds(segs.size());
             int64_t tiles = 0;
@@ -287,11 +293,11 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
                 d.first_tile = tiles;
                 tiles += (last_vec - d.first_vec + 1 + tile_v - 1) / tile_v;
                 d.prog_start = s.prog_start; d.prog_len = s.prog_len;
-                d.fifo_start = s.fifo_start; d.fifo_len = s.fifo_len;
+                d.pre_start = s.pre_start; d.pre_words = s.pre_words;
                 d.streaming = 1; d.pad_ = 0;
                 for (int k = 0; k < s.prog_len; ++k) {
                     const ColInstr& in = P.col_instrs[s.prog_start + k];
-                    if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || in.store == 1) d.streaming = 0;
+                    if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || (in.store & STORE_KIND) == 1) d.streaming = 0;
                 }
             }
             *total = tiles;
@@ -304,7 +310,7 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
             e.direct_segs.upload(dd.data(), dd.size() * sizeof(DevColSegment));
         }
         e.instrs.upload(P.col_instrs.data(), P.col_instrs.size() * sizeof(ColInstr));
-        e.fifo.upload(P.col_fifo.data(), P.col_fifo.size());
+        e.pre.upload(P.col_pre.data(), P.col_pre.size() * sizeof(uint64_t));
     }
     // stepwise plan
     {
@@ -368,7 +374,8 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
     if (column) {
         ColumnLaunch L{};
         L.segs = (const DevColSegment*)e.segs.p; L.num_segs = (int)P.segs.size();
-        L.instrs = (const uint64_t*)e.instrs.p; L.fifo = (const uint8_t*)e.fifo.p;
+        L.instrs = (const uint64_t*)e.instrs.p; L.pre = (const uint64_t*)e.pre.p;
+        L.slot_threads = e.slot_threads; L.num_ranks = ctx->R; L.slot_direct = ctx->slot_direct;
         L.total_tiles = e.total_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
         L.num_blocks = ctx->num_blocks;
         rc = launch_column(L, ptrs, stream);
@@ -432,7 +439,8 @@ bool run_direct(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
     if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
     ColumnLaunch L{};
     L.segs = (const DevColSegment*)e.direct_segs.p; L.num_segs = (int)P.direct_segs.size();
-    L.instrs = (const uint64_t*)e.instrs.p; L.fifo = (const uint8_t*)e.fifo.p;
+    L.instrs = (const uint64_t*)e.instrs.p; L.pre = (const uint64_t*)e.pre.p;
+    L.slot_threads = e.slot_threads; L.num_ranks = ctx->R; L.slot_direct = ctx->slot_direct;
     L.total_tiles = e.direct_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
     L.num_blocks = ctx->num_blocks;
     int rc = launch_column(L, ptrs, stream);
@@ -550,7 +558,14 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             int u = std::atoi(value);
             if (u != 1 && u != 2 && u != 4) return fail(PCCL_ERR_INVALID, "vecs_per_thread must be 1, 2 or 4");
             ctx->vecs_per_thread = u; relink = true;
-        } else if (k == "fifo_depth") { ctx->fifo_depth = std::atoi(value); relink = true; }
+        } else if (k == "slot_direct") ctx->slot_direct = std::atoi(value) != 0;
+        else if (k == "lds_slots") { ctx->lds_slots = std::atoi(value) != 0; relink = true; }
+        else if (k == "slot_threads") {
+            int t = std::atoi(value);
+            if (t != 0 && t != 64 && t != 128 && t != 256) return fail(PCCL_ERR_INVALID, "slot_threads must be 0 (automatic), 64, 128 or 256");
+            if ((size_t)t * ctx->R * 16 > 64 * 1024) return fail(PCCL_ERR_INVALID, "slot_threads x ranks x 16 bytes exceeds the 64 KiB of LDS a workgroup may use");
+            ctx->slot_threads = t; relink = true;
+        }
         else if (k == "step_tile_bytes") {
             int64_t b = std::atoll(value);
             if (b < 4096 || b % 4096) return fail(PCCL_ERR_INVALID, "step_tile_bytes must be a positive multiple of 4096");
@@ -692,6 +707,10 @@ int pccl_hip_op_info(pccl_hip_ctx* ctx, const char* name, pccl_program_info* out
         OpEntry& e = find_entry(ctx, name);
         link_entry(ctx, e);
         fill_info(e.prog, out);
+        if (e.slot_threads > 0) {   // the traffic of the runner this context would launch
+            out->column_load_bytes = e.prog.slot_load_bytes;
+            out->column_store_bytes = e.prog.slot_store_bytes;
+        }
         return 0;
     });
 }

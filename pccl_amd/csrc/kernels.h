@@ -19,7 +19,7 @@ struct DevColSegment {
     int64_t first_vec;       // start / vector elems
     int64_t first_tile;      // prefix sum of tiles
     int32_t prog_start, prog_len;
-    int32_t fifo_start, fifo_len;
+    int32_t pre_start, pre_words;   // first-touch rank list, 8 ranks per 64-bit word (0xFF = none)
     int32_t streaming;       // 1: every load is a first touch and every live store is final
     int32_t pad_;
 };
@@ -43,11 +43,15 @@ struct ColumnLaunch {
     const DevColSegment* segs;
     int32_t num_segs;
     const uint64_t* instrs;   // ColInstr words
-    const uint8_t* fifo;
+    const uint64_t* pre;      // first-touch rank lists of the segments
     int64_t total_tiles;
     int32_t dtype;
-    int32_t vecs_per_thread;  // 1, 2 or 4
+    int32_t vecs_per_thread;  // 1, 2 or 4 (register runner)
     int32_t num_blocks;       // 0: one workgroup per tile
+    int32_t slot_threads;     // 0: register runner (re-read values go through memory);
+                              // 64, 128 or 256: workgroup size of the slot runner (re-read values in LDS)
+    int32_t num_ranks;        // slot runner: LDS slots per thread
+    int32_t slot_direct;      // slot runner: 1 = first touches are loaded straight into LDS
 };
 
 struct StepwiseLaunch {

@@ -42,11 +42,11 @@ __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
 
 __device__ __forceinline__ uint32_t f32_op(uint32_t ua, uint32_t ub, int redop) {
-    float a = as_f32(ua), b = as_f32(ub), r;
-    if (redop == PCCL_SUM) r = a + b;
-    else if (redop == PCCL_MAX) r = (a != a || b != b) ? as_f32(0x7FFFFFFFu) : (a > b ? a : b);
-    else r = (a != a || b != b) ? as_f32(0x7FFFFFFFu) : (a < b ? a : b);
-    return (r != r) ? 0x7FFFFFFFu : as_u32(r);
+    const float a = as_f32(ua), b = as_f32(ub);
+    if (redop == PCCL_SUM) { const float r = a + b; return (r != r) ? 0x7FFFFFFFu : as_u32(r); }
+    // one unordered compare, one ordered compare, two selects on the bit patterns
+    const uint32_t pick = redop == PCCL_MAX ? (a > b ? ua : ub) : (a < b ? ua : ub);
+    return __builtin_isunordered(a, b) ? 0x7FFFFFFFu : pick;
 }
 
 // float -> bf16 bits in the HIGH half of the result, round to nearest even, canonical NaN
@@ -414,9 +414,52 @@ __device__ __forceinline__ void column_tile(const PCCL_CONST uint64_t* prog, int
 #pragma unroll
             for (int u = 0; u < U; ++u) acc[u] = a[u];
         }
-        if (in.store) {
+        if (in.store & 3) {
 #pragma unroll
             for (int u = 0; u < U; ++u) { if (NT) stv_nt(self + off[u], acc[u]); else stv(self + off[u], acc[u]); }
+        }
+    }
+}
+
+// A tile that the segment boundary cuts: whole vectors inside the segment run the program on
+// 16-byte accesses, cut vectors element by element; every value goes through memory.
+template <int DT>
+__device__ __forceinline__ void column_edge_tile(const DevColSegment& seg, const PCCL_CONST uint64_t* prog, const RankPtrs& ptrs,
+                                                 int64_t vfirst, int64_t tile_v, int tid, int nthreads) {
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int VE = 16 / ES;
+    char* const* s_ptr = ptrs.p;
+    for (int64_t v = vfirst + tid; v < vfirst + tile_v; v += nthreads) {
+        int64_t e0 = v * VE, e1 = e0 + VE;
+        if (e0 < seg.start) e0 = seg.start;
+        if (e1 > seg.end) e1 = seg.end;
+        if (e0 >= e1) continue;
+        if (e1 - e0 == VE) {
+            int64_t o = v * 16;
+            u32x4 acc = u32x4{0, 0, 0, 0};
+            for (int k = 0; k < seg.prog_len; ++k) {
+                const ColInstrDev in = unpack_instr(prog[k]);
+                u32x4 a = in.a_src == 2 ? acc : ldv(s_ptr[in.peer + (in.a_first ? kMaxR : 0)] + o);
+                if (in.b_src != 0) {
+                    u32x4 b = in.b_src == 2 ? acc : ldv(s_ptr[in.self + (in.b_first ? kMaxR : 0)] + o);
+                    acc = vec_op<DT>(a, b, in.redop);
+                } else acc = a;
+                if (in.store & 3) stv(s_ptr[in.self] + o, acc);
+            }
+        } else {
+            for (int64_t e = e0; e < e1; ++e) {
+                int64_t o = e * ES;
+                uint32_t acc = 0;
+                for (int k = 0; k < seg.prog_len; ++k) {
+                    const ColInstrDev in = unpack_instr(prog[k]);
+                    uint32_t a = in.a_src == 2 ? acc : load_elem<DT>(s_ptr[in.peer + (in.a_first ? kMaxR : 0)] + o);
+                    if (in.b_src != 0) {
+                        uint32_t b = in.b_src == 2 ? acc : load_elem<DT>(s_ptr[in.self + (in.b_first ? kMaxR : 0)] + o);
+                        acc = elem_op<DT>(a, b, in.redop);
+                    } else acc = a;
+                    if (in.store & 3) store_elem<DT>(s_ptr[in.self] + o, acc);
+                }
+            }
         }
     }
 }
@@ -426,7 +469,6 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
     constexpr int64_t TILE_V = (int64_t)kThreads * U;
-    char* const* s_ptr = ptrs.p;   // read straight from the kernel-argument segment (scalar loads)
     const int tid = threadIdx.x;
 
     // Workgroup b runs on XCD b % 8 (round-robin dispatch): give every XCD one contiguous slab of
@@ -453,39 +495,103 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
             if (seg.streaming) column_tile<DT, U, true>(prog, seg.prog_len, ptrs, vfirst, tid);
             else column_tile<DT, U, false>(prog, seg.prog_len, ptrs, vfirst, tid);
         } else {
-            // edge tile: vectors may be cut by the segment boundary or lie outside it
-            for (int64_t v = vfirst + tid; v < vfirst + TILE_V; v += kThreads) {
-                int64_t e0 = v * VE, e1 = e0 + VE;
-                if (e0 < seg.start) e0 = seg.start;
-                if (e1 > seg.end) e1 = seg.end;
-                if (e0 >= e1) continue;
-                if (e1 - e0 == VE) {
-                    int64_t o = v * 16;
-                    u32x4 acc = u32x4{0, 0, 0, 0};
-                    for (int k = 0; k < seg.prog_len; ++k) {
-                        const ColInstrDev in = unpack_instr(prog[k]);
-                        u32x4 a = in.a_src == 2 ? acc : ldv(s_ptr[in.peer + (in.a_first ? kMaxR : 0)] + o);
-                        if (in.b_src != 0) {
-                            u32x4 b = in.b_src == 2 ? acc : ldv(s_ptr[in.self + (in.b_first ? kMaxR : 0)] + o);
-                            acc = vec_op<DT>(a, b, in.redop);
-                        } else acc = a;
-                        if (in.store) stv(s_ptr[in.self] + o, acc);
-                    }
-                } else {
-                    for (int64_t e = e0; e < e1; ++e) {
-                        int64_t o = e * ES;
-                        uint32_t acc = 0;
-                        for (int k = 0; k < seg.prog_len; ++k) {
-                            const ColInstrDev in = unpack_instr(prog[k]);
-                            uint32_t a = in.a_src == 2 ? acc : load_elem<DT>(s_ptr[in.peer + (in.a_first ? kMaxR : 0)] + o);
-                            if (in.b_src != 0) {
-                                uint32_t b = in.b_src == 2 ? acc : load_elem<DT>(s_ptr[in.self + (in.b_first ? kMaxR : 0)] + o);
-                                acc = elem_op<DT>(a, b, in.redop);
-                            } else acc = a;
-                            if (in.store) store_elem<DT>(s_ptr[in.self] + o, acc);
-                        }
-                    }
-                }
+            column_edge_tile<DT>(seg, prog, ptrs, vfirst, TILE_V, tid, kThreads);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------- column runner, values kept in LDS
+//
+// The same segment programs, with every value the program reads more than once kept on chip:
+// each thread owns one 16-byte LDS slot per rank (slot r of thread t holds the current value of
+// rank r at the thread's position).  A tile first fetches every rank the program reads by first
+// touch - up to 8 independent streaming loads in flight per thread - into the slots, then runs
+// the program on the slots (MEM operands read a slot, a write that is read back later goes to its
+// slot) and sends only the last value of each rank to memory.  Each rank buffer is therefore read
+// at most once and written at most once per position whatever the shape of the program (chains,
+// halving-doubling butterflies, trees).  A thread only ever touches its own slots, so no barrier
+// is needed.  Results are bit-identical to the op-by-op execution for the same reason as above.
+
+template <int N>
+__device__ __forceinline__ void slot_fetch(uint64_t word, const RankPtrs& ptrs, u32x4* slots, int T, int tid, int64_t off) {
+    u32x4 v[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = ldv_nt(ptrs.p[kMaxR + (int)((word >> (8 * i)) & 0xFF)] + off);
+#pragma unroll
+    for (int i = 0; i < N; ++i) slots[(int)((word >> (8 * i)) & 0xFF) * T + tid] = v[i];
+}
+
+// The same fetch without staging registers: a 128-bit load that the memory pipeline writes
+// straight into LDS (lane l of the wave lands at the wave-uniform LDS base + 16 l), so a thread
+// can have every first-touch load of its program in flight at once.
+__device__ __forceinline__ void slot_fetch_direct(int rank, const RankPtrs& ptrs, u32x4* slots, int T, int tid, int64_t off) {
+    const char* g = ptrs.p[kMaxR + rank] + off;
+    u32x4* wave_base = slots + rank * T + (tid & ~63);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                     (__attribute__((address_space(3))) void*)wave_base, 16, 0, 2 /* nt */);
+}
+
+template <int DT, bool DIRECT>
+__global__ __launch_bounds__(kThreads) void column_slot_kernel(ColumnLaunch L, RankPtrs ptrs) {
+    extern __shared__ u32x4 slots[];
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int VE = 16 / ES;
+    const int T = blockDim.x;
+    const int tid = threadIdx.x;
+    const int64_t tile_v = T;
+    constexpr int kXcds = 8;
+    const int64_t slab = (L.total_tiles + kXcds - 1) / kXcds;
+    for (int64_t w = blockIdx.x; w < slab * kXcds; w += gridDim.x) {
+        const int64_t tile = (w % kXcds) * slab + w / kXcds;
+        if (tile >= L.total_tiles) continue;
+        int lo = 0, hi = L.num_segs;
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (as_const(L.segs)[mid].first_tile <= tile) lo = mid; else hi = mid;
+        }
+        const DevColSegment seg = load_const(L.segs + lo);
+        const int64_t vfirst = seg.first_vec + (tile - seg.first_tile) * tile_v;
+        const PCCL_CONST uint64_t* prog = as_const(L.instrs) + seg.prog_start;
+        const bool interior = vfirst * VE >= seg.start && (vfirst + tile_v) * VE <= seg.end;
+        if (!interior) {
+            column_edge_tile<DT>(seg, prog, ptrs, vfirst, tile_v, tid, T);
+            continue;
+        }
+        const int64_t off = (vfirst + tid) * 16;
+        const PCCL_CONST uint64_t* pre = as_const(L.pre) + seg.pre_start;
+        if constexpr (DIRECT) {
+            for (int i = 0; i < seg.pre_words; ++i) {
+                uint64_t word = pre[i];
+                for (int j = 0; j < 8 && (word & 0xFF) != 0xFF; ++j, word >>= 8)
+                    slot_fetch_direct((int)(word & 0xFF), ptrs, slots, T, tid, off);
+            }
+            // the loads above write LDS behind the compiler's back: wait for all of them before
+            // any slot is read, and keep the slot reads below this point
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else {
+            for (int i = 0; i < seg.pre_words; ++i) {
+                uint64_t word = pre[i];
+                if ((word >> 56) != 0xFF) { slot_fetch<8>(word, ptrs, slots, T, tid, off); continue; }
+                if (((word >> 24) & 0xFF) != 0xFF) { slot_fetch<4>(word, ptrs, slots, T, tid, off); word >>= 32; }
+                if (((word >> 8) & 0xFF) != 0xFF) { slot_fetch<2>(word, ptrs, slots, T, tid, off); word >>= 16; }
+                if ((word & 0xFF) != 0xFF) slot_fetch<1>(word, ptrs, slots, T, tid, off);
+            }
+        }
+        u32x4 acc = u32x4{0, 0, 0, 0};
+        // programs are padded to a multiple of 4 instructions: one scalar load brings in four
+        for (int k = 0; k < seg.prog_len; k += 4) {
+            const uint64_t w[4] = {prog[k], prog[k + 1], prog[k + 2], prog[k + 3]};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const ColInstrDev in = unpack_instr(w[j]);
+                const u32x4 a = in.a_src == 2 ? acc : slots[in.peer * T + tid];
+                if (in.b_src != 0) {
+                    const u32x4 b = in.b_src == 2 ? acc : slots[in.self * T + tid];
+                    acc = vec_op<DT>(a, b, in.redop);
+                } else acc = a;
+                const int kind = in.store & 3;
+                if (kind == 1) slots[in.self * T + tid] = acc;
+                if (kind == 2 || (kind == 1 && (in.store & 4))) stv_nt(ptrs.p[in.self] + off, acc);
             }
         }
     }
@@ -517,6 +623,12 @@ static int launch_column_dt(const ColumnLaunch& L, const RankPtrs& ptrs, hipStre
     if (L.num_blocks > 0 && grid > L.num_blocks) grid = L.num_blocks;
     if (grid > (1 << 30)) grid = 1 << 30;
     if (grid <= 0) return 0;
+    if (L.slot_threads > 0) {
+        const size_t lds = (size_t)L.num_ranks * L.slot_threads * 16;
+        if (L.slot_direct) hipLaunchKernelGGL((column_slot_kernel<DT, true>), dim3((unsigned)grid), dim3(L.slot_threads), lds, s, L, ptrs);
+        else hipLaunchKernelGGL((column_slot_kernel<DT, false>), dim3((unsigned)grid), dim3(L.slot_threads), lds, s, L, ptrs);
+        return (int)hipGetLastError();
+    }
     switch (L.vecs_per_thread) {
         case 1: hipLaunchKernelGGL((column_kernel<DT, 1>), dim3((unsigned)grid), dim3(kThreads), 0, s, L, ptrs); break;
         case 2: hipLaunchKernelGGL((column_kernel<DT, 2>), dim3((unsigned)grid), dim3(kThreads), 0, s, L, ptrs); break;

@@ -41,6 +41,56 @@ constexpr size_t kPairLimit = 20000000;   // access pairs examined by the race c
 
 }  // namespace
 
+// Last step of building a segment's column program: mark the last write of every rank and list
+// the ranks the program reads by first touch (what a runner that keeps re-read values on chip
+// has to fetch up front).
+static void finish_column_program(Program& P, ColSegment& seg, std::vector<ColInstr>& prog) {
+    uint64_t seen = 0;
+    for (size_t n = prog.size(); n-- > 0;) {
+        if (!(seen >> prog[n].self & 1)) prog[n].store |= STORE_LAST;
+        seen |= 1ull << prog[n].self;
+    }
+    std::vector<uint8_t> pre;
+    uint64_t listed = 0;
+    auto want = [&](uint8_t r) { if (!(listed >> r & 1)) { listed |= 1ull << r; pre.push_back(r); } };
+    for (const ColInstr& in : prog) {
+        if (in.a_src == SRC_MEM && in.a_first) want(in.peer);
+        if (in.b_src == SRC_MEM && in.b_first) want(in.self);
+    }
+    seg.pre_start = (int)P.col_pre.size();
+    for (size_t i = 0; i < pre.size(); i += 8) {
+        uint64_t w = ~0ull;
+        for (size_t j = i; j < pre.size() && j < i + 8; ++j) w = (w & ~(0xFFull << (8 * (j - i)))) | ((uint64_t)pre[j] << (8 * (j - i)));
+        P.col_pre.push_back(w);
+    }
+    seg.pre_words = (int)P.col_pre.size() - seg.pre_start;
+    // pad with no-ops (acc = acc, nothing stored) so that a runner may read four instructions at
+    // a time; programs start at multiples of four words because every program is padded
+    ColInstr nop{};
+    nop.a_src = SRC_ACC; nop.b_src = SRC_NONE;
+    while (prog.size() % 4) prog.push_back(nop);
+    seg.prog_len = (int)prog.size();
+}
+
+// Memory traffic of one segment under the two ways of running its program: every MEM operand
+// loaded and every live store written (re-read values go through memory), or first touches
+// fetched once and only final values written (re-read values stay on chip).
+static void count_column_traffic(const Program& P, const ColSegment& seg, int es, int64_t* loads, int64_t* stores,
+                                 int64_t* slot_loads, int64_t* slot_stores) {
+    const int64_t bytes = (seg.end - seg.start) * es;
+    for (int k = 0; k < seg.prog_len; ++k) {
+        const ColInstr& in = P.col_instrs[seg.prog_start + k];
+        const int kind = in.store & STORE_KIND;
+        if (in.a_src == SRC_MEM) *loads += bytes;
+        if (in.b_src == SRC_MEM) *loads += bytes;
+        if (kind) *stores += bytes;
+        if (kind == 2 || (kind == 1 && (in.store & STORE_LAST))) *slot_stores += bytes;
+    }
+    for (int w = 0; w < seg.pre_words; ++w)
+        for (int j = 0; j < 8; ++j)
+            if ((P.col_pre[seg.pre_start + w] >> (8 * j) & 0xFF) != 0xFF) *slot_loads += bytes;
+}
+
 Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOptions& opt) {
     const int R = (int)graphs.size();
     if (R <= 0 || R > PCCL_HIP_MAX_VRANKS) throw Error{PCCL_ERR_INVALID, "number of virtual ranks must be 1.." + std::to_string(PCCL_HIP_MAX_VRANKS)};
@@ -341,7 +391,6 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
             ColSegment seg;
             seg.start = cuts[i]; seg.end = cuts[i + 1];
             seg.prog_start = (int)P.col_instrs.size();
-            seg.fifo_start = (int)P.col_fifo.size();
             // build + optimise the column program
             std::vector<ColInstr> prog;
             uint64_t written = 0;  // ranks an earlier instruction of this program wrote
@@ -376,27 +425,13 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                              (prog[m].b_src == SRC_MEM && prog[m].self == prog[n].self);
                 if (!reread) prog[n].store = 2;
             }
-            // first-touch loads may be issued early through the FIFO (nothing before them writes
-            // the location, so any earlier issue point reads the same value)
-            if (opt.fifo_depth > 0)
-                for (auto& in : prog) {
-                    if (in.a_src == SRC_MEM && in.a_first) { in.a_src = SRC_FIFO; P.col_fifo.push_back(in.peer); }
-                    if (in.b_src == SRC_MEM && in.b_first) { in.b_src = SRC_FIFO; P.col_fifo.push_back(in.self); }
-                }
             seg.prog_len = (int)prog.size();
-            seg.fifo_len = (int)P.col_fifo.size() - seg.fifo_start;
+            finish_column_program(P, seg, prog);
             P.col_instrs.insert(P.col_instrs.end(), prog.begin(), prog.end());
             P.segs.push_back(seg);
         }
-        for (auto& seg : P.segs) {
-            int64_t n = seg.end - seg.start;
-            for (int k = 0; k < seg.prog_len; ++k) {
-                const ColInstr& in = P.col_instrs[seg.prog_start + k];
-                if (in.a_src == SRC_MEM || in.a_src == SRC_FIFO) P.column_load_bytes += n * es;
-                if (in.b_src == SRC_MEM || in.b_src == SRC_FIFO) P.column_load_bytes += n * es;
-                if (in.store) P.column_store_bytes += n * es;
-            }
-        }
+        for (auto& seg : P.segs)
+            count_column_traffic(P, seg, es, &P.column_load_bytes, &P.column_store_bytes, &P.slot_load_bytes, &P.slot_store_bytes);
 
         // ---- direct plan: the same programs with the caller's input tensors as the source of
         // every first-touch load and the output tensors as the destination of every store, so
@@ -444,6 +479,8 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                 if (base)
                     for (int k = 0; k < base->prog_len && valid; ++k) {
                         ColInstr in = P.col_instrs[base->prog_start + k];
+                        in.store &= STORE_KIND;
+                        if (in.a_src == SRC_ACC && in.b_src == SRC_NONE && !in.store) continue;   // padding
                         if (in.a_src == SRC_MEM) valid = in.a_first ? in_window(in.peer) : out_window(in.peer);
                         if (valid && in.b_src == SRC_MEM) valid = in.b_first ? in_window(in.self) : out_window(in.self);
                         if (in.store && !out_window(in.self)) {
@@ -475,20 +512,14 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                 ColSegment d;
                 d.start = a; d.end = b;
                 d.prog_start = (int)P.col_instrs.size(); d.prog_len = (int)prog.size();
+                prev_prog = prog;                      // compared before the finishing marks are added
+                finish_column_program(P, d, prog);
                 P.col_instrs.insert(P.col_instrs.end(), prog.begin(), prog.end());
                 P.direct_segs.push_back(d);
-                prev_prog.swap(prog);
             }
             if (!valid) P.direct_segs.clear();
-            for (auto& seg : P.direct_segs) {
-                int64_t len = seg.end - seg.start;
-                for (int k = 0; k < seg.prog_len; ++k) {
-                    const ColInstr& in = P.col_instrs[seg.prog_start + k];
-                    if (in.a_src == SRC_MEM || in.a_src == SRC_FIFO) P.direct_load_bytes += len * es;
-                    if (in.b_src == SRC_MEM || in.b_src == SRC_FIFO) P.direct_load_bytes += len * es;
-                    if (in.store) P.direct_store_bytes += len * es;
-                }
-            }
+            for (auto& seg : P.direct_segs)
+                count_column_traffic(P, seg, es, &P.direct_load_bytes, &P.direct_store_bytes, &P.direct_slot_load_bytes, &P.direct_slot_store_bytes);
         }
     }
     return P;

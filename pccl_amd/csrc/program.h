@@ -24,18 +24,22 @@ struct LinkedOp {
 };
 
 // Operand sources of a column instruction.
-enum : uint8_t { SRC_NONE = 0, SRC_MEM = 1, SRC_ACC = 2, SRC_FIFO = 3 };
+enum : uint8_t { SRC_NONE = 0, SRC_MEM = 1, SRC_ACC = 2 };
+// ColInstr::store: low two bits as documented there; STORE_LAST marks the last write of that rank
+// in the program (its value must reach memory even when a later instruction reads it back).
+enum : uint8_t { STORE_KIND = 3, STORE_LAST = 4 };
 
 // One step of a segment's column program: acc = a (copy) or acc = a (op) b (reduce), then
 // optionally mem[self] = acc.  a is the peer's value, b the own value.
 struct ColInstr {
     uint8_t self;
     uint8_t peer;
-    uint8_t a_src;   // SRC_MEM | SRC_ACC | SRC_FIFO
-    uint8_t b_src;   // SRC_NONE (copy) | SRC_MEM | SRC_ACC | SRC_FIFO
+    uint8_t a_src;   // SRC_MEM | SRC_ACC
+    uint8_t b_src;   // SRC_NONE (copy) | SRC_MEM | SRC_ACC
     uint8_t redop;
-    uint8_t store;   // 0: the write is dead (overwritten before anything reads it from memory),
-                     // 1: written and read back later by this program, 2: final value (streaming store)
+    uint8_t store;   // & STORE_KIND: 0: the write is dead (overwritten before anything reads it from
+                     // memory), 1: written and read back later by this program, 2: final value
+                     // (streaming store); | STORE_LAST: no later instruction writes this rank
     uint8_t a_first; // 1: this load is the first access to (peer, position) in the program
     uint8_t b_first;
 };
@@ -44,7 +48,9 @@ static_assert(sizeof(ColInstr) == 8, "ColInstr is read as one 8-byte word on the
 struct ColSegment {
     int64_t start = 0, end = 0;  // element positions [start, end)
     int32_t prog_start = 0, prog_len = 0;
-    int32_t fifo_start = 0, fifo_len = 0;  // entries in Program::col_fifo (ranks, consumption order)
+    int32_t pre_start = 0, pre_words = 0;  // words in Program::col_pre: the ranks this program reads by
+                                           // first touch, 8 per word (one byte each, 0xFF = none), in
+                                           // program order without repeats
 };
 
 struct StepOpPlan {
@@ -68,11 +74,13 @@ struct Program {
     bool position_aligned = false;
     std::vector<ColSegment> segs;
     std::vector<ColInstr> col_instrs;
-    std::vector<uint8_t> col_fifo;
-    int64_t column_load_bytes = 0, column_store_bytes = 0;
+    std::vector<uint64_t> col_pre;
+    int64_t column_load_bytes = 0, column_store_bytes = 0;   // with values re-read through memory
+    int64_t slot_load_bytes = 0, slot_store_bytes = 0;       // with re-read values kept on chip
     // direct plan (staging fused into the program; valid when non-empty): covers [0, tensor_elems)
     std::vector<ColSegment> direct_segs;
     int64_t direct_load_bytes = 0, direct_store_bytes = 0;
+    int64_t direct_slot_load_bytes = 0, direct_slot_store_bytes = 0;
     std::vector<int64_t> direct_in_start, direct_in_end, direct_out_start, direct_out_end;  // windows per rank
 
     // stepwise plan
@@ -85,7 +93,6 @@ struct Program {
 struct LinkOptions {
     bool check_races = true;
     bool conflict_deps = true;     // order data ops by memory conflicts instead of raw chain order
-    int fifo_depth = 0;            // 0: every first-touch load is SRC_MEM
     int64_t step_tile_bytes = 128 * 1024;
 };
 

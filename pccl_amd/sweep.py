@@ -1,6 +1,7 @@
 """Timing sweep over the benchmark configurations other than the headline one.
 
     python -m pccl_amd.sweep [--config c3|c4|c5|all] [--mode auto|column|stepwise] [--reps N]
+                             [--option KEY=VALUE ...]
 
 Prints one JSON line per measurement: kernel time by HIP events on the launch stream, algorithmic
 bytes (reduce 3*n*esize, copy 2*n*esize summed over the linked program) and GB/s.  Inputs are drawn
@@ -45,12 +46,17 @@ def timed(fn, reps):
     return ms[len(ms) // 2], ms[0]
 
 
+OPTIONS: list = []   # (key, value) engine options applied to every case
+
+
 def run_case(label, world, jsons, make_in, out_elems, mode, reps, inplace):
     eng = Engine(world, 0)
     try:
         for r, j in enumerate(jsons):
             eng.register_operation_json("op", j, r)
         eng.set_option("mode", mode)
+        for key, val in OPTIONS:
+            eng.set_option(key, val)
         info = eng.op_info("op")
         x = make_in()
         if inplace:
@@ -74,7 +80,12 @@ def main() -> int:
     ap.add_argument("--config", default="all")
     ap.add_argument("--mode", default="auto")
     ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
+                    help="engine option for every case (e.g. lds_slots=0); repeatable")
     args = ap.parse_args()
+    for kv in args.option:
+        key, _, val = kv.partition("=")
+        OPTIONS.append((key, val))
     g = torch.Generator(device="cuda").manual_seed(0)
     want = args.config
 
