@@ -31,6 +31,11 @@
  *   NaN results        canonical NaN (0x7FFFFFFF / 0x7FFF), the value PTX add.f32 / add.f16x2 /
  *                      add.bf16x2 produce.  PARITY UNPINNED (no CUDA device to confirm; taken from
  *                      the PTX ISA description of NaN payloads).
+ *   fp8 add            e4m3 / e5m2 widened to f16, one f16 add, narrowed round-to-nearest-even with
+ *                      saturation to the largest finite value (vec.h:272-426).  PINNED over all
+ *                      65,536 operand pairs of both formats by torch CPU: float8 -> float16 views,
+ *                      float16 add, clamp to +-max, float16 -> float8.  NaN results are written as
+ *                      0x7F: PARITY UNPINNED.
  *   copy               memcpy.  PINNED trivially.
  *   signals + runner   counting semaphores.  PINNED by the closed forms of the reference's own
  *                      correctness script (tests/test_correctness.py:142-289) and by brute-force
@@ -49,6 +54,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <stdio.h>
+#include <math.h>
 #ifdef _OPENMP
 #include <omp.h>
 #endif
@@ -168,6 +174,63 @@ static inline float sel_min_f32(float a, float b) {
     return a < b ? a : b;
 }
 
+/* fp8 (reference vec.h:272-426): both operands are widened to f16 (exact), added with one f16
+ * rounding (__hadd2), and narrowed with __nv_cvt_halfraw2_to_fp8x2(..., __NV_SATFINITE, type):
+ * round to nearest even, everything beyond the largest finite value - infinities included -
+ * becomes that value with the sign kept.  E4M3 is the OCP "FN" format (bias 7, no infinities,
+ * S.1111.111 is NaN, largest finite 448); E5M2 is IEEE-like (bias 15, largest finite 57344).
+ * A NaN result is written as 0x7F in both formats: canonical choice, parity unpinned (no CUDA
+ * device to confirm the payload the conversion instruction produces). */
+static inline float fp8_to_f32(uint8_t v, int e5m2) {
+    const int mbits = e5m2 ? 2 : 3, bias = e5m2 ? 15 : 7;
+    const uint32_t sign = (uint32_t)(v & 0x80u) << 24;
+    const int exp = (v & 0x7F) >> mbits, man = v & ((1 << mbits) - 1);
+    if (e5m2) {
+        if (exp == 31) return u2f(sign | (man ? 0x7FC00000u : 0x7F800000u));
+    } else if ((v & 0x7F) == 0x7F) return u2f(sign | 0x7FC00000u);
+    float mag;
+    if (exp == 0) mag = ldexpf((float)man, 1 - bias - mbits);
+    else mag = ldexpf((float)(man | (1 << mbits)), exp - bias - mbits);
+    return sign ? -mag : mag;
+}
+
+static inline uint8_t f32_to_fp8_satfinite(float f, int e5m2) {
+    const int mbits = e5m2 ? 2 : 3, bias = e5m2 ? 15 : 7;
+    const uint8_t maxnorm = e5m2 ? 0x7B : 0x7E;
+    if (f != f) return 0x7F;
+    const uint8_t sign = (f2u(f) >> 31) ? 0x80 : 0x00;
+    const double a = fabs((double)f);
+    const double maxval = e5m2 ? 57344.0 : 448.0;
+    if (a >= maxval) return sign | maxnorm;                 /* saturate (also +-inf) */
+    if (a == 0.0) return sign;
+    int e;
+    (void)frexp(a, &e);                                     /* a = m * 2^e, m in [0.5, 1) */
+    int ue = e - 1;                                         /* a in [2^ue, 2^(ue+1)) */
+    if (ue < 1 - bias) ue = 1 - bias;                       /* subnormal range: fixed quantum */
+    const double quantum = ldexp(1.0, ue - mbits);
+    const double q = a / quantum;                           /* exact: power-of-two scaling */
+    double fl = floor(q);
+    const double rem = q - fl;
+    if (rem > 0.5 || (rem == 0.5 && fmod(fl, 2.0) == 1.0)) fl += 1.0;
+    /* fl is the significand in units of the quantum: in [0, 2^(mbits+1)] */
+    int k = (int)fl;
+    int be = ue + bias;                                     /* biased exponent if normal */
+    if (ue == 1 - bias && k < (1 << mbits)) return sign | (uint8_t)k;          /* subnormal or zero */
+    if (k == (2 << mbits)) { k >>= 1; be += 1; }            /* rounding carried into the exponent */
+    uint8_t out = (uint8_t)((be << mbits) | (k - (1 << mbits)));
+    if (out > maxnorm) out = maxnorm;                       /* cannot happen below maxval; guard */
+    return sign | out;
+}
+
+static inline uint8_t oracle_red_fp8(uint8_t a, uint8_t b, int redop, int e5m2) {
+    const float x = fp8_to_f32(a, e5m2), y = fp8_to_f32(b, e5m2);
+    float r;
+    if (redop == RED_SUM) r = f16_to_f32(f32_to_f16_rne(x + y));   /* = __hadd2 on the widened pair */
+    else if (redop == RED_MAX) r = sel_max_f32(x, y);
+    else r = sel_min_f32(x, y);
+    return f32_to_fp8_satfinite(r, e5m2);
+}
+
 /* ---------------------------------------------------------------- vector ops over a range */
 
 #define LOOP_HDR _Pragma("omp parallel for schedule(static) if (n > 65536)")
@@ -193,12 +256,16 @@ static void reduce_range(int dtype, int redop, const void* a, const void* b, voi
         if (redop == RED_SUM) { LOOP_HDR for (int64_t i = 0; i < n; i++) pc[i] = oracle_add_f16(pa[i], pb[i]); }
         else if (redop == RED_MAX) { LOOP_HDR for (int64_t i = 0; i < n; i++) pc[i] = f32_to_f16_rne(sel_max_f32(f16_to_f32(pa[i]), f16_to_f32(pb[i]))); }
         else { LOOP_HDR for (int64_t i = 0; i < n; i++) pc[i] = f32_to_f16_rne(sel_min_f32(f16_to_f32(pa[i]), f16_to_f32(pb[i]))); }
+    } else if (dtype == DT_F8E4M3 || dtype == DT_F8E5M2) {
+        const uint8_t* pa = a; const uint8_t* pb = b; uint8_t* pc = c;
+        const int e5m2 = dtype == DT_F8E5M2;
+        LOOP_HDR for (int64_t i = 0; i < n; i++) pc[i] = oracle_red_fp8(pa[i], pb[i], redop, e5m2);
     }
 }
 
 /* Exposed for unit tests of the arithmetic alone. */
 int pccl_oracle_reduce(int dtype, int redop, const void* a, const void* b, void* c, int64_t n) {
-    if (dtype == DT_F8E4M3 || dtype == DT_F8E5M2 || pccl_oracle_elem_size(dtype) == 0) {
+    if (pccl_oracle_elem_size(dtype) == 0) {
         snprintf(g_err, sizeof g_err, "reduce: dtype %d not supported by the oracle", dtype);
         return -1;
     }
@@ -299,7 +366,6 @@ int pccl_oracle_run(int R, const int32_t* nops, const oracle_op* const* ops, int
                     if (bad) { snprintf(g_err, sizeof g_err, "rank %d op %d: range outside the %lld-element buffer", r, i, (long long)buf_elems); rc = -1; goto out2; }
                     char* self = bufs[r]; const char* peer = bufs[o->peer];
                     if (o->kind == K_REDUCE) {
-                        if (dtype == DT_F8E4M3 || dtype == DT_F8E5M2) { snprintf(g_err, sizeof g_err, "fp8 reduce is not restated by the oracle"); rc = -1; goto out2; }
                         reduce_range(dtype, o->redop, peer + (int64_t)o->off0 * es, self + (int64_t)o->off1 * es,
                                      self + (int64_t)o->off2 * es, n);
                         st.bytes += 3 * n * es;

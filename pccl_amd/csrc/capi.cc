@@ -730,8 +730,7 @@ int pccl_hip_last_kernel_ms(pccl_hip_ctx* ctx, const char* name, float* ms) {
 int pccl_hip_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream) {
     return guarded([&] {
         if (!a || !b || !c) return fail(PCCL_ERR_INVALID, "null argument");
-        if (dtype != PCCL_F32 && dtype != PCCL_F16 && dtype != PCCL_BF16 && dtype != PCCL_I32)
-            return fail(PCCL_ERR_UNSUPPORTED, "reduce supports float32, float16, bfloat16 and int32");
+        if (dtype < PCCL_F32 || dtype > PCCL_I32) return fail(PCCL_ERR_UNSUPPORTED, "unknown dtype");
         if (redop < PCCL_SUM || redop > PCCL_MIN) return fail(PCCL_ERR_INVALID, "bad reduce operator");
         int es = elem_size(dtype);
         if ((uintptr_t)a % es || (uintptr_t)b % es || (uintptr_t)c % es) return fail(PCCL_ERR_INVALID, "pointers must be aligned to the element size");

@@ -151,8 +151,6 @@ RankGraph load_graph_json(const char* text, size_t len) {
                         if (o.redop < 0)
                             throw Error{PCCL_ERR_UNSUPPORTED, "reduce_op '" + ro->s + "' is not supported (sum, max, min are)"};
                     }
-                    if (g.dtype == PCCL_F8E4M3 || g.dtype == PCCL_F8E5M2)
-                        throw Error{PCCL_ERR_UNSUPPORTED, "reduce on " + dtype_name + " is not implemented by the HIP plugin (copies are)"};
                     check_i32(o.off2, "dst_offset");
                 } else {
                     o.kind = OpKind::Copy;
@@ -257,8 +255,6 @@ RankGraph graph_from_triggers(const pccl_trigger* trig, const pccl_primitive_met
         o.off0 = trig[i].offset_0; o.off1 = trig[i].offset_1; o.off2 = trig[i].offset_2;
         o.size = trig[i].size;
         o.redop = PCCL_SUM;  // the reference runtime has no other operator
-        if (o.kind == OpKind::Reduce && (dt == PCCL_F8E4M3 || dt == PCCL_F8E5M2))
-            throw Error{PCCL_ERR_UNSUPPORTED, "fp8 reduce is not implemented by the HIP plugin"};
         o.channel = meta[i].channel;
         if (o.channel < 0 || o.channel >= PCCL_HIP_MAX_CHANNELS) throw Error{PCCL_ERR_PARSE, "channel out of range"};
         o.num_deps_declared = meta[i].num_dependencies;

@@ -85,6 +85,47 @@ __device__ __forceinline__ uint32_t f16x2_op(uint32_t ua, uint32_t ub, int redop
     return u;
 }
 
+// fp8 (reference vec.h:272-426): widen both operands (exact), add with one f16 rounding, narrow
+// with round-to-nearest-even and saturation to the largest finite value; NaN results are 0x7F.
+// The conversion instructions of gfx950 implement the OCP formats (fp8 = E4M3, bf8 = E5M2); the
+// saturation is done here with a clamp so that it does not depend on the overflow mode bit.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+template <bool E5M2, bool HI>
+__device__ __forceinline__ uint32_t fp8_pair_op(uint32_t x, uint32_t y, uint32_t out, int redop) {
+    constexpr float kMax = E5M2 ? 57344.0f : 448.0f;
+    f32x2 a, b;
+    if constexpr (E5M2) { a = __builtin_amdgcn_cvt_pk_f32_bf8(x, HI); b = __builtin_amdgcn_cvt_pk_f32_bf8(y, HI); }
+    else { a = __builtin_amdgcn_cvt_pk_f32_fp8(x, HI); b = __builtin_amdgcn_cvt_pk_f32_fp8(y, HI); }
+    float r0, r1;
+    if (redop == PCCL_SUM) {
+        // the float sum of two f16-representable values rounds to f16 exactly as their f16 sum
+        r0 = (float)(_Float16)(a.x + b.x);
+        r1 = (float)(_Float16)(a.y + b.y);
+    } else if (redop == PCCL_MAX) {
+        r0 = a.x > b.x ? a.x : b.x; r1 = a.y > b.y ? a.y : b.y;
+    } else {
+        r0 = a.x < b.x ? a.x : b.x; r1 = a.y < b.y ? a.y : b.y;
+    }
+    const bool n0 = (r0 != r0) || __builtin_isunordered(a.x, b.x), n1 = (r1 != r1) || __builtin_isunordered(a.y, b.y);
+    r0 = n0 ? 0.0f : __builtin_fminf(__builtin_fmaxf(r0, -kMax), kMax);
+    r1 = n1 ? 0.0f : __builtin_fminf(__builtin_fmaxf(r1, -kMax), kMax);
+    if constexpr (E5M2) out = __builtin_amdgcn_cvt_pk_bf8_f32(r0, r1, out, HI);
+    else out = __builtin_amdgcn_cvt_pk_fp8_f32(r0, r1, out, HI);
+    constexpr int sh = HI ? 16 : 0;
+    if (n0) out = (out & ~(0xFFu << sh)) | (0x7Fu << sh);
+    if (n1) out = (out & ~(0xFF00u << sh)) | (0x7F00u << sh);
+    return out;
+}
+
+template <bool E5M2>
+__device__ __forceinline__ uint32_t fp8x4_op(uint32_t a, uint32_t b, int redop) {
+    uint32_t out = 0;
+    out = fp8_pair_op<E5M2, false>(a, b, out, redop);
+    out = fp8_pair_op<E5M2, true>(a, b, out, redop);
+    return out;
+}
+
 __device__ __forceinline__ uint32_t i32_op(uint32_t a, uint32_t b, int redop) {
     if (redop == PCCL_SUM) return a + b;
     int x = (int)a, y = (int)b;
@@ -97,7 +138,8 @@ __device__ __forceinline__ uint32_t word_op(uint32_t a, uint32_t b, int redop) {
     else if constexpr (DT == PCCL_I32) return i32_op(a, b, redop);
     else if constexpr (DT == PCCL_BF16) return bf16x2_op(a, b, redop);
     else if constexpr (DT == PCCL_F16) return f16x2_op(a, b, redop);
-    else return a;  // fp8: no reduce (rejected at graph load)
+    else if constexpr (DT == PCCL_F8E4M3) return fp8x4_op<false>(a, b, redop);
+    else return fp8x4_op<true>(a, b, redop);
 }
 
 template <int DT>
@@ -644,7 +686,8 @@ int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
         case PCCL_F16: return launch_column_dt<PCCL_F16>(L, ptrs, s);
         case PCCL_BF16: return launch_column_dt<PCCL_BF16>(L, ptrs, s);
         case PCCL_I32: return launch_column_dt<PCCL_I32>(L, ptrs, s);
-        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_column_dt<PCCL_F8E4M3>(L, ptrs, s);
+        case PCCL_F8E4M3: return launch_column_dt<PCCL_F8E4M3>(L, ptrs, s);
+        case PCCL_F8E5M2: return launch_column_dt<PCCL_F8E5M2>(L, ptrs, s);
         default: return (int)hipErrorInvalidValue;
     }
 }
@@ -690,7 +733,8 @@ int launch_level(const StepwiseLaunch& L, int item_begin, int item_end, const Ra
         case PCCL_F16: return launch_level_dt<PCCL_F16>(L, item_begin, item_end, ptrs, s);
         case PCCL_BF16: return launch_level_dt<PCCL_BF16>(L, item_begin, item_end, ptrs, s);
         case PCCL_I32: return launch_level_dt<PCCL_I32>(L, item_begin, item_end, ptrs, s);
-        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_level_dt<PCCL_F8E4M3>(L, item_begin, item_end, ptrs, s);
+        case PCCL_F8E4M3: return launch_level_dt<PCCL_F8E4M3>(L, item_begin, item_end, ptrs, s);
+        case PCCL_F8E5M2: return launch_level_dt<PCCL_F8E5M2>(L, item_begin, item_end, ptrs, s);
         default: return (int)hipErrorInvalidValue;
     }
 }
@@ -704,13 +748,15 @@ int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, s
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const char* pa = (const char*)a; const char* pb = (const char*)b; char* pc = (char*)c;
-    int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : 2;
+    int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : (dtype == PCCL_F16 || dtype == PCCL_BF16) ? 2 : 1;
     int grid = grid_for_tiles(((int64_t)n * es + kPrimTileBytes - 1) / kPrimTileBytes);
     switch (dtype) {
         case PCCL_F32: hipLaunchKernelGGL((reduce_kernel<PCCL_F32>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
         case PCCL_F16: hipLaunchKernelGGL((reduce_kernel<PCCL_F16>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
         case PCCL_BF16: hipLaunchKernelGGL((reduce_kernel<PCCL_BF16>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
         case PCCL_I32: hipLaunchKernelGGL((reduce_kernel<PCCL_I32>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
+        case PCCL_F8E4M3: hipLaunchKernelGGL((reduce_kernel<PCCL_F8E4M3>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
+        case PCCL_F8E5M2: hipLaunchKernelGGL((reduce_kernel<PCCL_F8E5M2>), dim3(grid), dim3(kThreads), 0, s, pa, pb, pc, (int64_t)n, redop); break;
         default: return (int)hipErrorInvalidValue;
     }
     return (int)hipGetLastError();

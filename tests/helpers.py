@@ -23,8 +23,10 @@ from pccl_amd.dsl import ALGORITHMS, compile_to_json_string  # noqa: E402
 GOLDEN = os.path.join(ROOT, "tests", "golden")
 
 TORCH_DTYPE = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16,
-               "int32": torch.int32}
-RAW_NP = {"float32": np.float32, "float16": np.uint16, "bfloat16": np.uint16, "int32": np.int32}
+               "int32": torch.int32, "float8_e4m3": torch.float8_e4m3fn, "float8_e5m2": torch.float8_e5m2}
+RAW_NP = {"float32": np.float32, "float16": np.uint16, "bfloat16": np.uint16, "int32": np.int32,
+          "float8_e4m3": np.uint8, "float8_e5m2": np.uint8}
+FP8_MAX = {"float8_e4m3": 448.0, "float8_e5m2": 57344.0}
 
 
 def graph_jsons(alg: str, method: str, world: int, n: int, dtype: str, executor: str = "sm",
@@ -40,12 +42,16 @@ def to_raw(t: torch.Tensor) -> np.ndarray:
     t = t.contiguous()
     if t.dtype in (torch.bfloat16, torch.float16):
         return t.view(torch.int16).numpy().view(np.uint16).copy()
+    if t.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        return t.view(torch.uint8).numpy().copy()
     return t.numpy().copy()
 
 
 def from_raw(a: np.ndarray, dtype: str) -> torch.Tensor:
     if dtype in ("bfloat16", "float16"):
         return torch.from_numpy(a.view(np.int16).copy()).view(TORCH_DTYPE[dtype])
+    if dtype in FP8_MAX:
+        return torch.from_numpy(a.view(np.uint8).copy()).view(TORCH_DTYPE[dtype])
     return torch.from_numpy(a.copy())
 
 
@@ -64,6 +70,8 @@ def seeded_inputs(kind: str, world: int, n: int, dtype: str, seed: int = 0) -> L
         x = torch.arange(1, world + 1).view(world, 1).expand(world, n).float()
     else:
         raise ValueError(kind)
+    if dtype in FP8_MAX:   # torch's conversion does not saturate; keep the draw inside the finite range
+        x = x.clamp(-FP8_MAX[dtype], FP8_MAX[dtype])
     return [x[r].to(TORCH_DTYPE[dtype]).contiguous() for r in range(world)]
 
 
@@ -90,6 +98,8 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
         return torch.equal(a.view(torch.int16), b.view(torch.int16))
     if a.dtype == torch.float32:
         return torch.equal(a.view(torch.int32), b.view(torch.int32))
+    if a.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        return torch.equal(a.view(torch.uint8), b.view(torch.uint8))
     return torch.equal(a, b)
 
 
@@ -99,6 +109,9 @@ def mismatch_report(a: torch.Tensor, b: torch.Tensor) -> str:
         ne = (a.view(torch.int16) != b.view(torch.int16)).nonzero().flatten()
     elif a.dtype == torch.float32:
         ne = (a.view(torch.int32) != b.view(torch.int32)).nonzero().flatten()
+    elif a.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        a, b = a.view(torch.uint8), b.view(torch.uint8)
+        ne = (a != b).nonzero().flatten()
     else:
         ne = (a != b).nonzero().flatten()
     if len(ne) == 0:

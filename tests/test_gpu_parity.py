@@ -43,6 +43,8 @@ CASES = [
     ("rhd", 4, 4096, "bfloat16", 1, "randn"),
     ("tree", 32, 1 << 16, "float32", 1, "randn"),
     ("tree", 8, 8192, "float16", 1, "randn0.1"),
+    ("ring", 8, 1 << 16, "float8_e4m3", 2, "randn"),       # fp8: add in f16, saturating narrow
+    ("rhd", 8, 1 << 15, "float8_e5m2", 1, "randn"),
 ]
 
 

@@ -52,6 +52,23 @@ def test_reduce_matches_oracle(dtype, redop, n):
     assert bits_equal(dc, want), mismatch_report(dc, want)
 
 
+@pytest.mark.parametrize("dtype", ["float8_e4m3", "float8_e5m2"])
+@pytest.mark.parametrize("redop", ["sum", "max", "min"])
+def test_fp8_reduce_all_operand_pairs(dtype, redop):
+    """Reference vec.h:272-426 (widen to f16, add, narrow with saturation): every one of the 65,536
+    operand pairs, laid out so that vector bodies, heads and tails all occur (offset 3, odd length)."""
+    codes = torch.arange(256, dtype=torch.int16).to(torch.uint8)
+    a = torch.cat([torch.zeros(3, dtype=torch.uint8), codes.repeat_interleave(256)])
+    b = torch.cat([torch.zeros(3, dtype=torch.uint8), codes.repeat(256)])
+    want = torch.from_numpy(oracle.reduce(dtype, redop, a.numpy().copy(), b.numpy().copy()))
+    da, db = a.cuda(), b.cuda()
+    dc = torch.empty_like(da)
+    gpu_reduce(dtype, redop, da[3:], db[3:], dc[3:])
+    got = dc[3:].cpu()
+    bad = (got != want[3:]).nonzero().flatten()
+    assert bad.numel() == 0, [(hex(int(a[3 + i])), hex(int(b[3 + i])), hex(int(got[i])), hex(int(want[3 + i]))) for i in bad[:8]]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shift", [(0, 0, 0), (1, 1, 1), (3, 3, 3), (1, 2, 3), (0, 1, 0)])
 def test_reduce_unaligned_offsets(dtype, shift):

@@ -114,7 +114,7 @@ def test_load_errors():
     d = _doc(); d["tensor_info"]["dtype"] = "float64"
     assert "Unsupported dtype" in str(_load_err(d))             # reference: throws (sm_channel.h:71)
     d = _doc(); d["tensor_info"]["dtype"] = "float8_e4m3"
-    assert _load_err(d).code == ERR_UNSUPPORTED                 # fp8 reduce is not implemented here
+    assert HostGraph.from_json(json.dumps(d)).dtype == 3              # fp8 graphs load (reference vec.h:272-426)
     d = _doc(); d["operations"][2]["executor"] = "cuda_ce"
     assert _load_err(d).code == ERR_UNSUPPORTED
     d = _doc(); d["operations"][2]["params"]["reduce_op"] = "avg"

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import (TORCH_DTYPE, bits_equal, from_raw, graph_jsons, mismatch_report, oracle,
+from helpers import (FP8_MAX, TORCH_DTYPE, bits_equal, from_raw, graph_jsons, mismatch_report, oracle,
                      oracle_buffers, seeded_inputs, to_raw)
 
 
@@ -110,6 +110,52 @@ def test_max_min_match_torch(dtype, redop):
         nan = torch.isnan(want)
         assert torch.equal(torch.isnan(got), nan)
         assert torch.equal(got[~nan], want[~nan])
+
+
+@pytest.mark.parametrize("dtype", ["float8_e4m3", "float8_e5m2"])
+def test_fp8_sum_all_pairs_match_torch(dtype):
+    """Reference vec.h:272-426: widen to f16, one f16 add, narrow with round-to-nearest-even and
+    saturation to the largest finite value.  Independent authority: torch's CPU float8 <-> float16
+    conversions and float16 add over all 65,536 operand pairs; the saturation is a clamp in f16
+    before narrowing (every value between the largest finite one and its rounding boundary rounds
+    down to it either way).  NaN results are compared as "is NaN" plus the oracle's documented
+    canonical byte 0x7F."""
+    td = TORCH_DTYPE[dtype]
+    codes = torch.arange(256, dtype=torch.int16).to(torch.uint8)
+    a = codes.repeat_interleave(256)
+    b = codes.repeat(256)
+    got = oracle.reduce(dtype, "sum", a.numpy().copy(), b.numpy().copy())
+    s16 = a.view(td).to(torch.float16) + b.view(td).to(torch.float16)
+    nan = torch.isnan(s16)
+    want = s16.clamp(-FP8_MAX[dtype], FP8_MAX[dtype]).to(td).view(torch.uint8).numpy()
+    assert nan.sum() > 0
+    assert (got[nan.numpy()] == 0x7F).all()
+    assert np.array_equal(got[~nan.numpy()], want[~nan.numpy()])
+    # the widening itself: every code decodes to what torch decodes it to (x + (+0) keeps x, except
+    # that -0 + +0 = +0)
+    z = oracle.reduce(dtype, "sum", codes.numpy().copy(), np.zeros(256, np.uint8))
+    fin = ~torch.isnan(codes.view(td).to(torch.float32)).numpy()
+    back = torch.from_numpy(z).view(td).to(torch.float32).numpy()
+    orig = codes.view(td).to(torch.float32).numpy()
+    assert np.array_equal(back[fin], np.clip(orig[fin], -FP8_MAX[dtype], FP8_MAX[dtype]))
+
+
+@pytest.mark.parametrize("dtype", ["float8_e4m3", "float8_e5m2"])
+@pytest.mark.parametrize("redop", ["max", "min"])
+def test_fp8_max_min_all_pairs(dtype, redop):
+    """Extension: NaN-propagating selection; infinities (e5m2) saturate on the way out like every
+    other result of the fp8 path."""
+    td = TORCH_DTYPE[dtype]
+    codes = torch.arange(256, dtype=torch.int16).to(torch.uint8)
+    a = codes.repeat_interleave(256)
+    b = codes.repeat(256)
+    got = oracle.reduce(dtype, redop, a.numpy().copy(), b.numpy().copy())
+    fa, fb = a.view(td).to(torch.float32), b.view(td).to(torch.float32)
+    sel = torch.maximum(fa, fb) if redop == "max" else torch.minimum(fa, fb)
+    nan = torch.isnan(sel).numpy()
+    assert (got[nan] == 0x7F).all()
+    back = torch.from_numpy(got).view(td).to(torch.float32).numpy()
+    assert np.array_equal(back[~nan], np.clip(sel.numpy()[~nan], -FP8_MAX[dtype], FP8_MAX[dtype]))
 
 
 def test_int32_sum_wraps():
