@@ -170,3 +170,59 @@ def build_graph(name, builder_func, device=None) -> Graph:
     with CommunicationOp(name=name, device=device) as op:
         builder_func(op)
     return op.get_graph()
+
+
+class _PipelineStage:
+    def __init__(self, pipeline: "Pipeline"):
+        self._pipeline = pipeline
+        self._stream: Optional[Stream] = None
+
+    def __enter__(self) -> "_PipelineStage":
+        pipe = self._pipeline
+        if pipe._op is None:
+            raise RuntimeError("Pipeline.stage() must be used inside Pipeline.bind()")
+        channel = pipe._iteration % pipe.depth
+        pipe._iteration += 1
+        pipe._op.set_channel(channel)
+        self._stream = Stream(f"__pipe_ch{channel}")
+        self._stream.__enter__()
+        return self
+
+    def __exit__(self, *exc) -> bool:
+        if self._stream is not None:
+            self._stream.__exit__(*exc)
+        return False
+
+
+class _PipelineBinding:
+    def __init__(self, pipeline: "Pipeline", op: CommunicationOp):
+        self._pipeline, self._target = pipeline, op
+
+    def __enter__(self) -> "Pipeline":
+        self._pipeline._op = self._target
+        self._pipeline._iteration = 0
+        return self._pipeline
+
+    def __exit__(self, *exc) -> bool:
+        self._pipeline._op = None
+        return False
+
+
+class Pipeline:
+    """Step-level pipelining over channels (reference pccl/dsl/pipeline.py:64-88): the k-th
+    ``stage()`` of a bound pipeline puts its ops on channel ``k % depth`` and on the stream
+    ``__pipe_ch<channel>``, so stages on one channel run in order and different channels are
+    independent of each other."""
+
+    def __init__(self, depth: int = 2):
+        if depth < 1:
+            raise ValueError(f"Pipeline depth must be >= 1, got {depth}")
+        self.depth = depth
+        self._op: Optional[CommunicationOp] = None
+        self._iteration = 0
+
+    def bind(self, op: CommunicationOp) -> _PipelineBinding:
+        return _PipelineBinding(self, op)
+
+    def stage(self) -> _PipelineStage:
+        return _PipelineStage(self)

@@ -65,7 +65,59 @@ def load_reference_dsl():
     ring = _load("pccl.dsl.algorithms.ring", "pccl/dsl/algorithms/ring.py")
     rhd = _load("pccl.dsl.algorithms.recursive_hd", "pccl/dsl/algorithms/recursive_hd.py")
     tree = _load("pccl.dsl.algorithms.tree", "pccl/dsl/algorithms/tree.py")
+    pipe = _load("pccl.dsl.pipeline", "pccl/dsl/pipeline.py")
+    comp.decorators = sys.modules["pccl.dsl.decorators"]
+    comp.Pipeline = pipe.Pipeline
     return comp, ring, rhd, tree
+
+
+def pipelined_ring_allreduce(CommunicationOp, Pipeline, rank, world, n, dtype, depth):
+    """Ring allreduce whose steps rotate over `depth` channels through the Pipeline construct; every
+    notify / wait pair has its own signal id.  The schedule is the one the reference's bandwidth
+    script builds (tests/bench_allreduce_tma_bw.py:119-186); tests/test_emitter.py holds the same
+    function over the package under test."""
+    chunk = n // world
+    prev_rank, next_rank = (rank - 1) % world, (rank + 1) % world
+    with CommunicationOp(name=f"ar_pipe{depth}_rank{rank}") as op:
+        op.tensor(dtype=dtype, shape=(n,))
+        pipe = Pipeline(depth=depth)
+        sig = 0
+        with pipe.bind(op):
+            for _ in range(depth):
+                with pipe.stage():
+                    sig += 1
+                    op.notify(signal_id=sig, target_rank=next_rank)
+                    op.wait_notify(signal_id=sig, source_rank=prev_rank)
+            for step in range(world - 1):
+                with pipe.stage():
+                    off = ((rank - step - 1) % world) * chunk
+                    if step > 0:
+                        sig += 1
+                        op.wait_notify(signal_id=sig, source_rank=prev_rank)
+                    op.sm_reduce(reduce_op="sum", source_rank=prev_rank, src_offset=off, dst_offset=off,
+                                 remote_offset=off, count=chunk)
+                    sig += 1
+                    op.notify(signal_id=sig, target_rank=next_rank)
+            for step in range(world - 1):
+                with pipe.stage():
+                    off = ((rank - step) % world) * chunk
+                    sig += 1
+                    op.wait_notify(signal_id=sig, source_rank=prev_rank)
+                    op.sm_copy(source_rank=prev_rank, src_offset=off, dst_offset=off, size=chunk)
+                    sig += 1
+                    op.notify(signal_id=sig, target_rank=next_rank)
+            for _ in range(depth):
+                with pipe.stage():
+                    sig += 1
+                    op.wait_notify(signal_id=sig, source_rank=prev_rank)
+        return op.get_graph()
+
+
+PIPELINE_CASES = [
+    # (file stem, world, tensor_size, dtype, depth)
+    ("pipe_ring_ar_w4_n4096_bf16_d2", 4, 4096, "bfloat16", 2),
+    ("pipe_ring_ar_w3_n3072_f32_d3", 3, 3072, "float32", 3),
+]
 
 
 CASES = [
@@ -103,10 +155,19 @@ def main():
         index.append({"stem": stem, "algorithm": alg, "method": method, "world_size": world,
                       "tensor_size": n, "dtype": dtype, "executor": executor,
                       "num_channels": ch})
+    for stem, world, n, dtype, depth in PIPELINE_CASES:
+        for rank in range(world):
+            g = pipelined_ring_allreduce(comp.decorators.CommunicationOp, comp.Pipeline, rank, world, n, dtype, depth)
+            doc = json.loads(comp.compile_to_json_string(g))
+            with open(os.path.join(OUT, f"{stem}_rank{rank}.json"), "w") as f:
+                json.dump(doc, f, separators=(",", ":"))
+                f.write("\n")
+        index.append({"stem": stem, "algorithm": "pipelined_ring", "method": "build_allreduce", "world_size": world,
+                      "tensor_size": n, "dtype": dtype, "executor": "sm", "num_channels": depth})
     with open(os.path.join(OUT, "index.json"), "w") as f:
         json.dump(index, f, indent=1)
         f.write("\n")
-    print(f"wrote {sum(c[3] for c in CASES)} graphs to {OUT}")
+    print(f"wrote {sum(c[3] for c in CASES) + sum(c[1] for c in PIPELINE_CASES)} graphs to {OUT}")
 
 
 if __name__ == "__main__":

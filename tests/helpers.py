@@ -18,7 +18,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 from oracle import oracle  # noqa: E402
-from pccl_amd.dsl import ALGORITHMS, compile_to_json_string  # noqa: E402
+from pccl_amd.dsl import ALGORITHMS, CommunicationOp, Pipeline, compile_to_json_string  # noqa: E402
 
 GOLDEN = os.path.join(ROOT, "tests", "golden")
 
@@ -35,6 +35,56 @@ def graph_jsons(alg: str, method: str, world: int, n: int, dtype: str, executor:
     return [compile_to_json_string(getattr(a, method)(r, world, n, dtype=dtype, executor=executor,
                                                       num_channels=channels, **ext))
             for r in range(world)]
+
+
+def pipelined_ring_allreduce(rank: int, world: int, n: int, dtype: str, depth: int, reduce_op: str = "sum",
+                             paired_signals: bool = False):
+    """Ring allreduce whose steps rotate over `depth` channels through the Pipeline construct.
+
+    paired_signals=False numbers the signals exactly as the reference's bandwidth script does
+    (tests/bench_allreduce_tma_bw.py:119-186: one running counter over waits and notifies).  That
+    numbering makes step s+1 wait on an id nobody notifies; the reference's kernels get past such a
+    wait through their spin bail-out (cuda_executor.cu:946-961), exact semaphore semantics report a
+    deadlock.  paired_signals=True is the same schedule with the wait of step t+1 on the id step t
+    of the previous rank notifies, which is executable."""
+    chunk = n // world
+    prev_rank, next_rank = (rank - 1) % world, (rank + 1) % world
+    steps = [("reduce", ((rank - s - 1) % world) * chunk) for s in range(world - 1)] + \
+            [("copy", ((rank - s) % world) * chunk) for s in range(world - 1)]
+    with CommunicationOp(name=f"ar_pipe{depth}_rank{rank}") as op:
+        op.tensor(dtype=dtype, shape=(n,))
+        pipe = Pipeline(depth=depth)
+        sig = 0
+        with pipe.bind(op):
+            for _ in range(depth):
+                with pipe.stage():
+                    sig += 1
+                    op.notify(signal_id=sig, target_rank=next_rank)
+                    op.wait_notify(signal_id=sig, source_rank=prev_rank)
+            for t, (kind, off) in enumerate(steps):
+                with pipe.stage():
+                    if paired_signals:
+                        if t > 0:
+                            op.wait_notify(signal_id=100 + t - 1, source_rank=prev_rank)
+                    elif t > 0:
+                        sig += 1
+                        op.wait_notify(signal_id=sig, source_rank=prev_rank)
+                    if kind == "reduce":
+                        op.sm_reduce(reduce_op=reduce_op, source_rank=prev_rank, src_offset=off, dst_offset=off,
+                                     remote_offset=off, count=chunk)
+                    else:
+                        op.sm_copy(source_rank=prev_rank, src_offset=off, dst_offset=off, size=chunk)
+                    sig += 1
+                    op.notify(signal_id=100 + t if paired_signals else sig, target_rank=next_rank)
+            if paired_signals:
+                with pipe.stage():
+                    op.wait_notify(signal_id=100 + len(steps) - 1, source_rank=prev_rank)
+            else:
+                for _ in range(depth):
+                    with pipe.stage():
+                        sig += 1
+                        op.wait_notify(signal_id=sig, source_rank=prev_rank)
+        return op.get_graph()
 
 
 def to_raw(t: torch.Tensor) -> np.ndarray:

@@ -10,7 +10,8 @@ import os
 import pytest
 
 from helpers import GOLDEN
-from pccl_amd.dsl import (ALGORITHMS, CommunicationOp, Compiler, RecursiveHalvingDoubling, RingAllreduce,
+from helpers import pipelined_ring_allreduce
+from pccl_amd.dsl import (ALGORITHMS, CommunicationOp, Compiler, Pipeline, RecursiveHalvingDoubling, RingAllreduce,
                           Stream, TreeAllreduce, build_graph, compile_to_json_string, ragged_cuts)
 
 with open(os.path.join(GOLDEN, "graphs", "index.json")) as f:
@@ -19,10 +20,14 @@ with open(os.path.join(GOLDEN, "graphs", "index.json")) as f:
 
 @pytest.mark.parametrize("case", INDEX, ids=[c["stem"] for c in INDEX])
 def test_emitted_json_equals_reference_emitter(case):
-    alg = ALGORITHMS[case["algorithm"]]()
     for rank in range(case["world_size"]):
-        g = getattr(alg, case["method"])(rank, case["world_size"], case["tensor_size"], dtype=case["dtype"],
-                                         executor=case["executor"], num_channels=case["num_channels"])
+        if case["algorithm"] == "pipelined_ring":    # built with the Pipeline construct (reference pipeline.py)
+            g = pipelined_ring_allreduce(rank, case["world_size"], case["tensor_size"], case["dtype"],
+                                         case["num_channels"])
+        else:
+            g = getattr(ALGORITHMS[case["algorithm"]](), case["method"])(
+                rank, case["world_size"], case["tensor_size"], dtype=case["dtype"],
+                executor=case["executor"], num_channels=case["num_channels"])
         mine = json.loads(compile_to_json_string(g))
         with open(os.path.join(GOLDEN, "graphs", f"{case['stem']}_rank{rank}.json")) as f:
             ref = json.load(f)
@@ -148,3 +153,28 @@ def test_ragged_cuts_rule():
     g = TreeAllreduce().build_allreduce(0, 4, 4099, dtype="int32", executor="sm", cuts=ragged_cuts(4099, 5))
     reduces = [o for o in g.ops.values() if o.primitive == "sm.reduce"]
     assert sum(o.params["count"] for o in reduces) == 2 * 4099   # rank 0 reduces twice over the whole tensor
+
+
+def test_pipeline_construct():                # reference pccl/dsl/pipeline.py:64-88
+    with pytest.raises(ValueError):
+        Pipeline(depth=0)
+    with CommunicationOp(name="p") as op:
+        op.tensor(dtype="float32", shape=(64,))
+        pipe = Pipeline(depth=2)
+        with pytest.raises(RuntimeError):
+            with pipe.stage():
+                pass
+        with pipe.bind(op):
+            made = []
+            for k in range(5):
+                with pipe.stage():
+                    made.append(op.sm_copy(source_rank=1, src_offset=0, dst_offset=0, size=8))
+    doc = json.loads(compile_to_json_string(op.get_graph()))
+    ops = sorted(doc["operations"], key=lambda o: o["index"])
+    assert sorted(o["channel"] for o in ops) == [0, 0, 0, 1, 1]
+    # stages of one channel are chained, channels are independent: two roots, two leaves
+    assert sum(1 for o in ops if not o["dependencies"]) == 2
+    assert sum(1 for o in ops if not o["next_ops"]) == 2
+    for o in ops:
+        for d in o["dependencies"]:
+            assert ops[d]["channel"] == o["channel"]

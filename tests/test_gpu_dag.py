@@ -1,0 +1,122 @@
+"""Graphs that are not single chains, through the level-scheduled runner and (where the ops are
+position-aligned) the column runner: Pipeline-built graphs, fork / join over streams with several
+dependencies and successors per op, and `noop` nodes — the ground the reference covers with its
+DAG kernel (cuda_executor.cu:526-918: remaining_deps counters, up to 8 successors per op).
+"""
+import json
+
+import pytest
+import torch
+
+from helpers import (bits_equal, graph_jsons, mismatch_report, oracle_buffers, pipelined_ring_allreduce,
+                     seeded_inputs)
+from pccl_amd.dsl import CommunicationOp, Stream, compile_to_json_string
+
+pytestmark = pytest.mark.gpu
+
+
+def run(engine, name, jsons, inputs, mode):
+    for r, j in enumerate(jsons):
+        engine.register_operation_json(name, j, r)
+    engine.set_option("mode", mode)
+    dev = [x.cuda() for x in inputs]
+    engine.execute_inplace(name, dev, sync=True)
+    return [d.cpu() for d in dev]
+
+
+@pytest.mark.parametrize("world,depth,dtype", [(4, 2, "float32"), (8, 3, "bfloat16"), (3, 3, "float16")])
+@pytest.mark.parametrize("mode", ["column", "stepwise"])
+def test_pipeline_built_ring(engine_factory, world, depth, dtype, mode):
+    """Steps rotate over `depth` channels (reference pccl/dsl/pipeline.py); consecutive steps of a
+    rank are ordered only through the signal chain around the ring."""
+    n = world * 4096
+    jsons = [compile_to_json_string(pipelined_ring_allreduce(r, world, n, dtype, depth, paired_signals=True))
+             for r in range(world)]
+    x = seeded_inputs("randn", world, n, dtype, seed=5)
+    want = oracle_buffers(jsons, x, dtype)
+    # the pipelined schedule computes what the plain ring computes, in the same order
+    plain = oracle_buffers(graph_jsons("ring", "build_allreduce", world, n, dtype, "sm", 1), x, dtype)
+    assert all(bits_equal(a, b) for a, b in zip(want, plain))
+    engine = engine_factory(world)
+    got = run(engine, "pipe", jsons, x, mode)
+    info = engine.op_info("pipe")
+    assert info["residual_signals"] == 0 and info["num_data_ops"] == 2 * (world - 1) * world
+    for r in range(world):
+        assert bits_equal(got[r], want[r]), f"rank {r}: {mismatch_report(got[r], want[r])}"
+
+
+def fork_join_graph(rank, chunk, dtype):
+    """Per rank, over a tensor of 9 chunks of which the first four are only ever read: four
+    independent streams each copy one of the peer's chunks 0..3 into own chunks 4..7; the main
+    stream joins all four (one op with four dependencies) and reduces the peer's chunk 0 with own
+    chunk 5 into own chunk 4 (read-after-write on stream b, write-after-write on stream a); four
+    more streams fork from that op (four successors) and overwrite own chunks 5..8."""
+    peer = 1 - rank
+    with CommunicationOp(name=f"fj{rank}") as op:
+        op.tensor(dtype=dtype, shape=(9 * chunk,))
+        for k, name in enumerate("abcd"):
+            with Stream(name):
+                op.set_channel(k % 2)
+                op.sm_copy(source_rank=peer, src_offset=k * chunk, dst_offset=(4 + k) * chunk, size=chunk)
+        op.set_channel(0)
+        for name in "abcd":
+            op.wait(name)
+        joined = op.sm_reduce(reduce_op="sum", source_rank=peer, remote_offset=0, src_offset=5 * chunk,
+                              dst_offset=4 * chunk, count=chunk)
+        for k, name in enumerate("efgh"):
+            with Stream(name):
+                op.set_channel(1 + k % 2)
+                op.wait_for(joined)
+                op.sm_copy(source_rank=peer, src_offset=((k + 3) % 4) * chunk, dst_offset=(5 + k) * chunk, size=chunk)
+        return op.get_graph()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_fork_join_over_streams(engine_factory, dtype):
+    chunk = 4099          # odd: offsets off 16-byte alignment
+    jsons = [compile_to_json_string(fork_join_graph(r, chunk, dtype)) for r in range(2)]
+    doc = json.loads(jsons[0])
+    assert max(len(o["dependencies"]) for o in doc["operations"]) >= 4
+    assert max(len(o["next_ops"]) for o in doc["operations"]) >= 4
+    x = seeded_inputs("randn", 2, 9 * chunk, dtype, seed=9)
+    want = oracle_buffers(jsons, x, dtype)
+    engine = engine_factory(2)
+    got = run(engine, "fj", jsons, x, "auto")
+    info = engine.op_info("fj")
+    assert info["position_aligned"] == 0 and info["num_levels"] == 3
+    for r in range(2):
+        assert bits_equal(got[r], want[r]), f"rank {r}: {mismatch_report(got[r], want[r])}"
+
+
+def test_noop_nodes_are_contracted(engine_factory):
+    """A `noop` between two data ops keeps their order and costs nothing: the linked program has
+    the same data ops and levels as the graph without it."""
+    world, n = 2, 4096
+    base = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)
+    with_noop = []
+    for text in base:
+        doc = json.loads(text)
+        ops = doc["operations"]
+        # splice a noop after the first data op: it takes over that op's successors
+        k = next(i for i, o in enumerate(ops) if o["primitive"].endswith("reduce"))
+        new_index = len(ops)
+        noop = {"index": new_index, "executor": "cuda_sm", "primitive": "noop", "channel": ops[k]["channel"],
+                "dependencies": [k], "next_ops": list(ops[k]["next_ops"]), "params": {}}
+        for nxt in ops[k]["next_ops"]:
+            ops[nxt]["dependencies"] = [new_index if d == k else d for d in ops[nxt]["dependencies"]]
+        ops[k]["next_ops"] = [new_index]
+        ops.append(noop)
+        with_noop.append(json.dumps(doc))
+    x = seeded_inputs("randn", world, n, "float32", seed=2)
+    want = oracle_buffers(base, x, "float32")
+    assert all(bits_equal(a, b) for a, b in zip(oracle_buffers(with_noop, x, "float32"), want))
+    engine = engine_factory(world)
+    got = run(engine, "noop", with_noop, x, "stepwise")
+    plain = engine_factory(world)
+    for r, j in enumerate(base):
+        plain.register_operation_json("plain", j, r)
+    a, b = engine.op_info("noop"), plain.op_info("plain")
+    assert (a["num_data_ops"], a["num_levels"]) == (b["num_data_ops"], b["num_levels"])
+    assert a["num_ops"] == b["num_ops"] + world
+    for r in range(world):
+        assert bits_equal(got[r], want[r])

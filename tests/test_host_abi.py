@@ -281,3 +281,24 @@ def test_linker_rejects_partially_overlapping_in_place_op():
 def test_residual_signals_are_counted():
     jsons = _two_rank(lambda op, me, other: op.notify(signal_id=9, target_rank=other))   # never awaited
     assert _link(jsons).info()["residual_signals"] == 2
+
+
+def test_reference_numbered_pipeline_schedule_is_reported_as_deadlock():
+    """The pipelined ring of the reference's bandwidth script (tests/bench_allreduce_tma_bw.py:119-186)
+    numbers waits and notifies with one running counter, so every wait after the first step is on
+    an id nobody notifies; the reference gets past it through the spin bail-out of its wait
+    (cuda_executor.cu:946-961).  Linked with exact semaphore semantics this is a deadlock, reported
+    at link time, by the product's linker and by the oracle alike."""
+    from helpers import pipelined_ring_allreduce, oracle_buffers, seeded_inputs
+    from pccl_amd.dsl import compile_to_json_string
+    world, n = 4, 4096
+    jsons = [compile_to_json_string(pipelined_ring_allreduce(r, world, n, "float32", 2)) for r in range(world)]
+    with pytest.raises(PcclError, match="deadlock"):
+        HostProgram([HostGraph.from_json(j) for j in jsons])
+    with pytest.raises(Exception, match="deadlock"):
+        oracle_buffers(jsons, seeded_inputs("randn", world, n, "float32"), "float32")
+    # the same schedule with paired signal ids links, race-free
+    jsons = [compile_to_json_string(pipelined_ring_allreduce(r, world, n, "float32", 2, paired_signals=True))
+             for r in range(world)]
+    info = HostProgram([HostGraph.from_json(j) for j in jsons]).info()
+    assert info["residual_signals"] == 0 and info["position_aligned"] == 1 and info["num_data_ops"] == 24
