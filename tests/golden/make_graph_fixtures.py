@@ -66,6 +66,21 @@ def load_reference_dsl():
     rhd = _load("pccl.dsl.algorithms.recursive_hd", "pccl/dsl/algorithms/recursive_hd.py")
     tree = _load("pccl.dsl.algorithms.tree", "pccl/dsl/algorithms/tree.py")
     pipe = _load("pccl.dsl.pipeline", "pccl/dsl/pipeline.py")
+    # the channelize pass and the cost model it consults: plain Python, loaded without running
+    # superopt/__init__ (which needs z3)
+    _pkg("pccl.dsl.superopt", os.path.join(REF, "pccl/dsl/superopt"))
+    _load("pccl.dsl.superopt.rule", "pccl/dsl/superopt/rule.py")
+    _load("pccl.dsl.superopt.cost_model", "pccl/dsl/superopt/cost_model.py")
+    chan = _load("pccl.dsl.passes.channelize", "pccl/dsl/passes/channelize.py")
+
+    def compile_channelized(graph, num_channels):
+        dep.DependencyAnalysisPass().run(graph)
+        dce.DeadCodeEliminationPass().run(graph)
+        chan.ChannelizePass(num_channels=num_channels).run(graph)
+        dep.DependencyAnalysisPass().run(graph)
+        return gen.RuntimeGraphGenerator(indent=2).generate_string(graph)
+
+    comp.compile_channelized = compile_channelized
     comp.decorators = sys.modules["pccl.dsl.decorators"]
     comp.Pipeline = pipe.Pipeline
     return comp, ring, rhd, tree
@@ -111,6 +126,38 @@ def pipelined_ring_allreduce(CommunicationOp, Pipeline, rank, world, n, dtype, d
                     sig += 1
                     op.wait_notify(signal_id=sig, source_rank=prev_rank)
         return op.get_graph()
+
+
+def chained_gather(CommunicationOp, rank, world, chunk, dtype, pieces, kind):
+    """A chain that the channelize pass accepts: `pieces` same-type data ops from the next rank whose
+    source ranges follow one another, a notify / wait pair between every two, closed by a notify.
+    tests/helpers.py holds the same function over the package under test."""
+    peer = (rank + 1) % world
+    with CommunicationOp(name=f"chain_{kind}_rank{rank}") as op:
+        op.tensor(dtype=dtype, shape=(pieces * chunk,))
+        op.notify(signal_id=1, target_rank=(rank - 1) % world)
+        op.wait_notify(signal_id=1, source_rank=peer)
+        for k in range(pieces):
+            if kind == "copy":
+                op.sm_copy(source_rank=peer, src_offset=k * chunk, dst_offset=k * chunk, size=chunk)
+            else:
+                op.tma_reduce(reduce_op="sum", source_rank=peer, src_offset=k * chunk, dst_offset=k * chunk,
+                              remote_offset=k * chunk, count=chunk)
+            if k % 2 == 1:
+                op.notify(signal_id=10 + k, target_rank=(rank - 1) % world)
+                op.wait_notify(signal_id=10 + k, source_rank=peer)
+        op.notify(signal_id=2, target_rank=(rank - 1) % world)
+        op.wait_notify(signal_id=2, source_rank=peer)
+        return op.get_graph()
+
+
+CHANNELIZE_CASES = [
+    # (file stem, world, chunk, dtype, pieces, kind, num_channels)
+    ("chan_copy_w2_c65536_f32_p8_nc2", 2, 65536, "float32", 8, "copy", 2),
+    ("chan_reduce_w2_c16384_bf16_p7_nc3", 2, 16384, "bfloat16", 7, "reduce", 3),
+    ("chan_copy_w2_c256_f16_p6_nc2", 2, 256, "float16", 6, "copy", 2),       # below min_data_size: untouched
+    ("chan_copy_w2_c65536_f32_p2_nc2", 2, 65536, "float32", 2, "copy", 2),   # chain not longer than channels
+]
 
 
 PIPELINE_CASES = [
@@ -164,10 +211,20 @@ def main():
                 f.write("\n")
         index.append({"stem": stem, "algorithm": "pipelined_ring", "method": "build_allreduce", "world_size": world,
                       "tensor_size": n, "dtype": dtype, "executor": "sm", "num_channels": depth})
+    for stem, world, chunk, dtype, pieces, kind, nc in CHANNELIZE_CASES:
+        for rank in range(world):
+            g = chained_gather(comp.decorators.CommunicationOp, rank, world, chunk, dtype, pieces, kind)
+            doc = json.loads(comp.compile_channelized(g, nc))
+            with open(os.path.join(OUT, f"{stem}_rank{rank}.json"), "w") as f:
+                json.dump(doc, f, separators=(",", ":"))
+                f.write("\n")
+        index.append({"stem": stem, "algorithm": "chained_gather", "method": kind, "world_size": world,
+                      "tensor_size": pieces * chunk, "dtype": dtype, "executor": "sm" if kind == "copy" else "tma",
+                      "num_channels": nc, "pieces": pieces})
     with open(os.path.join(OUT, "index.json"), "w") as f:
         json.dump(index, f, indent=1)
         f.write("\n")
-    print(f"wrote {sum(c[3] for c in CASES) + sum(c[1] for c in PIPELINE_CASES)} graphs to {OUT}")
+    print(f"wrote {sum(c[3] for c in CASES) + sum(c[1] for c in PIPELINE_CASES) + sum(c[1] for c in CHANNELIZE_CASES)} graphs to {OUT}")
 
 
 if __name__ == "__main__":

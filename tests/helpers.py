@@ -87,6 +87,29 @@ def pipelined_ring_allreduce(rank: int, world: int, n: int, dtype: str, depth: i
         return op.get_graph()
 
 
+def chained_gather(rank: int, world: int, chunk: int, dtype: str, pieces: int, kind: str):
+    """`pieces` same-type data ops from the next rank whose source ranges follow one another, a
+    notify / wait pair after every second one, closed by a notify / wait: the shape of chain the
+    channelize pass (reference pccl/dsl/passes/channelize.py) looks for."""
+    peer = (rank + 1) % world
+    with CommunicationOp(name=f"chain_{kind}_rank{rank}") as op:
+        op.tensor(dtype=dtype, shape=(pieces * chunk,))
+        op.notify(signal_id=1, target_rank=(rank - 1) % world)
+        op.wait_notify(signal_id=1, source_rank=peer)
+        for k in range(pieces):
+            if kind == "copy":
+                op.sm_copy(source_rank=peer, src_offset=k * chunk, dst_offset=k * chunk, size=chunk)
+            else:
+                op.tma_reduce(reduce_op="sum", source_rank=peer, src_offset=k * chunk, dst_offset=k * chunk,
+                              remote_offset=k * chunk, count=chunk)
+            if k % 2 == 1:
+                op.notify(signal_id=10 + k, target_rank=(rank - 1) % world)
+                op.wait_notify(signal_id=10 + k, source_rank=peer)
+        op.notify(signal_id=2, target_rank=(rank - 1) % world)
+        op.wait_notify(signal_id=2, source_rank=peer)
+        return op.get_graph()
+
+
 def to_raw(t: torch.Tensor) -> np.ndarray:
     """CPU tensor -> numpy array of its storage bits (bf16/f16 as uint16)."""
     t = t.contiguous()

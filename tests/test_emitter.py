@@ -10,7 +10,9 @@ import os
 import pytest
 
 from helpers import GOLDEN
-from helpers import pipelined_ring_allreduce
+from helpers import chained_gather, pipelined_ring_allreduce
+from pccl_amd.dsl.channelize import (H100_PROFILE, MI355X_PROFILE, ChannelizePass, DeviceProfile,
+                                     critical_path_cost_us, op_latency_us)
 from pccl_amd.dsl import (ALGORITHMS, CommunicationOp, Compiler, Pipeline, RecursiveHalvingDoubling, RingAllreduce,
                           Stream, TreeAllreduce, build_graph, compile_to_json_string, ragged_cuts)
 
@@ -24,6 +26,13 @@ def test_emitted_json_equals_reference_emitter(case):
         if case["algorithm"] == "pipelined_ring":    # built with the Pipeline construct (reference pipeline.py)
             g = pipelined_ring_allreduce(rank, case["world_size"], case["tensor_size"], case["dtype"],
                                          case["num_channels"])
+        elif case["algorithm"] == "chained_gather":  # compiled with the channelize pass switched on
+            g = chained_gather(rank, case["world_size"], case["tensor_size"] // case["pieces"], case["dtype"],
+                               case["pieces"], case["method"])
+            mine = Compiler(enable_channelize=True, num_channels=case["num_channels"]).compile_to_dict(g)
+            with open(os.path.join(GOLDEN, "graphs", f"{case['stem']}_rank{rank}.json")) as f:
+                assert json.dumps(mine) == json.dumps(json.load(f)), f"rank {rank}"
+            continue
         else:
             g = getattr(ALGORITHMS[case["algorithm"]](), case["method"])(
                 rank, case["world_size"], case["tensor_size"], dtype=case["dtype"],
@@ -178,3 +187,33 @@ def test_pipeline_construct():                # reference pccl/dsl/pipeline.py:6
     for o in ops:
         for d in o["dependencies"]:
             assert ops[d]["channel"] == o["channel"]
+
+
+def test_cost_model_closed_forms():            # reference pccl/dsl/superopt/cost_model.py:113-200
+    p = H100_PROFILE
+    assert op_latency_us("notify", p) == 1.0
+    assert op_latency_us("sm.copy", p, 50_000) == pytest.approx(1.0 + 1.0)           # 50 KB at 50 GB/s
+    # reduce: max(transfer, compute): 120,000 B at 60 GB/s = 2 us; 30,000 elements at 35 Gop/s = 0.857 us
+    assert op_latency_us("tma.reduce", p, 120_000) == pytest.approx(1.0 + 2.0)
+    chain = [("sm.copy", 0)] * 4
+    edges = [(0, 1), (1, 2), (2, 3)]
+    assert critical_path_cost_us(chain, edges, p, 50_000) == pytest.approx(8.0)
+    split = [("sm.copy", 0), ("sm.copy", 0), ("sm.copy", 1), ("sm.copy", 1)]
+    assert critical_path_cost_us(split, [(0, 1), (2, 3)], p, 50_000) == pytest.approx(4.0 + 0.5)
+    assert critical_path_cost_us([], [], p) == 0.0
+    q = DeviceProfile.from_dict(MI355X_PROFILE.to_dict())
+    assert q == MI355X_PROFILE and q.bandwidth_gb_s["tma"] == q.bandwidth_gb_s["sm"]
+
+
+def test_channelize_leaves_non_contiguous_chains_alone():
+    """The ring template's consecutive steps work on descending chunks, which do not follow one
+    another, so the pass changes nothing there (whatever the profile)."""
+    for profile in (H100_PROFILE, MI355X_PROFILE):
+        g = RingAllreduce().build_allreduce(0, 8, 8 * 65536, dtype="float32", executor="sm")
+        before = json.dumps(Compiler().compile_to_dict(g))
+        g2 = RingAllreduce().build_allreduce(0, 8, 8 * 65536, dtype="float32", executor="sm")
+        after = json.dumps(Compiler(enable_channelize=True, num_channels=2, device_profile=profile).compile_to_dict(g2))
+        assert before == after
+    g = chained_gather(0, 2, 65536, "float32", 8, "copy")
+    ChannelizePass(num_channels=4, profile=MI355X_PROFILE).run(g)
+    assert sorted({o.channel for o in g.ops.values() if o.is_data}) == [0, 1, 2, 3]

@@ -120,3 +120,28 @@ def test_noop_nodes_are_contracted(engine_factory):
     assert a["num_ops"] == b["num_ops"] + world
     for r in range(world):
         assert bits_equal(got[r], want[r])
+
+
+def test_channelized_chain(engine_factory):
+    """A chain whose data ops the channelize pass (reference pccl/dsl/passes/channelize.py) has
+    moved to other channels while their dependencies still cross those channels: the labels change
+    the queues the ops sit in, not their order."""
+    from pccl_amd.dsl import Compiler
+    world, chunk, pieces = 2, 8192, 8
+    jsons = []
+    for rank in range(world):
+        peer = 1 - rank
+        with CommunicationOp(name=f"gather{rank}") as op:
+            op.tensor(dtype="float16", shape=(2 * pieces * chunk,))
+            for k in range(pieces):     # the peer's first half is never written: no signals needed
+                op.sm_copy(source_rank=peer, src_offset=k * chunk, dst_offset=(pieces + k) * chunk, size=chunk)
+        jsons.append(Compiler(enable_channelize=True, num_channels=2).compile_to_json(op.get_graph()))
+    doc = json.loads(jsons[0])
+    assert [o["channel"] for o in doc["operations"]] == [0, 0, 0, 0, 1, 1, 1, 1]
+    assert doc["operations"][4]["dependencies"] == [3]          # the chain still crosses the channels
+    x = seeded_inputs("randn", world, 2 * pieces * chunk, "float16", seed=11)
+    want = oracle_buffers(jsons, x, "float16")
+    got = run(engine_factory(world), "chan", jsons, x, "auto")
+    for r in range(world):
+        assert bits_equal(got[r], want[r]), mismatch_report(got[r], want[r])
+        assert bits_equal(got[r][pieces * chunk:], x[1 - r][:pieces * chunk])
