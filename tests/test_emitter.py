@@ -217,3 +217,24 @@ def test_channelize_leaves_non_contiguous_chains_alone():
     g = chained_gather(0, 2, 65536, "float32", 8, "copy")
     ChannelizePass(num_channels=4, profile=MI355X_PROFILE).run(g)
     assert sorted({o.channel for o in g.ops.values() if o.is_data}) == [0, 1, 2, 3]
+
+
+def test_algorithm_selector():                 # reference pccl/dsl/algorithms/selector.py:24-56
+    from pccl_amd.dsl.algorithms import select_algorithm, select_algorithm_cost_based
+    from pccl_amd.dsl.algorithms.selector import graph_cost_us
+    MB = 1 << 20
+    table = {(8, 4 * MB): RingAllreduce, (8, MB): RingAllreduce, (8, MB - 1): RecursiveHalvingDoubling,
+             (4, 1024): RecursiveHalvingDoubling, (2, 1024): RingAllreduce, (6, 1024): RingAllreduce,
+             (3, 64 * MB): RingAllreduce, (16, 65536): RecursiveHalvingDoubling}
+    for (world, size), want in table.items():
+        assert type(select_algorithm(world, size)) is want, (world, size)
+    # cost based: the candidate with the smallest critical path, found independently here
+    for world, nbytes, profile in ((8, 4096, H100_PROFILE), (8, 64 * MB, H100_PROFILE), (16, 4096, MI355X_PROFILE),
+                                   (6, 4096, H100_PROFILE)):
+        cands = [RingAllreduce()] + ([RecursiveHalvingDoubling(), TreeAllreduce()] if world & (world - 1) == 0 else [])
+        costs = [graph_cost_us(a.build_allreduce(rank=1, world_size=world, tensor_size=world * 1024,
+                                                 dtype="bfloat16", executor="tma"), profile, nbytes) for a in cands]
+        got = select_algorithm_cost_based(1, world, world * 1024, nbytes, device=profile)
+        assert type(got) is type(cands[costs.index(min(costs))])
+    # log-step schedules have the shorter critical path for small messages on 8 ranks
+    assert type(select_algorithm_cost_based(0, 8, 8192, 1024)) is not RingAllreduce
