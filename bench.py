@@ -123,7 +123,7 @@ def measured_traffic(mode: str, levels: int):
     """HBM bytes per execution of the headline graph from the committed rocprofv3 counter summaries
     (FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy): one launch of the column kernel, or one launch
     per dependency level of the level kernel."""
-    kernel = "level_kernel" if mode == "stepwise" else "column_kernel"
+    kernel = "level_kernel" if mode == "stepwise" else "column_slot_kernel"
     path = os.path.join(ROOT, "profiles", f"{kernel}_ring_allreduce_R8_bf16_512MiB.traffic.json")
     try:
         with open(path) as f:
@@ -272,7 +272,8 @@ def main() -> int:
                     "frac_of_hbm_peak": round(alg_bytes / (sw_ms * 1e-3) / 1e9 / PEAK_GBPS, 4),
                     "note": "HBM traffic equals the algorithmic bytes in this mode (profiles/level_kernel_*.md)"}
 
-    traffic = measured_traffic(args.mode, info["num_levels"]) if (n == N and channels == CHANNELS) else None
+    default_runner = not any(kv.split("=")[0] in ("lds_slots", "slot_threads", "slot_direct") for kv in args.option)
+    traffic = measured_traffic(args.mode, info["num_levels"]) if (n == N and channels == CHANNELS and default_runner) else None
     result = {
         "metric": "HBM GB/s (algorithmic schedule bytes read+written per second), 8-vrank 512MB bf16 ring allreduce graph",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -286,6 +287,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_GBPS, 4), "traffic": traffic,
                      "kernel_ms_avg": round(avg_ms, 4), "kernel_ms_min": round(min(kern_ms), 4),
+                     "kernel_ms_median": round(sorted(kern_ms)[len(kern_ms) // 2], 4),
                      "planned_load_bytes": info["column_load_bytes"], "planned_store_bytes": info["column_store_bytes"]},
         "end_to_end_staged": {"ms_per_call": round(staged_ms, 4), "GB/s": round(alg_bytes / (staged_ms * 1e-3) / 1e9, 1),
                               "note": "the reference's call shape (separate input and output tensors per rank, execute_operation_async); "
@@ -295,8 +297,8 @@ def main() -> int:
     }
     if result["roofline"]["frac"] > 1:
         result["roofline"]["note"] = ("achieved counts the schedule's algorithmic bytes (35 S); the column runner executes "
-                                      "the same ops with 16 S of HBM traffic (forwarded values and dead partial writes "
-                                      "stay in registers), so hbm_frac, not frac, is the memory system's utilisation")
+                                      "the same ops with 16 S of HBM traffic (forwarded values and re-read partial results "
+                                      "stay in registers and LDS), so hbm_frac, not frac, is the memory system's utilisation")
     if args.gpu_inputs:
         result["data"] = "synthetic (GPU generator: tuning run)"
     if traffic:
