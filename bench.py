@@ -93,6 +93,27 @@ def sha256_of(t) -> str:
     return h.hexdigest()
 
 
+def device_info(dev) -> dict:
+    """Name, CU count and - best effort, through rocm-smi - the clocks and power cap of the GPU."""
+    import re
+    import subprocess
+    import torch
+    props = torch.cuda.get_device_properties(dev)
+    info = {"name": props.name, "compute_units": props.multi_processor_count,
+            "hbm_gib": round(props.total_memory / 2**30, 1), "sclk_mhz": None, "mclk_mhz": None, "power_cap_w": None}
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks", "--showmaxpower"], capture_output=True, text=True,
+                             timeout=20).stdout
+        for key, pat in (("sclk_mhz", r"sclk clock level: \S+ \((\d+)Mhz\)"), ("mclk_mhz", r"mclk clock level: \S+ \((\d+)Mhz\)"),
+                         ("power_cap_w", r"Max Graphics Package Power \(W\): ([\d.]+)")):
+            m = re.search(pat, out)
+            if m:
+                info[key] = float(m.group(1))
+    except (OSError, subprocess.SubprocessError):
+        pass
+    return info
+
+
 def cpu_baseline(sample_elems: int, channels: int, reps: int = 3):
     """Time the CPU oracle on the same graph shape at `sample_elems` elements per rank."""
     import numpy as np
@@ -194,9 +215,16 @@ def main() -> int:
     log(f"inputs generated in {time.perf_counter() - t0:.1f} s")
     bufs = [p.clone() for p in pristine]
 
+    # the first execution in the process (tables just uploaded, nothing of the buffers in any cache)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    eng.execute_inplace("bench", bufs)
+    c1.record()
+    torch.cuda.synchronize()
+    cold_ms = c0.elapsed_time(c1)
+
     verify = {}
     if not args.no_verify:
-        eng.execute_inplace("bench", bufs, sync=True)
         same = all(torch.equal(bufs[0].view(torch.int16), b.view(torch.int16)) for b in bufs[1:])
         want = ring_expected(pristine, n, channels)
         exact = torch.equal(want.view(torch.int16), bufs[0].view(torch.int16))
@@ -288,11 +316,13 @@ def main() -> int:
                      "frac": round(achieved / PEAK_GBPS, 4), "traffic": traffic,
                      "kernel_ms_avg": round(avg_ms, 4), "kernel_ms_min": round(min(kern_ms), 4),
                      "kernel_ms_median": round(sorted(kern_ms)[len(kern_ms) // 2], 4),
+                     "kernel_ms_first_execution": round(cold_ms, 4),
                      "planned_load_bytes": info["column_load_bytes"], "planned_store_bytes": info["column_store_bytes"]},
         "end_to_end_staged": {"ms_per_call": round(staged_ms, 4), "GB/s": round(alg_bytes / (staged_ms * 1e-3) / 1e9, 1),
                               "note": "the reference's call shape (separate input and output tensors per rank, execute_operation_async); "
                                       "the staging copies are fused into the program, so this is again one launch"},
         "op_by_op": op_by_op,
+        "device": device_info(dev),
         "verify": verify,
     }
     if result["roofline"]["frac"] > 1:

@@ -294,7 +294,7 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
                 tiles += (last_vec - d.first_vec + 1 + tile_v - 1) / tile_v;
                 d.prog_start = s.prog_start; d.prog_len = s.prog_len;
                 d.pre_start = s.pre_start; d.pre_words = s.pre_words;
-                d.streaming = 1; d.pad_ = 0;
+                d.streaming = 1; d.pad_ = 0; d.bcast_mask = s.bcast_mask;
                 for (int k = 0; k < s.prog_len; ++k) {
                     const ColInstr& in = P.col_instrs[s.prog_start + k];
                     if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || (in.store & STORE_KIND) == 1) d.streaming = 0;

@@ -22,6 +22,7 @@ struct DevColSegment {
     int32_t pre_start, pre_words;   // first-touch rank list, 8 ranks per 64-bit word (0xFF = none)
     int32_t streaming;       // 1: every load is a first touch and every live store is final
     int32_t pad_;
+    uint64_t bcast_mask;     // ranks that receive the accumulator after the last instruction
 };
 
 struct DevStepOp {

@@ -419,8 +419,29 @@ __device__ __forceinline__ ColInstrDev unpack_instr(uint64_t w) {
     return i;
 }
 
+// Store one value to the same position of every rank in `mask` (the broadcast tail of a program).
+// Four rank pointers are fetched per round so that their scalar loads overlap.
+template <bool NT>
+__device__ __forceinline__ void broadcast_store(uint64_t mask, const RankPtrs& ptrs, int64_t off, u32x4 v) {
+    while (mask) {
+        int r[4];
+        int n = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            r[i] = mask ? __builtin_ctzll(mask) : 0;
+            if (mask) { mask &= mask - 1; n = i + 1; }
+        }
+        char* p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[i] = ptrs.p[r[i]];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (i < n) { if (NT) stv_nt(p[i] + off, v); else stv(p[i] + off, v); }
+    }
+}
+
 template <int DT, int U, bool NT>
-__device__ __forceinline__ void column_tile(const PCCL_CONST uint64_t* prog, int prog_len, const RankPtrs& s_ptr_tab, int64_t vfirst, int tid) {
+__device__ __forceinline__ void column_tile(const PCCL_CONST uint64_t* prog, int prog_len, uint64_t bcast_mask, const RankPtrs& s_ptr_tab, int64_t vfirst, int tid) {
     char* const* s_ptr = s_ptr_tab.p;   // kernel arguments: uniform indices become scalar loads
     int64_t off[U];
 #pragma unroll
@@ -461,6 +482,10 @@ __device__ __forceinline__ void column_tile(const PCCL_CONST uint64_t* prog, int
             for (int u = 0; u < U; ++u) { if (NT) stv_nt(self + off[u], acc[u]); else stv(self + off[u], acc[u]); }
         }
     }
+    if (bcast_mask) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) broadcast_store<NT>(bcast_mask, s_ptr_tab, off[u], acc[u]);
+    }
 }
 
 // A tile that the segment boundary cuts: whole vectors inside the segment run the program on
@@ -488,6 +513,7 @@ __device__ __forceinline__ void column_edge_tile(const DevColSegment& seg, const
                 } else acc = a;
                 if (in.store & 3) stv(s_ptr[in.self] + o, acc);
             }
+            for (uint64_t m = seg.bcast_mask; m; m &= m - 1) stv(s_ptr[__builtin_ctzll(m)] + o, acc);
         } else {
             for (int64_t e = e0; e < e1; ++e) {
                 int64_t o = e * ES;
@@ -501,6 +527,7 @@ __device__ __forceinline__ void column_edge_tile(const DevColSegment& seg, const
                     } else acc = a;
                     if (in.store & 3) store_elem<DT>(s_ptr[in.self] + o, acc);
                 }
+                for (uint64_t m = seg.bcast_mask; m; m &= m - 1) store_elem<DT>(s_ptr[__builtin_ctzll(m)] + o, acc);
             }
         }
     }
@@ -534,8 +561,8 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
             // A segment whose every load is a first touch and whose every live store is final is
             // pure streaming: run it with non-temporal accesses throughout (a separate loop
             // instance, so the cache-policy hints cannot be merged away with the cached forms).
-            if (seg.streaming) column_tile<DT, U, true>(prog, seg.prog_len, ptrs, vfirst, tid);
-            else column_tile<DT, U, false>(prog, seg.prog_len, ptrs, vfirst, tid);
+            if (seg.streaming) column_tile<DT, U, true>(prog, seg.prog_len, seg.bcast_mask, ptrs, vfirst, tid);
+            else column_tile<DT, U, false>(prog, seg.prog_len, seg.bcast_mask, ptrs, vfirst, tid);
         } else {
             column_edge_tile<DT>(seg, prog, ptrs, vfirst, TILE_V, tid, kThreads);
         }
@@ -636,6 +663,7 @@ __global__ __launch_bounds__(kThreads) void column_slot_kernel(ColumnLaunch L, R
                 if (kind == 2 || (kind == 1 && (in.store & 4))) stv_nt(ptrs.p[in.self] + off, acc);
             }
         }
+        if (seg.bcast_mask) broadcast_store<true>(seg.bcast_mask, ptrs, off, acc);
     }
 }
 

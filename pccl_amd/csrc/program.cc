@@ -50,6 +50,35 @@ static void finish_column_program(Program& P, ColSegment& seg, std::vector<ColIn
         if (!(seen >> prog[n].self & 1)) prog[n].store |= STORE_LAST;
         seen |= 1ull << prog[n].self;
     }
+    // Broadcast tail: allreduce-type programs end with a run of copies that all carry the same
+    // value (the ring's allgather phase, the tree's broadcast).  Keep the first of them - after it
+    // the accumulator holds that value - and turn the rest into one mask of ranks to store it to.
+    {
+        std::vector<int> cur(64);
+        for (int r = 0; r < 64; ++r) cur[r] = r;          // value ids: the original contents
+        int next_id = 64;
+        std::vector<int> out(prog.size());
+        for (size_t n = 0; n < prog.size(); ++n) {
+            out[n] = prog[n].b_src == SRC_NONE ? cur[prog[n].peer] : next_id++;
+            cur[prog[n].self] = out[n];
+        }
+        size_t s0 = prog.size();
+        while (s0 > 0 && prog[s0 - 1].b_src == SRC_NONE && out[s0 - 1] == out[prog.size() - 1]) --s0;
+        if (prog.size() - s0 >= 2) {
+            uint64_t mask = 0;
+            for (size_t n = s0 + 1; n < prog.size(); ++n) {
+                const int kind = prog[n].store & STORE_KIND;
+                if (kind == 2 || (kind == 1 && (prog[n].store & STORE_LAST))) mask |= 1ull << prog[n].self;
+            }
+            // the kept instruction: if a later copy of the run rewrites its rank (with the same
+            // value) the mask covers that rank; otherwise a live store of it is a final one
+            ColInstr& head = prog[s0];
+            if (!(head.store & STORE_LAST)) head.store = 0;
+            else if (head.store & STORE_KIND) head.store = (uint8_t)(2 | STORE_LAST);
+            prog.resize(s0 + 1);
+            seg.bcast_mask = mask;
+        }
+    }
     std::vector<uint8_t> pre;
     uint64_t listed = 0;
     auto want = [&](uint8_t r) { if (!(listed >> r & 1)) { listed |= 1ull << r; pre.push_back(r); } };
@@ -86,6 +115,9 @@ static void count_column_traffic(const Program& P, const ColSegment& seg, int es
         if (kind) *stores += bytes;
         if (kind == 2 || (kind == 1 && (in.store & STORE_LAST))) *slot_stores += bytes;
     }
+    const int tail = __builtin_popcountll(seg.bcast_mask);
+    *stores += bytes * tail;
+    *slot_stores += bytes * tail;
     for (int w = 0; w < seg.pre_words; ++w)
         for (int j = 0; j < 8; ++j)
             if ((P.col_pre[seg.pre_start + w] >> (8 * j) & 0xFF) != 0xFF) *slot_loads += bytes;
@@ -383,6 +415,7 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
             return s;
         };
         std::vector<int> prev_sig;
+        std::vector<std::vector<ColInstr>> raw_progs;   // per segment, before finish_column_program
         for (size_t i = 0; i < cover.size(); ++i) {
             if (cover[i].empty()) { prev_sig.clear(); continue; }
             std::vector<int> s = sig(cover[i]);
@@ -426,6 +459,7 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                 if (!reread) prog[n].store = 2;
             }
             seg.prog_len = (int)prog.size();
+            raw_progs.push_back(prog);            // the direct plan below starts from the unfinished form
             finish_column_program(P, seg, prog);
             P.col_instrs.insert(P.col_instrs.end(), prog.begin(), prog.end());
             P.segs.push_back(seg);
@@ -477,10 +511,8 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                 std::vector<ColInstr> prog;
                 uint64_t written = 0;
                 if (base)
-                    for (int k = 0; k < base->prog_len && valid; ++k) {
-                        ColInstr in = P.col_instrs[base->prog_start + k];
-                        in.store &= STORE_KIND;
-                        if (in.a_src == SRC_ACC && in.b_src == SRC_NONE && !in.store) continue;   // padding
+                    for (size_t k = 0; k < raw_progs[si].size() && valid; ++k) {
+                        ColInstr in = raw_progs[si][k];
                         if (in.a_src == SRC_MEM) valid = in.a_first ? in_window(in.peer) : out_window(in.peer);
                         if (valid && in.b_src == SRC_MEM) valid = in.b_first ? in_window(in.self) : out_window(in.self);
                         if (in.store && !out_window(in.self)) {

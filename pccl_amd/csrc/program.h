@@ -51,6 +51,8 @@ struct ColSegment {
     int32_t pre_start = 0, pre_words = 0;  // words in Program::col_pre: the ranks this program reads by
                                            // first touch, 8 per word (one byte each, 0xFF = none), in
                                            // program order without repeats
+    uint64_t bcast_mask = 0;               // ranks that receive the program's last value after its
+                                           // last instruction (the tail of copies of one value)
 };
 
 struct StepOpPlan {

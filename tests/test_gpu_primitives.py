@@ -112,7 +112,7 @@ def test_copy_bytes(nbytes, shift):
 def test_bad_arguments_are_errors():
     L = _lib.lib()
     x = torch.zeros(16, device="cuda")
-    assert L.pccl_hip_reduce(3, 0, x.data_ptr(), x.data_ptr(), x.data_ptr(), 4, None) == _lib.ERR_UNSUPPORTED
+    assert L.pccl_hip_reduce(17, 0, x.data_ptr(), x.data_ptr(), x.data_ptr(), 4, None) == _lib.ERR_UNSUPPORTED   # no such dtype
     assert L.pccl_hip_reduce(0, 9, x.data_ptr(), x.data_ptr(), x.data_ptr(), 4, None) == _lib.ERR_INVALID
     assert L.pccl_hip_reduce(0, 0, None, x.data_ptr(), x.data_ptr(), 4, None) == _lib.ERR_INVALID
     assert b"null" in L.pccl_hip_last_error()
