@@ -143,13 +143,22 @@ __device__ __forceinline__ uint32_t word_op(uint32_t a, uint32_t b, int redop) {
 }
 
 template <int DT>
-__device__ __forceinline__ u32x4 vec_op(u32x4 a, u32x4 b, int redop) {
+__device__ __forceinline__ u32x4 vec_op_words(u32x4 a, u32x4 b, int redop) {
     u32x4 r;
     r.x = word_op<DT>(a.x, b.x, redop);
     r.y = word_op<DT>(a.y, b.y, redop);
     r.z = word_op<DT>(a.z, b.z, redop);
     r.w = word_op<DT>(a.w, b.w, redop);
     return r;
+}
+
+// One decision on the operator per vector: each branch below inlines the word code with a
+// constant operator, so the four words run back to back without tests in between.
+template <int DT>
+__device__ __forceinline__ u32x4 vec_op(u32x4 a, u32x4 b, int redop) {
+    if (redop == PCCL_SUM) return vec_op_words<DT>(a, b, PCCL_SUM);
+    if (redop == PCCL_MAX) return vec_op_words<DT>(a, b, PCCL_MAX);
+    return vec_op_words<DT>(a, b, PCCL_MIN);
 }
 
 // one element at byte address granularity (heads, tails, partial vectors, misaligned ranges)
