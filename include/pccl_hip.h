@@ -147,6 +147,8 @@ typedef struct {
     int64_t column_store_bytes;
     int32_t num_items;          /* stepwise plan: (op, tile) work items */
     int32_t reserved_;
+    int64_t staged_load_bytes;  /* the same for a staged call that runs on the caller's tensors */
+    int64_t staged_store_bytes; /* (0 when the graph has no such plan and staging copies are used) */
 } pccl_program_info;
 
 /* One data op of the linked program, for inspection and tests. */

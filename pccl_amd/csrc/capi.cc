@@ -61,6 +61,8 @@ void fill_info(const Program& p, pccl_program_info* out) {
     out->column_load_bytes = p.column_load_bytes;
     out->column_store_bytes = p.column_store_bytes;
     out->num_items = (int)p.num_items;
+    out->staged_load_bytes = p.direct_load_bytes;
+    out->staged_store_bytes = p.direct_store_bytes;
 }
 
 }  // namespace
@@ -710,6 +712,8 @@ int pccl_hip_op_info(pccl_hip_ctx* ctx, const char* name, pccl_program_info* out
         if (e.slot_threads > 0) {   // the traffic of the runner this context would launch
             out->column_load_bytes = e.prog.slot_load_bytes;
             out->column_store_bytes = e.prog.slot_store_bytes;
+            out->staged_load_bytes = e.prog.direct_slot_load_bytes;
+            out->staged_store_bytes = e.prog.direct_slot_store_bytes;
         }
         return 0;
     });

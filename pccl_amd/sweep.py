@@ -69,7 +69,8 @@ def run_case(label, world, jsons, make_in, out_elems, mode, reps, inplace):
                           "data_ops": info["num_data_ops"], "algorithmic_bytes": b,
                           "ms_median": round(med, 4), "ms_min": round(best, 4),
                           "GB/s": round(b / (med * 1e-3) / 1e9, 1),
-                          "planned_traffic_bytes": info["column_load_bytes"] + info["column_store_bytes"]}),
+                          "planned_traffic_bytes": (info["column_load_bytes"] + info["column_store_bytes"]) if inplace
+                          else (info["staged_load_bytes"] + info["staged_store_bytes"])}),
               flush=True)
     finally:
         eng.close()
