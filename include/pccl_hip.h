@@ -167,6 +167,32 @@ void pccl_program_free(pccl_program* p);
 int pccl_program_get_info(const pccl_program* p, pccl_program_info* out);
 int pccl_program_get_ops(const pccl_program* p, pccl_linked_op* out, int cap);
 
+/* One segment of the column plan, for inspection and tests: the element positions [start, end) share
+ * one column program, instruction words [prog_start, prog_start + prog_len) and first-touch list
+ * words [pre_start, pre_start + pre_words) of the arrays pccl_program_get_column returns.  An
+ * instruction word holds, from the low byte up: self rank, peer rank, source of a (1 memory,
+ * 2 accumulator), source of b (0 none = copy, 1 memory, 2 accumulator), reduce operator, store (low
+ * two bits: 0 dead, 1 read back later, 2 final; bit 2: last write of that rank), a is a first
+ * touch, b is a first touch.  A first-touch word lists 8 ranks, one per byte, 0xFF = none.
+ * bcast_mask: ranks that receive the accumulator after the last instruction.  The windows say which
+ * positions of rank r a staged call reads from its input tensor and hands back in its output. */
+typedef struct {
+    int64_t start, end;
+    int32_t prog_start, prog_len;
+    int32_t pre_start, pre_words;
+    uint64_t bcast_mask;
+} pccl_column_segment;
+
+/* which = 0: the in-place plan; 1: the plan of a staged call that runs on the caller's tensors
+ * (no segments when the graph has none).  Each array is filled up to its capacity; the three
+ * counts needed are returned through n_segs / n_instrs / n_pre.  in_window / out_window (which = 1,
+ * may be NULL) receive 2 * num_vranks values: start and end per rank.  No reference counterpart. */
+int pccl_program_get_column(const pccl_program* p, int which,
+                            pccl_column_segment* segs, int seg_cap, int* n_segs,
+                            uint64_t* instrs, int instr_cap, int* n_instrs,
+                            uint64_t* pre, int pre_cap, int* n_pre,
+                            int64_t* in_window, int64_t* out_window);
+
 /* ------------------------------------------------------------------------------------------
  * Device executor.
  * ------------------------------------------------------------------------------------------ */

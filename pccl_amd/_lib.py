@@ -55,6 +55,12 @@ class ProgramInfo(ctypes.Structure):
         return {n: getattr(self, n) for n, _ in self._fields_ if not n.endswith("_")}
 
 
+class ColumnSegment(ctypes.Structure):
+    _fields_ = [("start", ctypes.c_int64), ("end", ctypes.c_int64), ("prog_start", ctypes.c_int32),
+                ("prog_len", ctypes.c_int32), ("pre_start", ctypes.c_int32), ("pre_words", ctypes.c_int32),
+                ("bcast_mask", ctypes.c_uint64)]
+
+
 class LinkedOp(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("rank", "channel", "op_index", "is_reduce", "redop",
                                               "peer_rank", "level", "num_deps")] + \
@@ -75,7 +81,8 @@ EXPORTS = [
     "pccl_graph_load_file", "pccl_graph_load_json", "pccl_graph_from_triggers", "pccl_graph_free",
     "pccl_graph_num_ops", "pccl_graph_dtype", "pccl_graph_tensor_elems", "pccl_graph_collective_type",
     "pccl_graph_get_triggers", "pccl_graph_get_meta", "pccl_graph_fused_steps", "pccl_program_link",
-    "pccl_program_free", "pccl_program_get_info", "pccl_program_get_ops", "pccl_hip_create",
+    "pccl_program_free", "pccl_program_get_info", "pccl_program_get_ops", "pccl_program_get_column",
+    "pccl_hip_create",
     "pccl_hip_destroy", "pccl_hip_register_file", "pccl_hip_register_json", "pccl_hip_register_triggers",
     "pccl_hip_set_option", "pccl_hip_execute", "pccl_hip_execute_inplace", "pccl_hip_sync",
     "pccl_hip_reset_signals", "pccl_hip_op_info", "pccl_hip_last_kernel_ms", "pccl_hip_reduce",
@@ -115,6 +122,8 @@ def lib() -> ctypes.CDLL:
         "pccl_program_free": (None, [vp]),
         "pccl_program_get_info": (i32, [vp, P(ProgramInfo)]),
         "pccl_program_get_ops": (i32, [vp, P(LinkedOp), i32]),
+        "pccl_program_get_column": (i32, [vp, i32, P(ColumnSegment), i32, P(ctypes.c_int), P(ctypes.c_uint64), i32,
+                                          P(ctypes.c_int), P(ctypes.c_uint64), i32, P(ctypes.c_int), P(i64), P(i64)]),
         "pccl_hip_create": (i32, [P(vp), i32, i32]),
         "pccl_hip_destroy": (i32, [vp]),
         "pccl_hip_register_file": (i32, [vp, cp, i32, cp]),
@@ -234,6 +243,26 @@ class HostProgram:
         out = ProgramInfo()
         check(lib().pccl_program_get_info(self._h, ctypes.byref(out)))
         return out.as_dict()
+
+    def column_plan(self, staged: bool = False) -> dict:
+        """Segments, instruction words and first-touch lists of the column plan (in place, or of a
+        staged call that runs on the caller's tensors), plus the staged windows per rank."""
+        L = lib()
+        ns, ni, npre = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        which = 1 if staged else 0
+        check(L.pccl_program_get_column(self._h, which, None, 0, ctypes.byref(ns), None, 0, ctypes.byref(ni),
+                                        None, 0, ctypes.byref(npre), None, None))
+        R = self.info()["num_vranks"]
+        segs = (ColumnSegment * max(ns.value, 1))()
+        instrs = (ctypes.c_uint64 * max(ni.value, 1))()
+        pre = (ctypes.c_uint64 * max(npre.value, 1))()
+        win_in, win_out = (ctypes.c_int64 * (2 * R))(), (ctypes.c_int64 * (2 * R))()
+        check(L.pccl_program_get_column(self._h, which, segs, ns.value, ctypes.byref(ns), instrs, ni.value,
+                                        ctypes.byref(ni), pre, npre.value, ctypes.byref(npre), win_in, win_out))
+        return {"segments": [segs[i] for i in range(ns.value)], "instrs": list(instrs)[:ni.value],
+                "pre": list(pre)[:npre.value],
+                "in_window": [(win_in[2 * r], win_in[2 * r + 1]) for r in range(R)],
+                "out_window": [(win_out[2 * r], win_out[2 * r + 1]) for r in range(R)]}
 
     def ops(self):
         n = self.info()["num_data_ops"]

@@ -178,6 +178,33 @@ int pccl_program_get_ops(const pccl_program* p, pccl_linked_op* out, int cap) {
     return (int)p->p.ops.size();
 }
 
+int pccl_program_get_column(const pccl_program* p, int which,
+                            pccl_column_segment* segs, int seg_cap, int* n_segs,
+                            uint64_t* instrs, int instr_cap, int* n_instrs,
+                            uint64_t* pre, int pre_cap, int* n_pre,
+                            int64_t* in_window, int64_t* out_window) {
+    if (!p || !n_segs || !n_instrs || !n_pre) return fail(PCCL_ERR_INVALID, "null argument");
+    if (which != 0 && which != 1) return fail(PCCL_ERR_INVALID, "which must be 0 (in place) or 1 (staged)");
+    const Program& P = p->p;
+    const std::vector<ColSegment>& src = which ? P.direct_segs : P.segs;
+    *n_segs = (int)src.size(); *n_instrs = (int)P.col_instrs.size(); *n_pre = (int)P.col_pre.size();
+    for (int i = 0; segs && i < seg_cap && i < (int)src.size(); ++i) {
+        segs[i].start = src[i].start; segs[i].end = src[i].end;
+        segs[i].prog_start = src[i].prog_start; segs[i].prog_len = src[i].prog_len;
+        segs[i].pre_start = src[i].pre_start; segs[i].pre_words = src[i].pre_words;
+        segs[i].bcast_mask = src[i].bcast_mask;
+    }
+    static_assert(sizeof(ColInstr) == sizeof(uint64_t), "instruction words");
+    if (instrs) std::memcpy(instrs, P.col_instrs.data(), sizeof(uint64_t) * std::min<size_t>(instr_cap, P.col_instrs.size()));
+    if (pre) std::memcpy(pre, P.col_pre.data(), sizeof(uint64_t) * std::min<size_t>(pre_cap, P.col_pre.size()));
+    if (which == 1 && !P.direct_segs.empty())
+        for (int r = 0; r < P.R; ++r) {
+            if (in_window) { in_window[2 * r] = P.direct_in_start[r]; in_window[2 * r + 1] = P.direct_in_end[r]; }
+            if (out_window) { out_window[2 * r] = P.direct_out_start[r]; out_window[2 * r + 1] = P.direct_out_end[r]; }
+        }
+    return 0;
+}
+
 }  // extern "C"
 
 // ------------------------------------------------------------------------------- device context
