@@ -185,3 +185,76 @@ def test_kernel_timing_option(engine_factory):
     ms = eng.last_kernel_ms("t")
     eng.set_option("timing", 0)
     assert 0.0 < ms < 50.0
+
+
+def test_registration_from_trigger_arrays(engine_factory):
+    """What a C++ engine that parses the JSON itself would hand over: the 32-byte triggers and the
+    88-byte metadata records (reference proxy_trigger.h:8-16, primitive.h:8-17)."""
+    from pccl_amd import _lib
+    from pccl_amd._lib import HostGraph
+    world, n = 4, 1 << 13
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2)
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        g = HostGraph.from_json(j)
+        trig, cnt = g.triggers()
+        meta, _ = g.meta()
+        _lib.check(eng._L.pccl_hip_register_triggers(eng._h, b"trig", r, trig, meta, cnt, b"allreduce"))
+    x = seeded_inputs("randn", world, n, "bfloat16", seed=8)
+    want = oracle_buffers(jsons, x, "bfloat16")
+    outs = eng.execute_operation("trig", [t.cuda() for t in x])
+    for r in range(world):
+        assert bits_equal(outs[r], want[r])
+
+
+def test_reregistration_replaces_the_operation_and_operations_share_the_rank_buffers(engine_factory):
+    """Registering a name again replaces its graphs (the next execution links the new ones); every
+    operation of an engine aliases the same rank buffers (reference engine_c.cc:191-196), which grow
+    with the largest graph registered and keep working for the smaller ones."""
+    world = 4
+    eng = engine_factory(world)
+    eng.set_option("fuse_staging", 0)           # go through the engine's rank buffers
+    try:
+        cases = {}
+        for name, alg, n, dtype in (("a", "ring", 1 << 12, "float32"), ("b", "rhd", 1 << 16, "float32")):
+            jsons = graph_jsons(alg, "build_allreduce", world, n, dtype, "sm", 1)
+            for r, j in enumerate(jsons):
+                eng.register_operation_json(name, j, r)
+            x = seeded_inputs("randn", world, n, dtype, seed=len(cases) + 1)
+            cases[name] = (jsons, x, oracle_buffers(jsons, x, dtype))
+        for name in ("a", "b", "a", "b"):
+            jsons, x, want = cases[name]
+            outs = eng.execute_operation(name, [t.cuda() for t in x])
+            assert all(bits_equal(o, w) for o, w in zip(outs, want)), name
+        # replace "a" by a tree on a different size
+        n2 = 3000
+        jsons = graph_jsons("tree", "build_allreduce", world, n2, "float32", "sm", 1)
+        for r, j in enumerate(jsons):
+            eng.register_operation_json("a", j, r)
+        x = seeded_inputs("uniform", world, n2, "float32", seed=9)
+        want = oracle_buffers(jsons, x, "float32")
+        outs = eng.execute_operation("a", [t.cuda() for t in x])
+        assert all(bits_equal(o, w) for o, w in zip(outs, want))
+        assert eng.op_info("a")["num_data_ops"] == 2 * (world - 1)
+        jsons_b, xb, want_b = cases["b"]
+        outs = eng.execute_operation("b", [t.cuda() for t in xb])
+        assert all(bits_equal(o, w) for o, w in zip(outs, want_b))
+    finally:
+        eng.set_option("fuse_staging", 1)
+
+
+def test_executions_follow_the_callers_stream(engine_factory):
+    """Kernels are enqueued on the current torch stream (reference cuda_device.cc:245-248,301): work
+    queued on a side stream before and after the call is ordered with it."""
+    world, n = 2, 1 << 20
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("s", j, r)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        x = [torch.full((n,), float(r + 1), device="cuda") for r in range(world)]   # produced on the side stream
+        outs = eng.execute_operation_async("s", x)
+        y = outs[0] * 2                                                             # consumed on it
+    side.synchronize()
+    assert torch.all(y == 6) and torch.all(outs[1] == 3)
