@@ -220,7 +220,10 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * the output tensors directly instead of staging through the engine's rank buffers);
  * "lds_slots" = "1" | "0" (column runner keeps values it re-reads in per-thread LDS slots, so each
  * rank buffer is read and written at most once per position; "0" re-reads them through memory);
- * "slot_threads" = 0 | 64 | 128 | 256 (workgroup size of that runner, 0 = from the rank count). */
+ * "slot_threads" = 0 | 64 | 128 | 256 (workgroup size of that runner, 0 = from the rank count);
+ * "slot_direct" = "1" | "0" (first touches loaded straight into LDS, or through registers);
+ * "level_graph" = "0" | "1" (the level runner launches level by level, or replays the launches of an
+ * execution as one HIP graph captured per set of rank pointers). */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
 
 /* Engine::exeOp / exeOpAsync (reference csrc/engine_c.cc:269-560): for every virtual rank r copy

@@ -238,7 +238,22 @@ struct OpEntry {
     int epoch = 0;                        // persistent runner: launches so far
     uint32_t ticket_base = 0;             // persistent runner: tickets consumed so far
     std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
+    // Level runner: the launches of one execution captured as a HIP graph, per set of rank
+    // pointers (kernel arguments are frozen at capture time).  A handful are kept.
+    struct LevelGraph { std::vector<char*> key; hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; uint64_t used = 0; };
+    std::vector<LevelGraph> level_graphs;
+    uint64_t graph_clock = 0;
+    bool graph_failed = false;            // capture did not work once: launch level by level from then on
+    void drop_graphs() {
+        for (auto& g : level_graphs) {
+            if (g.exec) (void)hipGraphExecDestroy(g.exec);
+            if (g.graph) (void)hipGraphDestroy(g.graph);
+        }
+        level_graphs.clear();
+    }
     void release() {
+        drop_graphs();
+        graph_failed = false;
         segs.release(); direct_segs.release(); instrs.release(); pre.release(); step_ops.release(); step_deps.release();
         item_op.release(); state.release();
         if (ev0) (void)hipEventDestroy(ev0);
@@ -267,6 +282,9 @@ struct pccl_hip_ctx {
     bool lds_slots = true;                // column runner keeps re-read values in LDS slots
     int slot_threads = 0;                 // slot runner workgroup size (0: chosen from the rank count)
     bool slot_direct = true;              // slot runner fetches first touches straight into LDS
+    bool level_graph = false;             // level runner replays its launches as one HIP graph (measured:
+                                          // no faster than launching level by level, so off by default)
+    hipStream_t capture_stream = nullptr; // private stream the level launches are captured on
     int64_t step_tile_bytes = 128 * 1024;
     bool fuse_staging = true;             // run staged calls on the caller's tensors when possible
     int wait_timeout_ms = 2000;           // a persistent launch gives up on a dependency after this long
@@ -426,7 +444,51 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
             e.ran_persistent = true;
         } else {
             rc = 0;
-            for (size_t l = 0; l + 1 < e.level_item_begin.size() && rc == 0; ++l)
+            const size_t nlevels = e.level_item_begin.size() - 1;
+            bool done = false;
+            if (ctx->level_graph && !e.graph_failed && nlevels >= 2) {
+                // one graph launch instead of one kernel launch per level; the graph holds only
+                // kernel nodes (no memset nodes) and is bound to this set of rank pointers
+                std::vector<char*> key(rank_bufs, rank_bufs + ctx->R);
+                OpEntry::LevelGraph* hit = nullptr;
+                for (auto& g : e.level_graphs) if (g.key == key) hit = &g;
+                if (!hit) {
+                    if (!ctx->capture_stream) HIP_TRY(hipStreamCreateWithFlags(&ctx->capture_stream, hipStreamNonBlocking));
+                    OpEntry::LevelGraph g;
+                    g.key = key;
+                    hipError_t st = hipStreamBeginCapture(ctx->capture_stream, hipStreamCaptureModeThreadLocal);
+                    if (st == hipSuccess) {
+                        int lrc = 0;
+                        for (size_t l = 0; l < nlevels && lrc == 0; ++l)
+                            lrc = launch_level(L, e.level_item_begin[l], e.level_item_begin[l + 1], ptrs, ctx->capture_stream);
+                        st = hipStreamEndCapture(ctx->capture_stream, &g.graph);
+                        if (st == hipSuccess && lrc != 0) st = (hipError_t)lrc;
+                    }
+                    if (st == hipSuccess) st = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
+                    if (st != hipSuccess) {
+                        if (g.exec) (void)hipGraphExecDestroy(g.exec);
+                        if (g.graph) (void)hipGraphDestroy(g.graph);
+                        (void)hipGetLastError();
+                        e.graph_failed = true;
+                    } else {
+                        if (e.level_graphs.size() >= 4) {   // forget the least recently used
+                            size_t old = 0;
+                            for (size_t i = 1; i < e.level_graphs.size(); ++i) if (e.level_graphs[i].used < e.level_graphs[old].used) old = i;
+                            (void)hipGraphExecDestroy(e.level_graphs[old].exec);
+                            (void)hipGraphDestroy(e.level_graphs[old].graph);
+                            e.level_graphs.erase(e.level_graphs.begin() + old);
+                        }
+                        e.level_graphs.push_back(g);
+                        hit = &e.level_graphs.back();
+                    }
+                }
+                if (hit) {
+                    hit->used = ++e.graph_clock;
+                    rc = (int)hipGraphLaunch(hit->exec, stream);
+                    done = true;
+                }
+            }
+            for (size_t l = 0; !done && l < nlevels && rc == 0; ++l)
                 rc = launch_level(L, e.level_item_begin[l], e.level_item_begin[l + 1], ptrs, stream);
         }
     }
@@ -539,6 +601,7 @@ int pccl_hip_destroy(pccl_hip_ctx* ctx) {
     (void)hipDeviceSynchronize();
     for (auto& kv : ctx->ops) kv.second.release();
     for (char* b : ctx->bufs) if (b) (void)hipFree(b);
+    if (ctx->capture_stream) (void)hipStreamDestroy(ctx->capture_stream);
     delete ctx;
     return 0;
 }
@@ -588,6 +651,7 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             if (u != 1 && u != 2 && u != 4) return fail(PCCL_ERR_INVALID, "vecs_per_thread must be 1, 2 or 4");
             ctx->vecs_per_thread = u; relink = true;
         } else if (k == "slot_direct") ctx->slot_direct = std::atoi(value) != 0;
+        else if (k == "level_graph") ctx->level_graph = std::atoi(value) != 0;
         else if (k == "lds_slots") { ctx->lds_slots = std::atoi(value) != 0; relink = true; }
         else if (k == "slot_threads") {
             int t = std::atoi(value);

@@ -145,3 +145,42 @@ def test_channelized_chain(engine_factory):
     for r in range(world):
         assert bits_equal(got[r], want[r]), mismatch_report(got[r], want[r])
         assert bits_equal(got[r][pieces * chunk:], x[1 - r][:pieces * chunk])
+
+
+@pytest.mark.parametrize("alg,world,n,dtype", [("ring", 8, 1 << 16, "bfloat16"), ("tree", 8, 5000, "float32")])
+def test_level_runner_graph_replays(engine_factory, alg, world, n, dtype):
+    """The level runner captures the launches of one execution as a HIP graph per set of rank
+    pointers.  Every replay - with other GPU work and synchronisations of the program in between,
+    on fresh data in the same tensors, and on a second set of tensors - must give what launching
+    level by level gives."""
+    jsons = graph_jsons(alg, "build_allreduce", world, n, dtype, "sm", 1)
+    engine = engine_factory(world)
+    for r, j in enumerate(jsons):
+        engine.register_operation_json("g", j, r)
+    engine.set_option("mode", "stepwise")
+    sets = [[torch.empty(n, dtype=seeded_inputs("randn", 1, 1, dtype)[0].dtype, device="cuda") for _ in range(world)]
+            for _ in range(2)]
+    scratch = torch.zeros(1 << 20, device="cuda")
+    for rep in range(6):
+        x = seeded_inputs("randn", world, n, dtype, seed=100 + rep)
+        want = oracle_buffers(jsons, x, dtype)
+        bufs = sets[rep % 2]
+        engine.set_option("level_graph", 0 if rep == 4 else 1)      # one eager execution in the middle
+        for b, t in zip(bufs, x):
+            b.copy_(t)
+        scratch.add_(1.0)                        # unrelated eager work on the same stream
+        engine.execute_inplace("g", bufs)
+        total = scratch.sum()                    # a library reduction between the replays
+        torch.cuda.synchronize()
+        assert total.item() == (rep + 1) * (1 << 20)
+        for r in range(world):
+            assert bits_equal(bufs[r], want[r]), f"replay {rep}, rank {r}: {mismatch_report(bufs[r], want[r])}"
+    engine.set_option("level_graph", 1)
+    # staged calls in this mode go through the engine's rank buffers: one more pointer set
+    x = seeded_inputs("randn", world, n, dtype, seed=55)
+    want = oracle_buffers(jsons, x, dtype)
+    for _ in range(2):
+        outs = engine.execute_operation("g", [t.cuda() for t in x])
+        for r in range(world):
+            assert bits_equal(outs[r], want[r])
+    engine.set_option("level_graph", 0)
