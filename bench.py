@@ -144,6 +144,8 @@ def measured_traffic(mode: str, levels: int):
     """HBM bytes per execution of the headline graph from the committed rocprofv3 counter summaries
     (FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy): one launch of the column kernel, or one launch
     per dependency level of the level kernel."""
+    if mode == "persistent":
+        return None
     kernel = "level_kernel" if mode == "stepwise" else "column_slot_kernel"
     path = os.path.join(ROOT, "profiles", f"{kernel}_ring_allreduce_R8_bf16_512MiB.traffic.json")
     try:

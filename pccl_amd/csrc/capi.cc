@@ -635,11 +635,7 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             if (v == "auto") ctx->mode = Mode::Auto;
             else if (v == "column") ctx->mode = Mode::Column;
             else if (v == "stepwise") ctx->mode = Mode::Stepwise;
-            else if (v == "persistent")
-                // The single-launch flag-ordered runner never drained on MI355X in three attempts
-                // (tile counters, bounded polls, store-published per-item flags with a wall-clock
-                // bound); the cause is not established, so the mode is refused, never launched.
-                return fail(PCCL_ERR_UNSUPPORTED, "mode 'persistent' is switched off: the flag-ordered single-launch runner does not drain on MI355X (cause not yet established); use 'stepwise' or 'column'");
+            else if (v == "persistent") ctx->mode = Mode::Persistent;
             else return fail(PCCL_ERR_INVALID, "mode must be auto, column, stepwise or persistent");
         } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
         else if (k == "timing") ctx->timing = std::atoi(value) != 0;

@@ -338,34 +338,44 @@ __global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int i
 // A claimed item only ever waits for items claimed earlier by workgroups that are already running,
 // so the scheme cannot deadlock whatever the grid size.
 //
-// Cross-workgroup visibility follows the pattern the ROCm scan primitives use on multi-XCD parts:
-// one flag word per item, published with an agent-scope atomic STORE after an agent-scope release
-// fence and polled with agent-scope atomic LOADs (both bypass the per-XCD L2).  A flag holds the
-// launch epoch, so flags are never cleared; the ticket counter is never reset either (the host
-// passes the ticket of this launch's item 0).  Every wait is bounded by wall-clock time: when
-// `timeout_ticks` of the 100 MHz counter have passed since the workgroup started, the waiter
-// records (op, predecessor) and every workgroup leaves at its next claim, so the grid always
-// drains and the host reports the stall as an error.
+// Cross-workgroup visibility: one flag word per item.  After its tile every wave makes its own
+// stores visible with an agent-scope release fence, the workgroup meets at a barrier, and one
+// thread publishes the flag with an agent-scope atomic store; waiters poll with agent-scope atomic
+// loads, meet at a barrier and every thread executes an agent-scope acquire fence before it
+// touches the data.  A flag holds the launch epoch, so flags are never cleared; the ticket counter
+// is never reset either (the host passes the ticket of this launch's item 0).  Every wait is
+// bounded by wall-clock time: when `timeout_ticks` of the 100 MHz counter have passed since the
+// workgroup started, the waiter records (op, predecessor) and every workgroup leaves at its next
+// claim, so the grid always drains and the host reports the stall as an error.
+//
+// Shape of the loop (it matters): the one thread that publishes an item and claims the next does
+// both in a single block that sits between two barriers, and the claimed item is read back as a
+// wave-uniform scalar, so the loop is controlled by scalar branches.  With the claim at the top of
+// the loop and the publish at the bottom - no barrier between them across the back edge - the
+// compiler merges the two single-thread blocks and lets the other 255 threads run ahead into the
+// next iteration's barrier while the claiming lane is masked off: they re-read the old item for
+// ever and the launch never drains.
+
+__device__ __forceinline__ int claim_item(const StepwiseLaunch& L) {
+    const int stalled = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return stalled ? L.num_items : (int)(atomicAdd(&L.state->ticket, 1u) - L.ticket_base);
+}
 
 template <int DT>
 __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     constexpr int ES = ElemBytes<DT>::value;
-    __shared__ int s_item;
+    __shared__ int s_word;   // broadcast slot: the claimed item, then the stall flag
     int32_t* flags = reinterpret_cast<int32_t*>(L.state + 1);
     const int tid = threadIdx.x;
     const uint64_t t_start = __builtin_amdgcn_s_memrealtime();
-    for (;;) {
-        if (tid == 0) {
-            int stalled = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_item = stalled ? L.num_items : (int)(atomicAdd(&L.state->ticket, 1u) - L.ticket_base);
-        }
-        __syncthreads();
-        const int item = s_item;
-        __syncthreads();
-        if (item >= L.num_items || item < 0) break;
+    if (tid == 0) s_word = claim_item(L);
+    __syncthreads();
+    int item = __builtin_amdgcn_readfirstlane(s_word);
+    __syncthreads();
+    while (item >= 0 && item < L.num_items) {
         const int opi = as_const(L.item_op)[item];
         const DevStepOp op = load_const(L.ops + opi);
-        // wait: thread t watches items t, t+256, ... of each predecessor
+        // wait: thread t watches items t, t+256, ... of each predecessor (no barrier in here)
         for (int k = 0; k < op.ndeps; ++k) {
             const int d = as_const(L.deps)[op.dep_start + k];
             const int first = as_const(L.ops)[d].first_item, nt = as_const(L.ops)[d].ntiles;
@@ -386,24 +396,26 @@ __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, 
         }
         __syncthreads();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        if (tid == 0) s_item = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) s_word = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        const bool stalled = s_item != 0;
-        __syncthreads();
-        if (stalled) break;   // a predecessor never arrived: do not touch the data, just drain
-        int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
-        int64_t cnt = op.size - e0 < L.tile_elems ? op.size - e0 : L.tile_elems;
+        const int stalled = __builtin_amdgcn_readfirstlane(s_word);
+        if (stalled) break;   // a predecessor never arrived: do not touch the data, just leave
+        const int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
+        const int64_t cnt = op.size - e0 < L.tile_elems ? op.size - e0 : L.tile_elems;
         char* self = ptrs.p[op.self];
         const char* peer = ptrs.p[op.peer];
         if (op.is_reduce)
             range_op<DT, true>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
         else
             range_copy_bytes(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
-        __syncthreads();  // every wave's stores are issued and counted before the publish
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");   // every wave: its own stores are visible
+        __syncthreads();
         if (tid == 0) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             __hip_atomic_store(&flags[item], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_word = claim_item(L);
         }
+        __syncthreads();
+        item = __builtin_amdgcn_readfirstlane(s_word);
     }
 }
 
@@ -745,7 +757,8 @@ int launch_persistent(const StepwiseLaunch& L, const RankPtrs& ptrs, void* strea
         case PCCL_F16: return launch_persistent_dt<PCCL_F16>(L, ptrs, s);
         case PCCL_BF16: return launch_persistent_dt<PCCL_BF16>(L, ptrs, s);
         case PCCL_I32: return launch_persistent_dt<PCCL_I32>(L, ptrs, s);
-        case PCCL_F8E4M3: case PCCL_F8E5M2: return launch_persistent_dt<PCCL_F8E4M3>(L, ptrs, s);
+        case PCCL_F8E4M3: return launch_persistent_dt<PCCL_F8E4M3>(L, ptrs, s);
+        case PCCL_F8E5M2: return launch_persistent_dt<PCCL_F8E5M2>(L, ptrs, s);
         default: return (int)hipErrorInvalidValue;
     }
 }

@@ -48,11 +48,7 @@ CASES = [
 ]
 
 
-PERSISTENT_OFF = pytest.mark.skip(reason="the persistent flag-ordered runner never drained on MI355X in "
-                                   "three forms (tile counters, bounded polls, store-published flags "
-                                   "with a wall-clock bound); the mode is refused by the library until "
-                                   "the cause is found")
-MODES = ["column", "stepwise", pytest.param("persistent", marks=PERSISTENT_OFF)]
+MODES = ["column", "stepwise", "persistent"]
 
 
 @pytest.mark.parametrize("alg,world,n,dtype,channels,kind", CASES)
@@ -128,7 +124,7 @@ def test_reduce_scatter_and_allgather(engine_factory, mode, channels, fuse):
         engine.set_option("fuse_staging", 1)
 
 
-@pytest.mark.parametrize("mode", ["stepwise", pytest.param("persistent", marks=PERSISTENT_OFF)])
+@pytest.mark.parametrize("mode", ["stepwise", "persistent"])
 def test_alltoall(engine_factory, mode):
     """reference tests/test_correctness.py:243-272: out[i] chunk = chunk r of rank i's input."""
     world, n = 4, 1 << 12
@@ -143,12 +139,27 @@ def test_alltoall(engine_factory, mode):
         assert bits_equal(got[r], want), mismatch_report(got[r], want)
 
 
-def test_persistent_mode_is_refused(engine_factory):
-    from pccl_amd._lib import PcclError, ERR_UNSUPPORTED
-    engine = engine_factory(2)
-    with pytest.raises(PcclError) as e:
-        engine.set_option("mode", "persistent")
-    assert e.value.code == ERR_UNSUPPORTED
+def test_persistent_runner_reports_a_wait_that_expires(engine_factory):
+    """Every wait of the persistent runner is bounded: with a 1 ms bound on a program that runs
+    longer than that, some workgroup's wait on a predecessor expires; it records which, every
+    workgroup leaves at its next claim (the launch drains normally), and the call reports the stall
+    instead of hanging.  The next execution, with the bound restored, is correct."""
+    from pccl_amd._lib import PcclError
+    world, n = 8, 1 << 27           # 512 MiB per rank: the 14 levels take about 3 ms
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)
+    engine = engine_factory(world)
+    for r, j in enumerate(jsons):
+        engine.register_operation_json("slow", j, r)
+    engine.set_option("mode", "persistent")
+    engine.set_option("wait_timeout_ms", 1)
+    bufs = [torch.ones(n, device="cuda") for _ in range(world)]
+    with pytest.raises(PcclError, match="gave up waiting"):
+        engine.execute_inplace("slow", bufs, sync=True)
+    engine.set_option("wait_timeout_ms", 2000)
+    for b in bufs:
+        b.fill_(1.0)
+    engine.execute_inplace("slow", bufs, sync=True)
+    assert all(torch.all(b == world) for b in bufs)
     engine.set_option("mode", "auto")
 
 
