@@ -236,7 +236,6 @@ struct OpEntry {
     bool timed = false;
     bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
     int epoch = 0;                        // persistent runner: launches so far
-    uint32_t ticket_base = 0;             // persistent runner: tickets consumed so far
     std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
     // Level runner: the launches of one execution captured as a HIP graph, per set of rank
     // pointers (kernel arguments are frozen at capture time).  A handful are kept.
@@ -382,7 +381,7 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
         e.item_op.upload(item_op.data(), item_op.size() * sizeof(int32_t));
         std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * ((size_t)P.num_items + 1), 0);
         e.state.upload(zeros.data(), zeros.size());
-        e.epoch = 0; e.ticket_base = 0;
+        e.epoch = 0;
     }
     HIP_TRY(hipEventCreate(&e.ev0));
     HIP_TRY(hipEventCreate(&e.ev1));
@@ -433,14 +432,9 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
         L.num_items = (int)P.num_items; L.tile_elems = P.tile_elems; L.state = (StepState*)e.state.p;
         L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
         if (ctx->mode == Mode::Persistent) {
-            int grid = ctx->num_blocks > 0 ? ctx->num_blocks : device_cu_count(ctx->device) * 8;
-            if (grid > L.num_items) grid = L.num_items;
-            L.num_blocks = grid;
-            L.epoch = ++e.epoch;
-            L.ticket_base = e.ticket_base;
+            L.epoch = ++e.epoch;                 // flags of this launch carry this value; never cleared
             L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
-            e.ticket_base += (uint32_t)L.num_items + (uint32_t)grid;   // every workgroup draws one ticket past the end
-            rc = launch_persistent(L, ptrs, stream);
+            rc = launch_persistent(L, ptrs, stream);   // sizes the grid to what is resident at once
             e.ran_persistent = true;
         } else {
             rc = 0;
@@ -549,7 +543,7 @@ void check_stall(OpEntry& e, const std::string& name) {
     if (st.error_op == 0) return;
     std::vector<char> zeros(e.state.bytes, 0);
     HIP_TRY(hipMemcpy(e.state.p, zeros.data(), zeros.size(), hipMemcpyHostToDevice));
-    e.epoch = 0; e.ticket_base = 0;
+    e.epoch = 0;
     const LinkedOp& a = e.prog.ops[st.error_op - 1];
     const LinkedOp& b = e.prog.ops[st.error_dep - 1];
     throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting: data op " + std::to_string(st.error_op - 1) +
@@ -782,7 +776,7 @@ int pccl_hip_reset_signals(pccl_hip_ctx* ctx, const char* name) {
             int rc = launch_fill_zero(e.state.p, e.state.bytes, ctx->last_stream);
             if (rc) return fail(PCCL_ERR_HIP, hipGetErrorString((hipError_t)rc));
             HIP_TRY(hipStreamSynchronize(ctx->last_stream));
-            e.epoch = 0; e.ticket_base = 0;
+            e.epoch = 0;
         }
         return 0;
     });

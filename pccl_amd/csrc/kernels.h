@@ -32,7 +32,7 @@ struct DevStepOp {
 };
 
 struct StepState {      // device memory of the persistent runner
-    uint32_t ticket;    // next work ticket; never reset, the host tracks where a launch starts
+    uint32_t reserved0;
     int32_t reserved;
     int32_t error_op;   // 1 + index of the op whose bounded wait expired (0 = none); host clears it
     int32_t error_dep;  // 1 + index of the predecessor it was waiting for
@@ -66,7 +66,7 @@ struct StepwiseLaunch {
     int32_t dtype;
     int32_t num_blocks;
     int32_t epoch;            // persistent runner: value a completed item's flag takes in this launch
-    uint32_t ticket_base;     // persistent runner: ticket of this launch's item 0
+    uint32_t reserved1;
     uint64_t timeout_ticks;   // persistent runner: 100 MHz ticks a workgroup may run before a wait gives up
 };
 

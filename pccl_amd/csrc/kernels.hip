@@ -195,59 +195,104 @@ __device__ __forceinline__ void stv_nt(char* p, u32x4 v) { __builtin_nontemporal
 // c[i] = a[i] (op) b[i] (IS_REDUCE) or c[i] = a[i], i in [0, n) elements, cooperatively by
 // `nthreads` threads.  Any alignment: when the three addresses are congruent modulo 16 the body runs
 // as 128-bit loads and stores with a scalar head and tail; otherwise element by element.
+//
+// How memory is touched is a policy: cached, streaming (non-temporal: data touched once), or
+// agent-coherent.  The coherent form marks every access with the agent scope bit (sc1), the bit
+// the agent-scope atomics carry: such a store is written through to memory before it is
+// acknowledged and such a load does not hit a stale copy in this XCD's L2, so data written by a
+// workgroup on one XCD can be consumed by a workgroup on another after a flag hand-over without
+// writing back or invalidating whole caches.  128-bit accesses with that bit are expressed as raw
+// buffer operations (wave-uniform base in a resource descriptor, 32-bit byte offset per lane).
 
-template <int DT, bool IS_REDUCE, bool NT = true>
+enum { MEM_CACHED = 0, MEM_STREAM = 1, MEM_COHERENT = 2 };
+constexpr int kAuxCoherent = 16 | 2;   // sc1 | nt
+
+template <int POLICY>
+struct Mem {
+    const char* base;
+    __device__ __forceinline__ explicit Mem(const char* b) : base(b) {}
+    __device__ __forceinline__ u32x4 ldv(int64_t off) const { return POLICY == MEM_STREAM ? ldv_nt(base + off) : ::pccl_hip::ldv(base + off); }
+    __device__ __forceinline__ void stv(int64_t off, u32x4 v) const { if (POLICY == MEM_STREAM) stv_nt((char*)base + off, v); else ::pccl_hip::stv((char*)base + off, v); }
+    template <int DT> __device__ __forceinline__ uint32_t lde(int64_t off) const { return load_elem<DT>(base + off); }
+    template <int DT> __device__ __forceinline__ void ste(int64_t off, uint32_t x) const { store_elem<DT>((char*)base + off, x); }
+};
+
+template <>
+struct Mem<MEM_COHERENT> {
+    __amdgpu_buffer_rsrc_t rs;
+    __device__ __forceinline__ explicit Mem(const char* b)
+        : rs(__builtin_amdgcn_make_buffer_rsrc((void*)b, 0, 0x7FFFFFFF, 0x00020000)) {}
+    __device__ __forceinline__ u32x4 ldv(int64_t off) const { return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, kAuxCoherent); }
+    __device__ __forceinline__ void stv(int64_t off, u32x4 v) const { __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)off, 0, kAuxCoherent); }
+    template <int DT> __device__ __forceinline__ uint32_t lde(int64_t off) const {
+        constexpr int ES = ElemBytes<DT>::value;
+        if constexpr (ES == 4) return __builtin_amdgcn_raw_buffer_load_b32(rs, (int)off, 0, kAuxCoherent);
+        else if constexpr (ES == 2) return __builtin_amdgcn_raw_buffer_load_b16(rs, (int)off, 0, kAuxCoherent);
+        else return __builtin_amdgcn_raw_buffer_load_b8(rs, (int)off, 0, kAuxCoherent);
+    }
+    template <int DT> __device__ __forceinline__ void ste(int64_t off, uint32_t x) const {
+        constexpr int ES = ElemBytes<DT>::value;
+        if constexpr (ES == 4) __builtin_amdgcn_raw_buffer_store_b32(x, rs, (int)off, 0, kAuxCoherent);
+        else if constexpr (ES == 2) __builtin_amdgcn_raw_buffer_store_b16((uint16_t)x, rs, (int)off, 0, kAuxCoherent);
+        else __builtin_amdgcn_raw_buffer_store_b8((uint8_t)x, rs, (int)off, 0, kAuxCoherent);
+    }
+};
+
+// The ranges handed to the coherent form must be shorter than 2 GiB (offsets are 32-bit).
+template <int DT, bool IS_REDUCE, int POLICY = MEM_STREAM>
 __device__ __forceinline__ void range_op(const char* a, const char* b, char* c, int64_t n, int redop,
                                          int tid, int nthreads) {
-    auto ldx = [](const char* p) { if constexpr (NT) return ldv_nt(p); else return ldv(p); };
-    auto stx = [](char* p, u32x4 v) { if constexpr (NT) stv_nt(p, v); else stv(p, v); };
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
+    const Mem<POLICY> A(a), B(b), C(c);
     uintptr_t ua = (uintptr_t)a, ub = (uintptr_t)b, uc = (uintptr_t)c;
     bool congruent = ((ua ^ uc) & 15) == 0 && (!IS_REDUCE || ((ub ^ uc) & 15) == 0);
     if (!congruent) {
         for (int64_t i = tid; i < n; i += nthreads) {
-            uint32_t x = load_elem<DT>(a + i * ES);
-            if constexpr (IS_REDUCE) x = elem_op<DT>(x, load_elem<DT>(b + i * ES), redop);
-            store_elem<DT>(c + i * ES, x);
+            uint32_t x = A.template lde<DT>(i * ES);
+            if constexpr (IS_REDUCE) x = elem_op<DT>(x, B.template lde<DT>(i * ES), redop);
+            C.template ste<DT>(i * ES, x);
         }
         return;
     }
     int64_t head = (int64_t)(((16 - (uc & 15)) & 15) / ES);
     if (head > n) head = n;
     if (tid < head) {
-        uint32_t x = load_elem<DT>(a + (int64_t)tid * ES);
-        if constexpr (IS_REDUCE) x = elem_op<DT>(x, load_elem<DT>(b + (int64_t)tid * ES), redop);
-        store_elem<DT>(c + (int64_t)tid * ES, x);
+        uint32_t x = A.template lde<DT>((int64_t)tid * ES);
+        if constexpr (IS_REDUCE) x = elem_op<DT>(x, B.template lde<DT>((int64_t)tid * ES), redop);
+        C.template ste<DT>((int64_t)tid * ES, x);
     }
-    a += head * ES; b += head * ES; c += head * ES; n -= head;
+    const int64_t h = head * ES;   // byte offset of the vector body
+    n -= head;
     int64_t nvec = n / VE;
     int64_t v = tid;
     // 4 vectors per thread per trip: all loads issued before the first store
     for (; v + 3 * (int64_t)nthreads < nvec; v += 4 * (int64_t)nthreads) {
-        u32x4 x0 = ldx(a + v * 16), x1 = ldx(a + (v + nthreads) * 16), x2 = ldx(a + (v + 2 * nthreads) * 16), x3 = ldx(a + (v + 3 * nthreads) * 16);
+        const int64_t o0 = h + v * 16, o1 = h + (v + nthreads) * 16, o2 = h + (v + 2 * nthreads) * 16, o3 = h + (v + 3 * nthreads) * 16;
+        u32x4 x0 = A.ldv(o0), x1 = A.ldv(o1), x2 = A.ldv(o2), x3 = A.ldv(o3);
         if constexpr (IS_REDUCE) {
-            u32x4 y0 = ldx(b + v * 16), y1 = ldx(b + (v + nthreads) * 16), y2 = ldx(b + (v + 2 * nthreads) * 16), y3 = ldx(b + (v + 3 * nthreads) * 16);
+            u32x4 y0 = B.ldv(o0), y1 = B.ldv(o1), y2 = B.ldv(o2), y3 = B.ldv(o3);
             x0 = vec_op<DT>(x0, y0, redop); x1 = vec_op<DT>(x1, y1, redop); x2 = vec_op<DT>(x2, y2, redop); x3 = vec_op<DT>(x3, y3, redop);
         }
-        stx(c + v * 16, x0); stx(c + (v + nthreads) * 16, x1); stx(c + (v + 2 * nthreads) * 16, x2); stx(c + (v + 3 * nthreads) * 16, x3);
+        C.stv(o0, x0); C.stv(o1, x1); C.stv(o2, x2); C.stv(o3, x3);
     }
     for (; v < nvec; v += nthreads) {
-        u32x4 x = ldx(a + v * 16);
-        if constexpr (IS_REDUCE) x = vec_op<DT>(x, ldx(b + v * 16), redop);
-        stx(c + v * 16, x);
+        u32x4 x = A.ldv(h + v * 16);
+        if constexpr (IS_REDUCE) x = vec_op<DT>(x, B.ldv(h + v * 16), redop);
+        C.stv(h + v * 16, x);
     }
     int64_t tail0 = nvec * VE;
     for (int64_t i = tail0 + tid; i < n; i += nthreads) {
-        uint32_t x = load_elem<DT>(a + i * ES);
-        if constexpr (IS_REDUCE) x = elem_op<DT>(x, load_elem<DT>(b + i * ES), redop);
-        store_elem<DT>(c + i * ES, x);
+        uint32_t x = A.template lde<DT>(h + i * ES);
+        if constexpr (IS_REDUCE) x = elem_op<DT>(x, B.template lde<DT>(h + i * ES), redop);
+        C.template ste<DT>(h + i * ES, x);
     }
 }
 
 // byte copy with the same structure (used by copies of every dtype and by staging)
+template <int POLICY = MEM_STREAM>
 __device__ __forceinline__ void range_copy_bytes(const char* a, char* c, int64_t nbytes, int tid, int nthreads) {
-    range_op<PCCL_F8E4M3, false>(a, nullptr, c, nbytes, 0, tid, nthreads);
+    range_op<PCCL_F8E4M3, false, POLICY>(a, nullptr, c, nbytes, 0, tid, nthreads);
 }
 
 template <int DT>
@@ -333,46 +378,43 @@ __global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int i
 // ------------------------------------------------------------------------------- persistent runner
 //
 // One persistent launch executes every data op of the linked program.  Work items are (op, tile)
-// pairs in level order; a workgroup takes the next item from one atomic ticket counter, waits
-// until every item of the op's predecessors has been published, runs the item, then publishes it.
-// A claimed item only ever waits for items claimed earlier by workgroups that are already running,
-// so the scheme cannot deadlock whatever the grid size.
+// pairs in level order, dealt round-robin to the workgroups: workgroup b runs items b, b + G,
+// b + 2G, ... in that order, waits before each until every item of the op's predecessors has been
+// published, runs it, then publishes it.  An item only ever waits for items with smaller numbers,
+// and every workgroup works through its items in increasing order, so the scheme cannot deadlock
+// as long as all G workgroups are resident at once; the launcher sizes G from the occupancy the
+// runtime reports.  (Handing out items through one atomic ticket counter instead cost about 90 ns
+// per item - same-address atomics from 8 XCDs are serialised - which more than doubled the time
+// of the headline graph.)
 //
-// Cross-workgroup visibility: one flag word per item.  After its tile every wave makes its own
-// stores visible with an agent-scope release fence, the workgroup meets at a barrier, and one
-// thread publishes the flag with an agent-scope atomic store; waiters poll with agent-scope atomic
-// loads, meet at a barrier and every thread executes an agent-scope acquire fence before it
-// touches the data.  A flag holds the launch epoch, so flags are never cleared; the ticket counter
-// is never reset either (the host passes the ticket of this launch's item 0).  Every wait is
-// bounded by wall-clock time: when `timeout_ticks` of the 100 MHz counter have passed since the
-// workgroup started, the waiter records (op, predecessor) and every workgroup leaves at its next
-// claim, so the grid always drains and the host reports the stall as an error.
+// Cross-workgroup visibility: one flag word per item.  All data accesses of this kernel are
+// agent-coherent (see Mem<MEM_COHERENT>), so handing an item over needs no cache-wide operation:
+// every wave waits until its stores have been acknowledged, the workgroup meets at a barrier, and
+// one thread publishes the flag with an agent-scope atomic store; waiters poll with agent-scope
+// atomic loads and meet at a barrier before they touch the data.  (With cached data accesses and
+// an agent-scope release / acquire fence per wave and item - a write-back and an invalidation of
+// the XCD's whole L2 each - the headline graph took 16 ms instead of 3.)  A flag holds the launch
+// epoch, so flags are never cleared.  Every wait is bounded by wall-clock time: when
+// `timeout_ticks` of the 100 MHz counter have passed since the workgroup started, the waiter
+// records (op, predecessor) and every workgroup leaves before its next item, so the grid always
+// drains and the host reports the stall as an error.
 //
-// Shape of the loop (it matters): the one thread that publishes an item and claims the next does
-// both in a single block that sits between two barriers, and the claimed item is read back as a
-// wave-uniform scalar, so the loop is controlled by scalar branches.  With the claim at the top of
-// the loop and the publish at the bottom - no barrier between them across the back edge - the
-// compiler merges the two single-thread blocks and lets the other 255 threads run ahead into the
-// next iteration's barrier while the claiming lane is masked off: they re-read the old item for
-// ever and the launch never drains.
-
-__device__ __forceinline__ int claim_item(const StepwiseLaunch& L) {
-    const int stalled = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return stalled ? L.num_items : (int)(atomicAdd(&L.state->ticket, 1u) - L.ticket_base);
-}
+// Shape of the loop (it matters): the item number is a wave-uniform scalar, so the loop is
+// controlled by scalar branches, and the single-thread blocks (stall check, publish) each sit
+// between two barriers.  An earlier form claimed the item in a single-thread block at the top of
+// the loop and published in another at the bottom, with no barrier between them across the back
+// edge; the compiler merged the two blocks and let the other 255 threads run ahead into the next
+// iteration's barrier while the claiming lane was masked off: they re-read the old item for ever
+// and the launch never drained.
 
 template <int DT>
 __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     constexpr int ES = ElemBytes<DT>::value;
-    __shared__ int s_word;   // broadcast slot: the claimed item, then the stall flag
+    __shared__ int s_word;   // broadcast slot of the stall flag
     int32_t* flags = reinterpret_cast<int32_t*>(L.state + 1);
     const int tid = threadIdx.x;
     const uint64_t t_start = __builtin_amdgcn_s_memrealtime();
-    if (tid == 0) s_word = claim_item(L);
-    __syncthreads();
-    int item = __builtin_amdgcn_readfirstlane(s_word);
-    __syncthreads();
-    while (item >= 0 && item < L.num_items) {
+    for (int item = blockIdx.x; item < L.num_items; item += gridDim.x) {
         const int opi = as_const(L.item_op)[item];
         const DevStepOp op = load_const(L.ops + opi);
         // wait: thread t watches items t, t+256, ... of each predecessor (no barrier in here)
@@ -394,8 +436,8 @@ __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, 
                 }
             }
         }
-        __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        __syncthreads();   // every flag this workgroup waited for has been seen; the data accesses below
+                           // are agent-coherent, so no cache needs to be invalidated first
         if (tid == 0) s_word = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         const int stalled = __builtin_amdgcn_readfirstlane(s_word);
@@ -405,17 +447,15 @@ __global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, 
         char* self = ptrs.p[op.self];
         const char* peer = ptrs.p[op.peer];
         if (op.is_reduce)
-            range_op<DT, true>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
+            range_op<DT, true, MEM_COHERENT>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
         else
-            range_copy_bytes(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");   // every wave: its own stores are visible
+            range_copy_bytes<MEM_COHERENT>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
+        // every wave: its write-through stores have been acknowledged (they are visible to the
+        // whole device) before the workgroup meets and one thread publishes the item
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == 0) {
-            __hip_atomic_store(&flags[item], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_word = claim_item(L);
-        }
-        __syncthreads();
-        item = __builtin_amdgcn_readfirstlane(s_word);
+        if (tid == 0) __hip_atomic_store(&flags[item], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();   // keeps the single-thread block away from the back edge (see above)
     }
 }
 
@@ -743,7 +783,12 @@ int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
 
 template <int DT>
 static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
-    int grid = L.num_blocks > 0 ? L.num_blocks : current_cus() * 8;
+    // every workgroup must be resident at once: never more than the runtime says fit
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, persistent_kernel<DT>, kThreads, 0) != hipSuccess || per_cu <= 0) per_cu = 1;
+    if (per_cu > 8) per_cu = 8;
+    const int resident = current_cus() * per_cu;
+    int grid = L.num_blocks > 0 && L.num_blocks < resident ? L.num_blocks : resident;
     if (grid > L.num_items) grid = L.num_items;
     if (grid <= 0) return 0;
     hipLaunchKernelGGL((persistent_kernel<DT>), dim3(grid), dim3(kThreads), 0, s, L, ptrs);
