@@ -94,23 +94,36 @@ def sha256_of(t) -> str:
 
 
 def device_info(dev) -> dict:
-    """Name, CU count and - best effort, through rocm-smi - the clocks and power cap of the GPU."""
+    """Name, CU count and - best effort, from the driver's sysfs files - the current clocks and the
+    power cap of the GPU (no helper program is started: a process that holds the GPU must not)."""
+    import glob
     import re
-    import subprocess
     import torch
     props = torch.cuda.get_device_properties(dev)
     info = {"name": props.name, "compute_units": props.multi_processor_count,
             "hbm_gib": round(props.total_memory / 2**30, 1), "sclk_mhz": None, "mclk_mhz": None, "power_cap_w": None}
-    try:
-        out = subprocess.run(["rocm-smi", "--showclocks", "--showmaxpower"], capture_output=True, text=True,
-                             timeout=20).stdout
-        for key, pat in (("sclk_mhz", r"sclk clock level: \S+ \((\d+)Mhz\)"), ("mclk_mhz", r"mclk clock level: \S+ \((\d+)Mhz\)"),
-                         ("power_cap_w", r"Max Graphics Package Power \(W\): ([\d.]+)")):
-            m = re.search(pat, out)
-            if m:
-                info[key] = float(m.group(1))
-    except (OSError, subprocess.SubprocessError):
-        pass
+
+    def current_level(pattern):
+        for path in sorted(glob.glob(pattern)):
+            try:
+                with open(path) as f:
+                    for line in f:
+                        m = re.match(r"\s*\d+:\s*(\d+)Mhz\s*\*", line)
+                        if m:
+                            return float(m.group(1))
+            except OSError:
+                pass
+        return None
+
+    info["sclk_mhz"] = current_level("/sys/class/drm/card*/device/pp_dpm_sclk")
+    info["mclk_mhz"] = current_level("/sys/class/drm/card*/device/pp_dpm_mclk")
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")):
+        try:
+            with open(path) as f:
+                info["power_cap_w"] = int(f.read().strip()) / 1e6
+            break
+        except (OSError, ValueError):
+            pass
     return info
 
 
@@ -302,6 +315,25 @@ def main() -> int:
                     "frac_of_hbm_peak": round(alg_bytes / (sw_ms * 1e-3) / 1e9 / PEAK_GBPS, 4),
                     "note": "HBM traffic equals the algorithmic bytes in this mode (profiles/level_kernel_*.md)"}
 
+    # and as one persistent launch whose workgroups order themselves through device-side flags
+    persistent = None
+    if args.mode == "auto":
+        eng.set_option("mode", "persistent")
+        for _ in range(2):
+            eng.execute_inplace("bench", bufs)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            eng.execute_inplace("bench", bufs)
+        e1.record()
+        torch.cuda.synchronize()
+        pm_ms = e0.elapsed_time(e1) / reps
+        eng.sync_operation("bench")      # would raise if a bounded wait had expired
+        eng.set_option("mode", "auto")
+        persistent = {"mode": "persistent", "ms_per_step": round(pm_ms, 4), "GB/s": round(alg_bytes / (pm_ms * 1e-3) / 1e9, 1),
+                      "frac_of_hbm_peak": round(alg_bytes / (pm_ms * 1e-3) / 1e9 / PEAK_GBPS, 4),
+                      "note": "one launch for the whole graph, every op moving its full bytes, ordering by per-item flags"}
+
     default_runner = not any(kv.split("=")[0] in ("lds_slots", "slot_threads", "slot_direct") for kv in args.option)
     traffic = measured_traffic(args.mode, info["num_levels"]) if (n == N and channels == CHANNELS and default_runner) else None
     result = {
@@ -324,6 +356,7 @@ def main() -> int:
                               "note": "the reference's call shape (separate input and output tensors per rank, execute_operation_async); "
                                       "the staging copies are fused into the program, so this is again one launch"},
         "op_by_op": op_by_op,
+        "single_launch_flag_ordered": persistent,
         "device": device_info(dev),
         "verify": verify,
     }

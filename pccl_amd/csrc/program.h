@@ -95,7 +95,7 @@ struct Program {
 struct LinkOptions {
     bool check_races = true;
     bool conflict_deps = true;     // order data ops by memory conflicts instead of raw chain order
-    int64_t step_tile_bytes = 128 * 1024;
+    int64_t step_tile_bytes = 16 * 1024;
 };
 
 // Throws Error (PCCL_ERR_LINK for deadlock, ambiguous signal pairing, races, bad ranks).
