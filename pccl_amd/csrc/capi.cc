@@ -634,7 +634,7 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
         } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
         else if (k == "timing") ctx->timing = std::atoi(value) != 0;
         else if (k == "fuse_staging") ctx->fuse_staging = std::atoi(value) != 0;
-        else if (k == "wait_timeout_ms") { ctx->wait_timeout_ms = std::atoi(value); if (ctx->wait_timeout_ms < 1) ctx->wait_timeout_ms = 1; }
+        else if (k == "wait_timeout_ms") { ctx->wait_timeout_ms = std::atoi(value); if (ctx->wait_timeout_ms < 0) ctx->wait_timeout_ms = 0; }   // 0: give up on the first predecessor that is not ready
         else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
         else if (k == "vecs_per_thread") {
             int u = std::atoi(value);

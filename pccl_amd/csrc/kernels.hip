@@ -408,7 +408,8 @@ __global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int i
 // and the launch never drained.
 
 template <int DT>
-__global__ __launch_bounds__(kThreads) void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
+void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     constexpr int ES = ElemBytes<DT>::value;
     __shared__ int s_word;   // broadcast slot of the stall flag
     int32_t* flags = reinterpret_cast<int32_t*>(L.state + 1);
@@ -783,10 +784,21 @@ int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
 
 template <int DT>
 static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
-    // every workgroup must be resident at once: never more than the runtime says fit
+    // Every workgroup must be resident at once.  A workgroup is one wave per SIMD; a SIMD holds 512
+    // vector registers per lane and 800 scalar registers.  The kernel is compiled for 8 waves per
+    // SIMD (amdgpu_waves_per_eu: at most 64 vector and 96 scalar registers); take the smallest of
+    // that, the bound from the vector registers it reports and what the runtime says.  (A form of
+    // this kernel that needed 100 scalar registers fitted only 7 times per CU while the runtime's
+    // estimate said 8: the grid was one workgroup per CU too large and waits expired.)
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, persistent_kernel<DT>, kThreads, 0) != hipSuccess || per_cu <= 0) per_cu = 1;
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(persistent_kernel<DT>)) == hipSuccess && attr.numRegs > 0) {
+        const int by_vgpr = 512 / ((attr.numRegs + 7) / 8 * 8);
+        if (by_vgpr < per_cu) per_cu = by_vgpr;
+    }
     if (per_cu > 8) per_cu = 8;
+    if (per_cu < 1) per_cu = 1;
     const int resident = current_cus() * per_cu;
     int grid = L.num_blocks > 0 && L.num_blocks < resident ? L.num_blocks : resident;
     if (grid > L.num_items) grid = L.num_items;

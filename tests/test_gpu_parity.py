@@ -140,18 +140,18 @@ def test_alltoall(engine_factory, mode):
 
 
 def test_persistent_runner_reports_a_wait_that_expires(engine_factory):
-    """Every wait of the persistent runner is bounded: with a 1 ms bound on a program that runs
-    longer than that, some workgroup's wait on a predecessor expires; it records which, every
-    workgroup leaves at its next claim (the launch drains normally), and the call reports the stall
-    instead of hanging.  The next execution, with the bound restored, is correct."""
+    """Every wait of the persistent runner is bounded.  With the bound set to zero the first
+    workgroup that finds a predecessor not yet published gives up at once: it records which, every
+    other wait ends as soon as it sees that record, the launch drains normally, and the call reports
+    the stall instead of hanging.  The next execution, with the bound restored, is correct."""
     from pccl_amd._lib import PcclError
-    world, n = 8, 1 << 27           # 512 MiB per rank: the 14 levels take about 3 ms
+    world, n = 8, 1 << 24
     jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)
     engine = engine_factory(world)
     for r, j in enumerate(jsons):
         engine.register_operation_json("slow", j, r)
     engine.set_option("mode", "persistent")
-    engine.set_option("wait_timeout_ms", 1)
+    engine.set_option("wait_timeout_ms", 0)
     bufs = [torch.ones(n, device="cuda") for _ in range(world)]
     with pytest.raises(PcclError, match="gave up waiting"):
         engine.execute_inplace("slow", bufs, sync=True)
