@@ -110,6 +110,47 @@ def chained_gather(rank: int, world: int, chunk: int, dtype: str, pieces: int, k
         return op.get_graph()
 
 
+def random_program(seed: int, world: int, n: int, num_ops: int, dtype: str, aligned: bool,
+                   reduce_ops=("sum",)) -> List[str]:
+    """A random race-free program: `num_ops` reduces and copies over random ranks, peers and element
+    ranges (sizes and offsets of any parity), in one global order that notify / wait pairs enforce
+    from each op to the next (program order where both are on one rank).  With aligned=True every
+    op reads and writes the same element positions (the column runner's domain); otherwise source
+    and destination ranges differ (reduce: the own operand is read where the result is written).
+    Returns the per-rank JSON graphs."""
+    rng = np.random.default_rng(seed)
+    builders = []
+    for r in range(world):
+        op = CommunicationOp(name=f"rand{seed}_rank{r}")
+        op.__enter__()
+        op.tensor(dtype=dtype, shape=(n,))
+        builders.append(op)
+    prev_rank, used = None, [False] * world
+    for k in range(num_ops):
+        r = int(rng.integers(world))
+        peer = int(rng.integers(world - 1))
+        peer += peer >= r
+        size = int(rng.integers(1, max(2, n // 3)))
+        dst = int(rng.integers(0, n - size + 1))
+        src = dst if aligned else int(rng.integers(0, n - size + 1))
+        if prev_rank is not None and prev_rank != r:
+            builders[prev_rank].notify(signal_id=k, target_rank=r)
+            builders[r].wait_notify(signal_id=k, source_rank=prev_rank)
+        if rng.random() < 0.5:
+            builders[r].sm_reduce(reduce_op=str(rng.choice(reduce_ops)), source_rank=peer, remote_offset=src,
+                                  src_offset=dst, dst_offset=dst, count=size)
+        else:
+            builders[r].sm_copy(source_rank=peer, src_offset=src, dst_offset=dst, size=size)
+        prev_rank, used[r] = r, True
+    out = []
+    for r, op in enumerate(builders):
+        if not used[r]:          # a rank with nothing to do still registers a graph
+            op.sm_copy(source_rank=(r + 1) % world, src_offset=0, dst_offset=0, size=0)
+        op.__exit__(None, None, None)
+        out.append(compile_to_json_string(op.get_graph()))
+    return out
+
+
 def to_raw(t: torch.Tensor) -> np.ndarray:
     """CPU tensor -> numpy array of its storage bits (bf16/f16 as uint16)."""
     t = t.contiguous()

@@ -12,7 +12,7 @@ import json
 import numpy as np
 import pytest
 
-from helpers import graph_jsons, oracle, pipelined_ring_allreduce
+from helpers import graph_jsons, oracle, pipelined_ring_allreduce, random_program
 from pccl_amd._lib import HostGraph, HostProgram
 from pccl_amd.dsl import compile_to_json_string, ragged_cuts
 
@@ -156,3 +156,22 @@ def test_staged_plan_reads_inputs_and_writes_outputs_only(method, world, channel
     S = n * 4
     if method != "build_allreduce" and channels == 1:
         assert info["staged_load_bytes"] + info["staged_store_bytes"] == (world + 1) * S   # R S one way, S the other
+
+
+@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("slots_mode", [False, True], ids=["memory", "slots"])
+def test_random_aligned_programs(seed, slots_mode):
+    """Random race-free programs (random ranks, peers, ranges of any parity, sum / max / min) whose ops
+    read and write the same positions: segments of many different op lists, forwarding, dead stores
+    and re-reads in every combination."""
+    world, n = 2 + seed % 5, 600 + 37 * seed
+    jsons = random_program(seed, world, n, 30 + 5 * seed, "int32", aligned=True, reduce_ops=("sum", "max", "min"))
+    x = inputs_for(world, n, seed)
+    want = [a.copy() for a in x]
+    oracle.run([oracle.Graph(json.loads(j)) for j in jsons], want)
+    prog = link(jsons)
+    assert prog.info()["position_aligned"] == 1
+    bufs = [a.copy() for a in x]
+    run_plan(prog.column_plan(), bufs, bufs, slots_mode)
+    for r in range(world):
+        assert np.array_equal(bufs[r], want[r]), f"rank {r}"
