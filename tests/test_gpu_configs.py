@@ -56,7 +56,7 @@ def rhd_expected(x, world, lo, n):
     return v[0]
 
 
-@pytest.mark.parametrize("mode", ["column", "stepwise"])
+@pytest.mark.parametrize("mode", ["column", "stepwise", "persistent"])
 def test_config3_rhd_16_ranks_64mb_f32_two_channels(engine_factory, mode):
     world, n = 16, 16_777_216
     print(f"config 3: RHD R={world} n={n} f32 2 channels, mode={mode}", flush=True)
@@ -76,7 +76,7 @@ def test_config3_rhd_16_ranks_64mb_f32_two_channels(engine_factory, mode):
     assert info["algorithmic_bytes"] == 75 * n * 4        # 5 (1 - 1/R) R S
 
 
-@pytest.mark.parametrize("mode", ["column", "stepwise"])
+@pytest.mark.parametrize("mode", ["column", "stepwise", "persistent"])
 @pytest.mark.parametrize("dtype,redop,kind", [("int32", "sum", "randint"), ("float32", "max", "randn")])
 def test_config5_tree_32_ranks_96mb_ragged(engine_factory, dtype, redop, kind, mode):
     world, n = 32, 25_165_824
@@ -134,15 +134,16 @@ def test_config4_reduce_scatter_allgather_fp16(engine_factory, nbytes, mode):
         assert same_bits(outs[r], whole), f"allgather rank {r}"
 
 
-def test_config2_headline_shape_in_both_modes_agree(engine_factory):
-    """512 MiB per rank, bf16, 4 channels: column and stepwise runners must produce the same bits."""
+def test_config2_headline_shape_in_all_modes_agree(engine_factory):
+    """512 MiB per rank, bf16, 4 channels: the column, level and persistent runners must produce the
+    same bits."""
     world, n = 8, 268_435_456
-    print("config 2: ring R=8 512 MiB bf16 4 channels, column vs stepwise", flush=True)
+    print("config 2: ring R=8 512 MiB bf16 4 channels, column vs stepwise vs persistent", flush=True)
     jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 4)
     x = dev_inputs("randn", world, n, "bfloat16")
     engine = engine_factory(world)
     results = {}
-    for mode in ("column", "stepwise"):
+    for mode in ("column", "stepwise", "persistent"):
         register(engine, f"c2_{mode}", jsons, mode)
         bufs = [t.clone() for t in x]
         engine.execute_inplace(f"c2_{mode}", bufs, sync=True)
@@ -151,6 +152,7 @@ def test_config2_headline_shape_in_both_modes_agree(engine_factory):
         results[mode] = bufs[0]
         del bufs
     assert same_bits(results["column"], results["stepwise"])
+    assert same_bits(results["column"], results["persistent"])
     per_ch, per_rank = n // 4, n // 32
     for ch in (0, 3):
         for c in (0, 5):
