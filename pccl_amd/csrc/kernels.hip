@@ -186,9 +186,22 @@ typedef const PCCL_GLOBAL u32x4* gvec_cptr;
 typedef PCCL_GLOBAL u32x4* gvec_ptr;
 __device__ __forceinline__ u32x4 ldv(const char* p) { return *(gvec_cptr)(p); }
 __device__ __forceinline__ void stv(char* p, u32x4 v) { *(gvec_ptr)(p) = v; }
-// streaming variants: data touched once (measured +5..10 % on MI355X over the cached forms)
+// Streaming variants for data touched once.  Two forms, both measured on MI355X:
+//  * pointer form, non-temporal (nt): used by the column runners, whose per-store scalar work
+//    matters (building a buffer descriptor per store cost the 32-rank tree 5 %, and the ring is
+//    the same either way);
+//  * raw buffer operations (wave-uniform base in a resource descriptor, 32-bit byte offset per
+//    lane) marked non-temporal AND agent scope (nt sc1): used by everything built on range_op.
+//    Headline graph with the level runner: cached 3.22 ms, sc1 3.18, nt 3.06 (as global or as
+//    buffer operations alike), nt sc1 2.99; plain copy 6.28 -> 6.55 TB/s.  The agent-scope bit also
+//    makes the access coherent across the XCDs' L2s (a store is written through before it is
+//    acknowledged, a load does not hit a stale line), which the persistent runner relies on.
 __device__ __forceinline__ u32x4 ldv_nt(const char* p) { return __builtin_nontemporal_load((gvec_cptr)(p)); }
 __device__ __forceinline__ void stv_nt(char* p, u32x4 v) { __builtin_nontemporal_store(v, (gvec_ptr)(p)); }
+constexpr int kAuxStream = 16 | 2;   // sc1 | nt
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const char* uniform_base) {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)uniform_base, 0, 0x7FFFFFFF, 0x00020000);
+}
 
 // ------------------------------------------------------------------------------- range primitives
 //
@@ -196,49 +209,44 @@ __device__ __forceinline__ void stv_nt(char* p, u32x4 v) { __builtin_nontemporal
 // `nthreads` threads.  Any alignment: when the three addresses are congruent modulo 16 the body runs
 // as 128-bit loads and stores with a scalar head and tail; otherwise element by element.
 //
-// How memory is touched is a policy: cached, streaming (non-temporal: data touched once), or
-// agent-coherent.  The coherent form marks every access with the agent scope bit (sc1), the bit
-// the agent-scope atomics carry: such a store is written through to memory before it is
-// acknowledged and such a load does not hit a stale copy in this XCD's L2, so data written by a
-// workgroup on one XCD can be consumed by a workgroup on another after a flag hand-over without
-// writing back or invalidating whole caches.  128-bit accesses with that bit are expressed as raw
-// buffer operations (wave-uniform base in a resource descriptor, 32-bit byte offset per lane).
+// How memory is touched is a policy: cached (plain global accesses) or streaming (the nt sc1 buffer
+// operations above, which are also what makes data handed from one workgroup to another through a
+// flag visible without writing back or invalidating whole caches).
 
-enum { MEM_CACHED = 0, MEM_STREAM = 1, MEM_COHERENT = 2 };
-constexpr int kAuxCoherent = 16 | 2;   // sc1 | nt
+enum { MEM_CACHED = 0, MEM_STREAM = 1, MEM_COHERENT = 1 };
 
 template <int POLICY>
-struct Mem {
+struct Mem {     // MEM_CACHED
     const char* base;
     __device__ __forceinline__ explicit Mem(const char* b) : base(b) {}
-    __device__ __forceinline__ u32x4 ldv(int64_t off) const { return POLICY == MEM_STREAM ? ldv_nt(base + off) : ::pccl_hip::ldv(base + off); }
-    __device__ __forceinline__ void stv(int64_t off, u32x4 v) const { if (POLICY == MEM_STREAM) stv_nt((char*)base + off, v); else ::pccl_hip::stv((char*)base + off, v); }
+    __device__ __forceinline__ u32x4 ldv(int64_t off) const { return ::pccl_hip::ldv(base + off); }
+    __device__ __forceinline__ void stv(int64_t off, u32x4 v) const { ::pccl_hip::stv((char*)base + off, v); }
     template <int DT> __device__ __forceinline__ uint32_t lde(int64_t off) const { return load_elem<DT>(base + off); }
     template <int DT> __device__ __forceinline__ void ste(int64_t off, uint32_t x) const { store_elem<DT>((char*)base + off, x); }
 };
 
 template <>
-struct Mem<MEM_COHERENT> {
+struct Mem<MEM_STREAM> {
     __amdgpu_buffer_rsrc_t rs;
-    __device__ __forceinline__ explicit Mem(const char* b)
-        : rs(__builtin_amdgcn_make_buffer_rsrc((void*)b, 0, 0x7FFFFFFF, 0x00020000)) {}
-    __device__ __forceinline__ u32x4 ldv(int64_t off) const { return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, kAuxCoherent); }
-    __device__ __forceinline__ void stv(int64_t off, u32x4 v) const { __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)off, 0, kAuxCoherent); }
+    __device__ __forceinline__ explicit Mem(const char* b) : rs(stream_rsrc(b)) {}
+    __device__ __forceinline__ u32x4 ldv(int64_t off) const { return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, kAuxStream); }
+    __device__ __forceinline__ void stv(int64_t off, u32x4 v) const { __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)off, 0, kAuxStream); }
     template <int DT> __device__ __forceinline__ uint32_t lde(int64_t off) const {
         constexpr int ES = ElemBytes<DT>::value;
-        if constexpr (ES == 4) return __builtin_amdgcn_raw_buffer_load_b32(rs, (int)off, 0, kAuxCoherent);
-        else if constexpr (ES == 2) return __builtin_amdgcn_raw_buffer_load_b16(rs, (int)off, 0, kAuxCoherent);
-        else return __builtin_amdgcn_raw_buffer_load_b8(rs, (int)off, 0, kAuxCoherent);
+        if constexpr (ES == 4) return __builtin_amdgcn_raw_buffer_load_b32(rs, (int)off, 0, kAuxStream);
+        else if constexpr (ES == 2) return __builtin_amdgcn_raw_buffer_load_b16(rs, (int)off, 0, kAuxStream);
+        else return __builtin_amdgcn_raw_buffer_load_b8(rs, (int)off, 0, kAuxStream);
     }
     template <int DT> __device__ __forceinline__ void ste(int64_t off, uint32_t x) const {
         constexpr int ES = ElemBytes<DT>::value;
-        if constexpr (ES == 4) __builtin_amdgcn_raw_buffer_store_b32(x, rs, (int)off, 0, kAuxCoherent);
-        else if constexpr (ES == 2) __builtin_amdgcn_raw_buffer_store_b16((uint16_t)x, rs, (int)off, 0, kAuxCoherent);
-        else __builtin_amdgcn_raw_buffer_store_b8((uint8_t)x, rs, (int)off, 0, kAuxCoherent);
+        if constexpr (ES == 4) __builtin_amdgcn_raw_buffer_store_b32(x, rs, (int)off, 0, kAuxStream);
+        else if constexpr (ES == 2) __builtin_amdgcn_raw_buffer_store_b16((uint16_t)x, rs, (int)off, 0, kAuxStream);
+        else __builtin_amdgcn_raw_buffer_store_b8((uint8_t)x, rs, (int)off, 0, kAuxStream);
     }
 };
 
-// The ranges handed to the coherent form must be shorter than 2 GiB (offsets are 32-bit).
+// The ranges handed to the streaming form must be shorter than 2 GiB (offsets are 32-bit) and their
+// base addresses wave-uniform.
 template <int DT, bool IS_REDUCE, int POLICY = MEM_STREAM>
 __device__ __forceinline__ void range_op(const char* a, const char* b, char* c, int64_t n, int redop,
                                          int tid, int nthreads) {
