@@ -146,7 +146,8 @@ typedef struct {
     int64_t column_load_bytes;  /* bytes the column plan loads / stores from memory per execution */
     int64_t column_store_bytes;
     int32_t num_items;          /* stepwise plan: (op, tile) work items */
-    int32_t reserved_;
+    int32_t num_gather_copies;  /* alltoall graphs: direct input-to-output copies the staged call composes
+                                   into (0 = no such plan, the call stages through the rank buffers) */
     int64_t staged_load_bytes;  /* the same for a staged call that runs on the caller's tensors */
     int64_t staged_store_bytes; /* (0 when the graph has no such plan and staging copies are used) */
 } pccl_program_info;

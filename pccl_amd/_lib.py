@@ -48,7 +48,7 @@ class ProgramInfo(ctypes.Structure):
                 ("residual_signals", ctypes.c_int32), ("buffer_elems", ctypes.c_int64),
                 ("algorithmic_bytes", ctypes.c_int64), ("column_load_bytes", ctypes.c_int64),
                 ("column_store_bytes", ctypes.c_int64), ("num_items", ctypes.c_int32),
-                ("reserved_", ctypes.c_int32), ("staged_load_bytes", ctypes.c_int64),
+                ("num_gather_copies", ctypes.c_int32), ("staged_load_bytes", ctypes.c_int64),
                 ("staged_store_bytes", ctypes.c_int64)]
 
     def as_dict(self):

@@ -61,6 +61,7 @@ void fill_info(const Program& p, pccl_program_info* out) {
     out->column_load_bytes = p.column_load_bytes;
     out->column_store_bytes = p.column_store_bytes;
     out->num_items = (int)p.num_items;
+    out->num_gather_copies = (int)p.gather.size();
     out->staged_load_bytes = p.direct_load_bytes;
     out->staged_store_bytes = p.direct_store_bytes;
 }
@@ -228,6 +229,8 @@ struct OpEntry {
     std::vector<std::unique_ptr<RankGraph>> graphs;
     bool linked = false;
     Program prog;
+    DevBuf gather;                        // gather plan of an alltoall graph (DevGatherCopy records)
+    int64_t gather_tiles = 0;
     DevBuf segs, direct_segs, instrs, pre, step_ops, step_deps, item_op, state;
     int64_t total_tiles = 0, direct_tiles = 0;
     int vecs_per_thread = 0;
@@ -253,6 +256,7 @@ struct OpEntry {
     void release() {
         drop_graphs();
         graph_failed = false;
+        gather.release(); gather_tiles = 0;
         segs.release(); direct_segs.release(); instrs.release(); pre.release(); step_ops.release(); step_deps.release();
         item_op.release(); state.release();
         if (ev0) (void)hipEventDestroy(ev0);
@@ -357,6 +361,19 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
         }
         e.instrs.upload(P.col_instrs.data(), P.col_instrs.size() * sizeof(ColInstr));
         e.pre.upload(P.col_pre.data(), P.col_pre.size() * sizeof(uint64_t));
+    }
+    if (!P.gather.empty()) {
+        std::vector<DevGatherCopy> gc(P.gather.size());
+        int64_t tiles = 0;
+        for (size_t i = 0; i < gc.size(); ++i) {
+            const Program::GatherCopy& g = P.gather[i];
+            gc[i].src_rank = g.src_rank; gc[i].dst_rank = g.dst_rank;
+            gc[i].src_off = g.src_off * es; gc[i].dst_off = g.dst_off * es; gc[i].bytes = g.elems * es;
+            gc[i].first_tile = tiles;
+            tiles += (gc[i].bytes + 4095) / 4096;
+        }
+        e.gather_tiles = tiles;
+        e.gather.upload(gc.data(), gc.size() * sizeof(DevGatherCopy));
     }
     // stepwise plan
     {
@@ -683,6 +700,30 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
             ctx->last_stream = s;
             if (sync) HIP_TRY(hipStreamSynchronize(s));
             return 0;
+        }
+
+        // alltoall as direct copies from the input tensors to the output tensors, when the program
+        // composes into such copies and no output overlaps an input
+        if (ct == "alltoall" && ctx->fuse_staging && e.gather.p && (ctx->mode == Mode::Auto || ctx->mode == Mode::Column) &&
+            in_bytes == (size_t)P.tensor_elems * es && out_bytes >= in_bytes) {
+            bool disjoint = true;
+            for (int r = 0; r < R && disjoint; ++r)
+                for (int q = 0; q < R && disjoint; ++q) {
+                    const uintptr_t o = (uintptr_t)outputs[r], i = (uintptr_t)inputs[q];
+                    if (o < i + in_bytes && i < o + in_bytes) disjoint = false;
+                    if (q != r && o < (uintptr_t)outputs[q] + in_bytes && (uintptr_t)outputs[q] < o + in_bytes) disjoint = false;
+                }
+            if (disjoint) {
+                RankPtrs src{}, dst{};
+                for (int r = 0; r < R; ++r) { src.p[r] = (char*)inputs[r]; dst.p[r] = (char*)outputs[r]; }
+                if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, s));
+                int grc = launch_gather((const DevGatherCopy*)e.gather.p, (int)P.gather.size(), e.gather_tiles, src, dst, s);
+                if (grc) return fail(PCCL_ERR_HIP, std::string("gather launch failed: ") + hipGetErrorString((hipError_t)grc));
+                if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, s)); e.timed = true; }
+                ctx->last_stream = s;
+                if (sync) HIP_TRY(hipStreamSynchronize(s));
+                return 0;
+            }
         }
 
         // layout of the staged data inside a rank buffer (reference engine_c.cc:468-548)

@@ -78,6 +78,11 @@ int launch_level(const StepwiseLaunch& L, int item_begin, int item_end, const Ra
 int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream);
 int launch_copy_bytes(const void* src, void* dst, size_t nbytes, void* stream);
 // One launch copying `bytes` from src.p[r] + src_off[r] to dst.p[r] + dst_off[r] for r < R.
+// One direct copy of a gather plan: `bytes` from src.p[src_rank] + src_off to dst.p[dst_rank] + dst_off;
+// first_tile = tiles of all earlier copies (4 KiB tiles, one workgroup each).
+struct DevGatherCopy { int64_t src_off, dst_off, bytes, first_tile; int32_t src_rank, dst_rank; };
+int launch_gather(const DevGatherCopy* copies, int n, int64_t total_tiles, const RankPtrs& src, const RankPtrs& dst, void* stream);
+
 struct StageOffsets { int64_t src[PCCL_HIP_MAX_VRANKS]; int64_t dst[PCCL_HIP_MAX_VRANKS]; };
 int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& off, int R, size_t bytes, void* stream);
 int launch_fill_zero(void* dst, size_t nbytes, void* stream);

@@ -347,6 +347,22 @@ __global__ __launch_bounds__(kThreads) void stage_kernel(RankPtrs src, RankPtrs 
     }
 }
 
+// A list of independent copies between rank tensors in one launch (the staged alltoall call composed
+// into direct copies): workgroup w finds its copy by binary search over the tile prefix sums.
+__global__ __launch_bounds__(kThreads) void gather_kernel(const DevGatherCopy* copies, int n, int64_t total_tiles, RankPtrs src, RankPtrs dst) {
+    for (int64_t w = blockIdx.x; w < total_tiles; w += gridDim.x) {
+        int lo = 0, hi = n;
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (as_const(copies)[mid].first_tile <= w) lo = mid; else hi = mid;
+        }
+        const DevGatherCopy c = load_const(copies + lo);
+        const int64_t b0 = (w - c.first_tile) * kPrimTileBytes;
+        const int64_t cnt = c.bytes - b0 < kPrimTileBytes ? c.bytes - b0 : kPrimTileBytes;
+        range_copy_bytes(src.p[c.src_rank] + c.src_off + b0, dst.p[c.dst_rank] + c.dst_off + b0, cnt, threadIdx.x, kThreads);
+    }
+}
+
 __global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* dst, int64_t nwords) {
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * kThreads) dst[i] = 0;
 }
@@ -891,6 +907,12 @@ int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& o
     int gx = (int)(ntiles < cap ? ntiles : cap);
     if (gx < 1) gx = 1;
     hipLaunchKernelGGL(stage_kernel, dim3(gx, R), dim3(kThreads), 0, (hipStream_t)stream, src, dst, off, (int64_t)bytes);
+    return (int)hipGetLastError();
+}
+
+int launch_gather(const DevGatherCopy* copies, int n, int64_t total_tiles, const RankPtrs& src, const RankPtrs& dst, void* stream) {
+    if (n <= 0 || total_tiles <= 0) return 0;
+    hipLaunchKernelGGL(gather_kernel, dim3(grid_for_tiles(total_tiles)), dim3(kThreads), 0, (hipStream_t)stream, copies, n, total_tiles, src, dst);
     return (int)hipGetLastError();
 }
 

@@ -391,6 +391,52 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
     }
     P.num_items = items;
 
+    // ---- gather plan: an alltoall graph whose ops are all copies out of regions nobody writes.
+    // Staged semantics (reference engine_c.cc:524-543): input r sits at [0, n) of buffer r, the
+    // program runs, output r is chunk r of the input region followed, for every other rank p, by
+    // the scratch chunk [n + p*chunk, n + (p+1)*chunk).  Composing that with the copies gives, for
+    // every output element, the input element it comes from - no buffer needed.  Abandoned (the
+    // call then stages through the rank buffers) if any output element would come from scratch the
+    // program never wrote, or if an op writes something another op reads or writes.
+    if (P.collective_type == "alltoall" && D > 0 && P.tensor_elems > 0 && P.tensor_elems % R == 0) {
+        const int64_t n = P.tensor_elems, chunk = n / R;
+        bool ok = true;
+        for (const LinkedOp& L : P.ops) if (L.is_reduce) ok = false;
+        // sources inside the input region, destinations outside it and mutually disjoint per rank
+        std::vector<std::vector<std::pair<int64_t, int>>> writes(R);   // (dst offset, op) per rank
+        for (int k = 0; k < D && ok; ++k) {
+            const LinkedOp& L = P.ops[k];
+            if (L.size <= 0) continue;
+            if (L.off0 < 0 || L.off0 + L.size > n || L.off1 < n) ok = false;
+            writes[L.rank].push_back({L.off1, k});
+        }
+        for (int r = 0; r < R && ok; ++r) {
+            std::sort(writes[r].begin(), writes[r].end());
+            for (size_t i = 1; i < writes[r].size(); ++i) {
+                const LinkedOp& prev = P.ops[writes[r][i - 1].second];
+                if (prev.off1 + prev.size > writes[r][i].first) ok = false;
+            }
+        }
+        for (int r = 0; r < R && ok; ++r)
+            for (int p = 0; p < R && ok; ++p) {
+                if (p == r) { P.gather.push_back({r, r, (int64_t)p * chunk, (int64_t)r * chunk, chunk}); continue; }
+                int64_t x = n + (int64_t)p * chunk;
+                const int64_t x_end = x + chunk;
+                while (x < x_end && ok) {        // walk the scratch chunk through the ops that wrote it
+                    const LinkedOp* hit = nullptr;
+                    for (auto& w : writes[r]) {
+                        const LinkedOp& L = P.ops[w.second];
+                        if (L.off1 <= x && x < L.off1 + L.size) { hit = &L; break; }
+                    }
+                    if (!hit) { ok = false; break; }
+                    const int64_t len = std::min(x_end, hit->off1 + hit->size) - x;
+                    P.gather.push_back({r, hit->peer, (int64_t)p * chunk + (x - (n + (int64_t)p * chunk)), hit->off0 + (x - hit->off1), len});
+                    x += len;
+                }
+            }
+        if (!ok) P.gather.clear();
+    }
+
     // ---- column plan
     P.position_aligned = D > 0;
     for (auto& L : P.ops) if (!L.position_aligned()) { P.position_aligned = false; break; }

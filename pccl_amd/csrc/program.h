@@ -85,6 +85,11 @@ struct Program {
     int64_t direct_slot_load_bytes = 0, direct_slot_store_bytes = 0;
     std::vector<int64_t> direct_in_start, direct_in_end, direct_out_start, direct_out_end;  // windows per rank
 
+    // gather plan of an alltoall graph (valid when non-empty): the staged call as direct copies from
+    // the callers' input tensors to their output tensors, element units
+    struct GatherCopy { int dst_rank, src_rank; int64_t dst_off, src_off, elems; };
+    std::vector<GatherCopy> gather;
+
     // stepwise plan
     int64_t tile_elems = 0;
     std::vector<StepOpPlan> step_ops;

@@ -124,19 +124,41 @@ def test_reduce_scatter_and_allgather(engine_factory, mode, channels, fuse):
         engine.set_option("fuse_staging", 1)
 
 
-@pytest.mark.parametrize("mode", ["stepwise", "persistent"])
-def test_alltoall(engine_factory, mode):
-    """reference tests/test_correctness.py:243-272: out[i] chunk = chunk r of rank i's input."""
-    world, n = 4, 1 << 12
+@pytest.mark.parametrize("mode", ["auto", "stepwise", "persistent"])
+@pytest.mark.parametrize("world,n", [(4, 1 << 12), (8, 8 * 1031), (3, 3 * 5000)])
+def test_alltoall(engine_factory, mode, world, n):
+    """reference tests/test_correctness.py:243-272: out[i] chunk = chunk r of rank i's input.  In
+    `auto` mode the staged call is composed into direct input-to-output copies (one launch); the
+    other modes stage through the rank buffers and their scratch region."""
     chunk = n // world
     jsons = graph_jsons("ring", "build_alltoall", world, n, "bfloat16", "tma", 1)
-    inputs = [torch.cat([torch.full((chunk,), r * 100 + i, dtype=torch.bfloat16) for i in range(world)])
-              for r in range(world)]
+    inputs = seeded_inputs("randn", world, n, "bfloat16", seed=13)
     got, info = run_gpu(engine_factory(world), jsons, inputs, mode)
-    assert info["position_aligned"] == 0
+    assert info["position_aligned"] == 0 and info["num_gather_copies"] == world * world
     for r in range(world):
-        want = torch.cat([torch.full((chunk,), i * 100 + r, dtype=torch.bfloat16) for i in range(world)])
+        want = torch.cat([inputs[i][r * chunk:(r + 1) * chunk] for i in range(world)])
         assert bits_equal(got[r], want), mismatch_report(got[r], want)
+
+
+def test_alltoall_falls_back_to_staging_when_it_must(engine_factory):
+    """Outputs that overlap inputs, or fuse_staging=0: the same result through the rank buffers."""
+    world, n = 4, 1 << 13
+    chunk = n // world
+    jsons = graph_jsons("ring", "build_alltoall", world, n, "float32", "sm", 1)
+    engine = engine_factory(world)
+    for r, j in enumerate(jsons):
+        engine.register_operation_json("a2a", j, r)
+    x = seeded_inputs("randn", world, n, "float32", seed=3)
+    want = [torch.cat([x[i][r * chunk:(r + 1) * chunk] for i in range(world)]) for r in range(world)]
+    dev = [t.cuda() for t in x]
+    outs = engine.execute_operation("a2a", dev, dev)          # in place: every output is an input
+    for r in range(world):
+        assert bits_equal(outs[r], want[r])
+    engine.set_option("fuse_staging", 0)
+    outs = engine.execute_operation("a2a", [t.cuda() for t in x])
+    engine.set_option("fuse_staging", 1)
+    for r in range(world):
+        assert bits_equal(outs[r], want[r])
 
 
 def test_persistent_runner_reports_a_wait_that_expires(engine_factory):

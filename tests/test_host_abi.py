@@ -302,3 +302,17 @@ def test_reference_numbered_pipeline_schedule_is_reported_as_deadlock():
              for r in range(world)]
     info = HostProgram([HostGraph.from_json(j) for j in jsons]).info()
     assert info["residual_signals"] == 0 and info["position_aligned"] == 1 and info["num_data_ops"] == 24
+
+
+def test_alltoall_gather_plan():
+    """A one-channel alltoall composes into R*R direct input-to-output copies; allreduce graphs and
+    the two-channel alltoall (whose scratch chunks the engine's output rule reads are not all
+    written by the program) have no such plan and are staged."""
+    from helpers import graph_jsons
+    for world in (3, 4, 8):
+        jsons = graph_jsons("ring", "build_alltoall", world, world * 512, "bfloat16", "sm", 1)
+        assert HostProgram([HostGraph.from_json(j) for j in jsons]).info()["num_gather_copies"] == world * world
+    jsons = graph_jsons("ring", "build_alltoall", 4, 4096, "bfloat16", "sm", 2)
+    assert HostProgram([HostGraph.from_json(j) for j in jsons]).info()["num_gather_copies"] == 0
+    jsons = graph_jsons("ring", "build_allreduce", 4, 4096, "bfloat16", "sm", 1)
+    assert HostProgram([HostGraph.from_json(j) for j in jsons]).info()["num_gather_copies"] == 0
