@@ -704,7 +704,7 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
 
         // alltoall as direct copies from the input tensors to the output tensors, when the program
         // composes into such copies and no output overlaps an input
-        if (ct == "alltoall" && ctx->fuse_staging && e.gather.p && (ctx->mode == Mode::Auto || ctx->mode == Mode::Column) &&
+        if (ct == "alltoall" && ctx->fuse_staging && e.gather.p && ctx->mode == Mode::Auto &&
             in_bytes == (size_t)P.tensor_elems * es && out_bytes >= in_bytes) {
             bool disjoint = true;
             for (int r = 0; r < R && disjoint; ++r)
