@@ -133,6 +133,18 @@ class Engine:
                                                     _current_stream_ptr(self.device), int(sync)))
         return bs
 
+    def prepare(self, name: str, inputs: TensorList, outputs: Optional[TensorList] = None) -> "PreparedCall":
+        """Check the tensors and build the argument arrays once; the returned object launches the
+        operation on those tensors with nothing but the C call per invocation (for loops that issue
+        the same small collective over and over: the checks and array building of
+        ``execute_operation_async`` cost more than a small kernel takes).  ``outputs=None`` means
+        in place on ``inputs``.  No counterpart in the reference."""
+        ins = self._as_list(inputs, "inputs")
+        outs = None if outputs is None else self._as_list(outputs, "outputs")
+        if any(x.nbytes != ins[0].nbytes for x in ins) or (outs and any(x.nbytes != outs[0].nbytes for x in outs)):
+            raise ValueError("all ranks must pass tensors of the same size")
+        return PreparedCall(self, name, ins, outs)
+
     def sync_operation(self, name: str) -> None:
         _lib.check(self._L.pccl_hip_sync(self._h, name.encode()))
 
@@ -170,6 +182,31 @@ class Engine:
         outs = self._as_list([slot[i][1] for i in range(self.num_vranks)], "outputs")
         del self._posted[name]
         self._launch(name, ins, outs, sync)
+
+
+class PreparedCall:
+    """An operation bound to fixed tensors (see ``Engine.prepare``).  Keeps the tensors alive."""
+
+    def __init__(self, engine: Engine, name: str, inputs: List[torch.Tensor], outputs: Optional[List[torch.Tensor]]):
+        self._engine, self._name = engine, name.encode()
+        self.inputs, self.outputs = inputs, outputs if outputs is not None else inputs
+        self._in = engine._ptrs(inputs)
+        self._out = None if outputs is None else engine._ptrs(outputs)
+        self._nb_in = inputs[0].nbytes
+        self._nb_out = self.outputs[0].nbytes
+        self._execute, self._inplace = engine._L.pccl_hip_execute, engine._L.pccl_hip_execute_inplace
+
+    def __call__(self, sync: bool = False, stream: Optional[int] = None):
+        """Launch on `stream` (a raw stream handle) or on the current torch stream."""
+        e = self._engine
+        st = _current_stream_ptr(e.device) if stream is None else stream
+        if self._out is None:
+            rc = self._inplace(e._h, self._name, self._in, self._nb_in, st, int(sync))
+        else:
+            rc = self._execute(e._h, self._name, self._in, self._out, self._nb_in, self._nb_out, st, int(sync))
+        if rc < 0:
+            _lib.check(rc)
+        return self.outputs
 
 
 class RankView:

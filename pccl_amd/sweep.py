@@ -1,7 +1,7 @@
 """Timing sweep over the benchmark configurations other than the headline one.
 
     python -m pccl_amd.sweep [--config c3|c4|c5|all] [--mode auto|column|stepwise] [--reps N]
-                             [--option KEY=VALUE ...]
+                             [--option KEY=VALUE ...] [--prepared]
 
 Prints one JSON line per measurement: kernel time by HIP events on the launch stream, algorithmic
 bytes (reduce 3*n*esize, copy 2*n*esize summed over the linked program) and GB/s.  Inputs are drawn
@@ -47,6 +47,7 @@ def timed(fn, reps):
 
 
 OPTIONS: list = []   # (key, value) engine options applied to every case
+PREPARED = False     # staged cases through Engine.prepare (argument arrays built once)
 
 
 def run_case(label, world, jsons, make_in, out_elems, mode, reps, inplace):
@@ -63,7 +64,8 @@ def run_case(label, world, jsons, make_in, out_elems, mode, reps, inplace):
             med, best = timed(lambda: eng.execute_inplace("op", x), reps)
         else:
             outs = [torch.empty(out_elems, dtype=x[0].dtype, device="cuda") for _ in range(world)]
-            med, best = timed(lambda: eng.execute_operation_async("op", x, outs), reps)
+            call = eng.prepare("op", x, outs) if PREPARED else (lambda: eng.execute_operation_async("op", x, outs))
+            med, best = timed(call, reps)
         b = info["algorithmic_bytes"]
         print(json.dumps({"case": label, "mode": mode, "in_place": inplace, "levels": info["num_levels"],
                           "data_ops": info["num_data_ops"], "algorithmic_bytes": b,
@@ -83,7 +85,11 @@ def main() -> int:
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
                     help="engine option for every case (e.g. lds_slots=0); repeatable")
+    ap.add_argument("--prepared", action="store_true",
+                    help="issue the staged calls (c4) through Engine.prepare: only the C call per invocation")
     args = ap.parse_args()
+    global PREPARED
+    PREPARED = args.prepared
     for kv in args.option:
         key, _, val = kv.partition("=")
         OPTIONS.append((key, val))

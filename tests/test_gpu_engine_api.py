@@ -258,3 +258,39 @@ def test_executions_follow_the_callers_stream(engine_factory):
         y = outs[0] * 2                                                             # consumed on it
     side.synchronize()
     assert torch.all(y == 6) and torch.all(outs[1] == 3)
+
+
+def test_prepared_calls(engine_factory):
+    """Engine.prepare binds an operation to fixed tensors; every invocation is just the C call."""
+    world, n = 8, 4096
+    chunk = n // world
+    jsons = graph_jsons("ring", "build_reduce_scatter", world, n, "float16", "sm", 1)
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("rs", j, r)
+    x = seeded_inputs("randn0.1", world, n, "float16", seed=6)
+    want = oracle_buffers(jsons, x, "float16")
+    ins = [t.cuda() for t in x]
+    outs = [torch.zeros(chunk, dtype=torch.float16, device="cuda") for _ in range(world)]
+    call = eng.prepare("rs", ins, outs)
+    for _ in range(3):
+        for o in outs:
+            o.zero_()
+        got = call(sync=True)
+        for r in range(world):
+            assert got[r] is outs[r] and bits_equal(outs[r], want[r][r * chunk:(r + 1) * chunk])
+    # in place, on an explicit stream handle
+    ar = graph_jsons("ring", "build_allreduce", world, n, "float16", "sm", 1)
+    for r, j in enumerate(ar):
+        eng.register_operation_json("ar", j, r)
+    bufs = [t.cuda() for t in x]
+    call = eng.prepare("ar", bufs)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    call(stream=side.cuda_stream)
+    side.synchronize()
+    want = oracle_buffers(ar, x, "float16")
+    for r in range(world):
+        assert bits_equal(bufs[r], want[r])
+    with pytest.raises(ValueError, match="expected 8 tensors"):
+        eng.prepare("ar", bufs[:3])
