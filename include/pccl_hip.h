@@ -216,7 +216,9 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * 289-298, csrc/engine_c.cc:351): key "mode" = "auto" | "column" | "stepwise" | "persistent";
  * "num_blocks" = workgroup cap of a launch (0 = sized to the device); "check_races" = "0" | "1";
  * "timing" = "0" | "1" (record HIP events around the program); "vecs_per_thread" = 1 | 2 | 4;
- * "step_tile_bytes"; "wait_timeout_ms" (how long a persistent launch waits for a predecessor);
+ * "step_tile_bytes" (work item of the level and persistent runners: 0 = chosen from the program's
+ * size, 4 to 32 KiB, else a multiple of 4096); "wait_timeout_ms" (how long a persistent launch waits
+ * for a predecessor);
  * "fuse_staging" = "1" | "0" (allreduce-type calls in column mode read the input tensors and write
  * the output tensors directly instead of staging through the engine's rank buffers);
  * "lds_slots" = "1" | "0" (column runner keeps values it re-reads in per-thread LDS slots, so each

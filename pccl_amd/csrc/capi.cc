@@ -288,7 +288,7 @@ struct pccl_hip_ctx {
     bool level_graph = false;             // level runner replays its launches as one HIP graph (measured:
                                           // no faster than launching level by level, so off by default)
     hipStream_t capture_stream = nullptr; // private stream the level launches are captured on
-    int64_t step_tile_bytes = 16 * 1024;   // work item of the level and persistent runners (persistent: 3.30 ms at 16 KiB, 3.36 at 32, 3.61 at 128, 3.86 at 8 on the headline graph)
+    int64_t step_tile_bytes = 0;   // work item of the level and persistent runners; 0 = automatic, 32 KiB for large programs (persistent, headline graph: 3.91 ms at 8 KiB, 3.16 at 16, 3.10 at 32, 3.35 at 64; sizes that do not divide the ops are slower)
     bool fuse_staging = true;             // run staged calls on the caller's tensors when possible
     int wait_timeout_ms = 2000;           // a persistent launch gives up on a dependency after this long
     hipStream_t last_stream = nullptr;
@@ -396,7 +396,7 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
         e.step_ops.upload(so.data(), so.size() * sizeof(DevStepOp));
         e.step_deps.upload(P.step_deps.data(), P.step_deps.size() * sizeof(int32_t));
         e.item_op.upload(item_op.data(), item_op.size() * sizeof(int32_t));
-        std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * ((size_t)P.num_items + 1), 0);
+        std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * ((size_t)P.num_items + P.ops.size() + 1), 0);
         e.state.upload(zeros.data(), zeros.size());
         e.epoch = 0;
     }
@@ -668,7 +668,7 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
         }
         else if (k == "step_tile_bytes") {
             int64_t b = std::atoll(value);
-            if (b < 4096 || b % 4096) return fail(PCCL_ERR_INVALID, "step_tile_bytes must be a positive multiple of 4096");
+            if (b < 0 || b % 4096) return fail(PCCL_ERR_INVALID, "step_tile_bytes must be 0 (automatic) or a positive multiple of 4096");
             ctx->step_tile_bytes = b; relink = true;
         } else return fail(PCCL_ERR_INVALID, "unknown option '" + k + "'");
         if (relink) {

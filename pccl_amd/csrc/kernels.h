@@ -37,7 +37,8 @@ struct StepState {      // device memory of the persistent runner
     int32_t error_op;   // 1 + index of the op whose bounded wait expired (0 = none); host clears it
     int32_t error_dep;  // 1 + index of the predecessor it was waiting for
     int32_t pad[28];
-    // followed by int32 flag[num_items]: the epoch of the launch that last completed the item
+    // followed by int32 flag[num_items] (the epoch of the launch that last completed the item) and
+    // int32 ready[num_ops] (the epoch of the launch in which the op's first tile last saw all predecessors done)
 };
 
 struct ColumnLaunch {

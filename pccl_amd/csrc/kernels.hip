@@ -411,17 +411,22 @@ __global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int i
 // per item - same-address atomics from 8 XCDs are serialised - which more than doubled the time
 // of the headline graph.)
 //
-// Cross-workgroup visibility: one flag word per item.  All data accesses of this kernel are
-// agent-coherent (see Mem<MEM_COHERENT>), so handing an item over needs no cache-wide operation:
-// every wave waits until its stores have been acknowledged, the workgroup meets at a barrier, and
-// one thread publishes the flag with an agent-scope atomic store; waiters poll with agent-scope
-// atomic loads and meet at a barrier before they touch the data.  (With cached data accesses and
-// an agent-scope release / acquire fence per wave and item - a write-back and an invalidation of
-// the XCD's whole L2 each - the headline graph took 16 ms instead of 3.)  A flag holds the launch
-// epoch, so flags are never cleared.  Every wait is bounded by wall-clock time: when
-// `timeout_ticks` of the 100 MHz counter have passed since the workgroup started, the waiter
-// records (op, predecessor) and every workgroup leaves before its next item, so the grid always
-// drains and the host reports the stall as an error.
+// Cross-workgroup visibility: one flag word per item and one "ready" word per op.  All data
+// accesses of this kernel are agent-coherent (see Mem<MEM_COHERENT>), so handing an item over
+// needs no cache-wide operation: every wave waits until its stores have been acknowledged, the
+// workgroup meets at a barrier, and one thread publishes the item's flag with an agent-scope
+// atomic store.  The workgroup that runs an op's first tile polls the flags of all tiles of all
+// predecessors and then publishes the op's ready word; the op's other tiles (higher item numbers,
+// so the ordering argument above still holds) wait for that one word.  (With every tile polling
+// all the flags itself - a thousand words per predecessor at 16 KiB tiles - the polls were a sixth
+// of the data traffic again, in coherent loads.  One completion counter per op, incremented by
+// every finished tile, was worse still: same-address atomics serialise, 8.1 ms.  With cached data
+// accesses and an agent-scope release / acquire fence per wave and item - a write-back and an
+// invalidation of the XCD's whole L2 each - the headline graph took 16 ms.)  Flags and ready words
+// hold the launch epoch, so they are never cleared.  Every wait is bounded by wall-clock time:
+// when `timeout_ticks` of the 100 MHz counter have passed since the workgroup started, the waiter
+// records (op, predecessor), and it and every workgroup that finds itself waiting afterwards leave
+// before their next item, so the grid always drains and the host reports the stall as an error.
 //
 // Shape of the loop (it matters): the item number is a wave-uniform scalar, so the loop is
 // controlled by scalar branches, and the single-thread blocks (stall check, publish) each sit
@@ -435,38 +440,64 @@ template <int DT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
 void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     constexpr int ES = ElemBytes<DT>::value;
-    __shared__ int s_word;   // broadcast slot of the stall flag
-    int32_t* flags = reinterpret_cast<int32_t*>(L.state + 1);
+    __shared__ int s_stalled;   // set by a waiter that gave up (or saw that another workgroup had)
+    int32_t* flags = reinterpret_cast<int32_t*>(L.state + 1);   // one per item
+    int32_t* ready = flags + L.num_items;                       // one per op
     const int tid = threadIdx.x;
     const uint64_t t_start = __builtin_amdgcn_s_memrealtime();
-    for (int item = blockIdx.x; item < L.num_items; item += gridDim.x) {
-        const int opi = as_const(L.item_op)[item];
-        const DevStepOp op = load_const(L.ops + opi);
-        // wait: thread t watches items t, t+256, ... of each predecessor (no barrier in here)
-        for (int k = 0; k < op.ndeps; ++k) {
-            const int d = as_const(L.deps)[op.dep_start + k];
-            const int first = as_const(L.ops)[d].first_item, nt = as_const(L.ops)[d].ntiles;
-            for (int t = tid; t < nt; t += kThreads) {
-                int nap = 1;
-                while (__hip_atomic_load(&flags[first + t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != L.epoch) {
-                    if (__builtin_amdgcn_s_memrealtime() - t_start > L.timeout_ticks) {
-                        __hip_atomic_store(&L.state->error_dep, d + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        __hip_atomic_store(&L.state->error_op, opi + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        break;
-                    }
-                    if (__hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-                    __builtin_amdgcn_s_sleep(1);
-                    for (int z = 1; z < nap; ++z) __builtin_amdgcn_s_sleep(8);
-                    if (nap < 32) nap <<= 1;
+    if (tid == 0) s_stalled = 0;
+    __syncthreads();
+    // The loop is software-pipelined over the workgroup's items: the descriptor of the next item and
+    // (thread 0) a first look at its ready word are fetched while the current item's data is moving,
+    // so that in the common case - the predecessors finished long ago - an item starts its loads
+    // without a dependent chain of three memory round trips in front of them.
+    int item = blockIdx.x;
+    if (item >= L.num_items) return;
+    int opi = as_const(L.item_op)[item];
+    DevStepOp op = load_const(L.ops + opi);
+    int32_t seen = 0;   // thread 0: the ready word of `op` as last read (0 = not read)
+    for (;;) {
+        const int next = item + (int)gridDim.x;
+        const bool has_next = next < L.num_items;
+        const int nopi = has_next ? as_const(L.item_op)[next] : 0;
+        // wait (no barrier in here).  `word` is what this thread watches, `dep` who is late if it
+        // never arrives.
+        auto wait_for = [&](int32_t* word, int dep) {
+            int nap = 1;
+            while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != L.epoch) {
+                if (__builtin_amdgcn_s_memrealtime() - t_start > L.timeout_ticks) {
+                    __hip_atomic_store(&L.state->error_dep, dep + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&L.state->error_op, opi + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_stalled = 1;
+                    return;
                 }
+                if (__hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { s_stalled = 1; return; }
+                __builtin_amdgcn_s_sleep(1);
+                for (int z = 1; z < nap; ++z) __builtin_amdgcn_s_sleep(8);
+                if (nap < 4) nap <<= 1;   // at most about a microsecond between two looks
             }
+        };
+        const bool opens = item == op.first_item;   // wave-uniform
+        if (opens) {
+            // the op's first tile checks every tile of every predecessor: thread t watches items
+            // t, t + 256, ... of each
+            for (int k = 0; k < op.ndeps; ++k) {
+                const int d = as_const(L.deps)[op.dep_start + k];
+                const int first = as_const(L.ops)[d].first_item, nt = as_const(L.ops)[d].ntiles;
+                for (int t = tid; t < nt; t += kThreads) wait_for(&flags[first + t], d);
+            }
+        } else if (tid == 0 && op.ndeps > 0 && seen != L.epoch) {
+            // every other tile waits for the first tile's verdict, one word
+            wait_for(&ready[opi], as_const(L.deps)[op.dep_start]);
         }
-        __syncthreads();   // every flag this workgroup waited for has been seen; the data accesses below
-                           // are agent-coherent, so no cache needs to be invalidated first
-        if (tid == 0) s_word = __hip_atomic_load(&L.state->error_op, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        const int stalled = __builtin_amdgcn_readfirstlane(s_word);
+        __syncthreads();   // everything this workgroup waited for has been seen; the data accesses
+                           // below are agent-coherent, so no cache needs to be invalidated first
+        const int stalled = __builtin_amdgcn_readfirstlane(s_stalled);
         if (stalled) break;   // a predecessor never arrived: do not touch the data, just leave
+        if (opens && tid == 0 && op.ntiles > 1 && op.ndeps > 0)
+            __hip_atomic_store(&ready[opi], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        DevStepOp nop = op;
+        if (has_next) nop = load_const(L.ops + nopi);
         const int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
         const int64_t cnt = op.size - e0 < L.tile_elems ? op.size - e0 : L.tile_elems;
         char* self = ptrs.p[op.self];
@@ -475,12 +506,17 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
             range_op<DT, true, MEM_COHERENT>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
         else
             range_copy_bytes<MEM_COHERENT>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
+        int32_t nseen = 0;
+        if (tid == 0 && has_next && next != nop.first_item && nop.ndeps > 0)
+            nseen = __hip_atomic_load(&ready[nopi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // every wave: its write-through stores have been acknowledged (they are visible to the
         // whole device) before the workgroup meets and one thread publishes the item
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) __hip_atomic_store(&flags[item], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();   // keeps the single-thread block away from the back edge (see above)
+        if (!has_next) break;
+        item = next; opi = nopi; op = nop; seen = nseen;
     }
 }
 
@@ -824,7 +860,10 @@ static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, h
     if (per_cu > 8) per_cu = 8;
     if (per_cu < 1) per_cu = 1;
     const int resident = current_cus() * per_cu;
-    int grid = L.num_blocks > 0 && L.num_blocks < resident ? L.num_blocks : resident;
+    // Default: 4 workgroups per CU.  On the headline graph 3, 4 and 5 per CU take 3.05 to 3.07 ms,
+    // 8 per CU 3.10 ms, 2 per CU 3.34 ms (32 KiB items).
+    const int wanted = L.num_blocks > 0 ? L.num_blocks : current_cus() * 4;
+    int grid = wanted < resident ? wanted : resident;
     if (grid > L.num_items) grid = L.num_items;
     if (grid <= 0) return 0;
     hipLaunchKernelGGL((persistent_kernel<DT>), dim3(grid), dim3(kThreads), 0, s, L, ptrs);

@@ -376,7 +376,18 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
     }
 
     // ---- stepwise plan
-    P.tile_elems = std::max<int64_t>(opt.step_tile_bytes / es, 1024);
+    int64_t tile_bytes = opt.step_tile_bytes;
+    if (tile_bytes <= 0) {
+        // automatic: 32 KiB items (the fastest on large programs), halved down to 4 KiB while an
+        // average level has fewer than 1024 items - a small program is bound by the latency of its
+        // chain of levels, and needs its few bytes spread over many workgroups
+        int64_t bytes = 0;
+        for (const LinkedOp& L : P.ops) bytes += L.size * es;
+        const int64_t per_level = bytes / std::max(1, P.num_levels);
+        tile_bytes = 32 * 1024;
+        while (tile_bytes > 4096 && per_level / tile_bytes < 1024) tile_bytes >>= 1;
+    }
+    P.tile_elems = std::max<int64_t>(tile_bytes / es, 1024);
     P.step_ops.resize(D);
     int64_t items = 0;
     for (int k = 0; k < D; ++k) {

@@ -100,7 +100,7 @@ struct Program {
 struct LinkOptions {
     bool check_races = true;
     bool conflict_deps = true;     // order data ops by memory conflicts instead of raw chain order
-    int64_t step_tile_bytes = 16 * 1024;
+    int64_t step_tile_bytes = 0;   // bytes per work item of the stepwise plan; 0 = chosen from the program's size
 };
 
 // Throws Error (PCCL_ERR_LINK for deadlock, ambiguous signal pairing, races, bad ranks).
