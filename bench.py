@@ -332,7 +332,7 @@ def main() -> int:
         eng.set_option("mode", "auto")
         persistent = {"mode": "persistent", "ms_per_step": round(pm_ms, 4), "GB/s": round(alg_bytes / (pm_ms * 1e-3) / 1e9, 1),
                       "frac_of_hbm_peak": round(alg_bytes / (pm_ms * 1e-3) / 1e9 / PEAK_GBPS, 4),
-                      "note": "one launch for the whole graph, every op moving its full bytes, ordering by per-item flags"}
+                      "note": "one launch for the whole graph, every op moving its full bytes, ordering by device-side flags (one per work item, one ready word per op)"}
 
     default_runner = not any(kv.split("=")[0] in ("lds_slots", "slot_threads", "slot_direct") for kv in args.option)
     traffic = measured_traffic(args.mode, info["num_levels"]) if (n == N and channels == CHANNELS and default_runner) else None
