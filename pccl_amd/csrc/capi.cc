@@ -112,36 +112,43 @@ int pccl_graph_dtype(const pccl_graph* g) { return g ? g->g.dtype : PCCL_ERR_INV
 int64_t pccl_graph_tensor_elems(const pccl_graph* g) { return g ? g->g.tensor_elems : 0; }
 const char* pccl_graph_collective_type(const pccl_graph* g) { return g ? g->g.collective_type.c_str() : ""; }
 
+// How many of `have` records fit into a caller's array of `cap` (a negative cap holds none).
+static size_t fits(int cap, size_t have) { return cap <= 0 ? 0 : std::min<size_t>((size_t)cap, have); }
+
 int pccl_graph_get_triggers(const pccl_graph* g, pccl_trigger* out, int cap) {
-    if (!g || !out) return fail(PCCL_ERR_INVALID, "null argument");
-    std::vector<pccl_trigger> t;
-    graph_to_triggers(g->g, &t, nullptr);
-    int n = std::min<int>(cap, (int)t.size());
-    std::memcpy(out, t.data(), sizeof(pccl_trigger) * n);
-    return (int)t.size();
+    return guarded([&] {
+        if (!g || !out) return fail(PCCL_ERR_INVALID, "null argument");
+        std::vector<pccl_trigger> t;
+        graph_to_triggers(g->g, &t, nullptr);
+        std::memcpy(out, t.data(), sizeof(pccl_trigger) * fits(cap, t.size()));
+        return (int)t.size();
+    });
 }
 
 int pccl_graph_get_meta(const pccl_graph* g, pccl_primitive_meta* out, int cap) {
-    if (!g || !out) return fail(PCCL_ERR_INVALID, "null argument");
-    std::vector<pccl_primitive_meta> m;
-    graph_to_triggers(g->g, nullptr, &m);
-    int n = std::min<int>(cap, (int)m.size());
-    std::memcpy(out, m.data(), sizeof(pccl_primitive_meta) * n);
-    return (int)m.size();
+    return guarded([&] {
+        if (!g || !out) return fail(PCCL_ERR_INVALID, "null argument");
+        std::vector<pccl_primitive_meta> m;
+        graph_to_triggers(g->g, nullptr, &m);
+        std::memcpy(out, m.data(), sizeof(pccl_primitive_meta) * fits(cap, m.size()));
+        return (int)m.size();
+    });
 }
 
 int pccl_graph_fused_steps(const pccl_graph* g, pccl_fused_step* steps, int cap, int* channel_offsets,
                            int* num_channels) {
-    if (!g) return fail(PCCL_ERR_INVALID, "null argument");
-    std::vector<pccl_fused_step> s;
-    std::vector<int> off;
-    if (!build_fused_steps(g->g, &s, &off))
-        return fail(PCCL_ERR_UNSUPPORTED, "graph is not a set of per-channel linear chains of at most 128 steps");
-    if (steps) std::memcpy(steps, s.data(), sizeof(pccl_fused_step) * std::min<int>(cap, (int)s.size()));
-    if (channel_offsets)
-        for (size_t i = 0; i < off.size() && i <= PCCL_HIP_MAX_CHANNELS; ++i) channel_offsets[i] = off[i];
-    if (num_channels) *num_channels = (int)off.size() - 1;
-    return (int)s.size();
+    return guarded([&] {
+        if (!g) return fail(PCCL_ERR_INVALID, "null argument");
+        std::vector<pccl_fused_step> s;
+        std::vector<int> off;
+        if (!build_fused_steps(g->g, &s, &off))
+            return fail(PCCL_ERR_UNSUPPORTED, "graph is not a set of per-channel linear chains of at most 128 steps");
+        if (steps) std::memcpy(steps, s.data(), sizeof(pccl_fused_step) * fits(cap, s.size()));
+        if (channel_offsets)
+            for (size_t i = 0; i < off.size() && i <= PCCL_HIP_MAX_CHANNELS; ++i) channel_offsets[i] = off[i];
+        if (num_channels) *num_channels = (int)off.size() - 1;
+        return (int)s.size();
+    });
 }
 
 int pccl_program_link(const pccl_graph* const* graphs, int num_vranks, pccl_program** out) {
@@ -166,7 +173,7 @@ int pccl_program_get_info(const pccl_program* p, pccl_program_info* out) {
 
 int pccl_program_get_ops(const pccl_program* p, pccl_linked_op* out, int cap) {
     if (!p || !out) return fail(PCCL_ERR_INVALID, "null argument");
-    int n = std::min<int>(cap, (int)p->p.ops.size());
+    const int n = (int)fits(cap, p->p.ops.size());
     for (int k = 0; k < n; ++k) {
         const LinkedOp& L = p->p.ops[k];
         pccl_linked_op& o = out[k];
@@ -196,8 +203,8 @@ int pccl_program_get_column(const pccl_program* p, int which,
         segs[i].bcast_mask = src[i].bcast_mask;
     }
     static_assert(sizeof(ColInstr) == sizeof(uint64_t), "instruction words");
-    if (instrs) std::memcpy(instrs, P.col_instrs.data(), sizeof(uint64_t) * std::min<size_t>(instr_cap, P.col_instrs.size()));
-    if (pre) std::memcpy(pre, P.col_pre.data(), sizeof(uint64_t) * std::min<size_t>(pre_cap, P.col_pre.size()));
+    if (instrs) std::memcpy(instrs, P.col_instrs.data(), sizeof(uint64_t) * fits(instr_cap, P.col_instrs.size()));
+    if (pre) std::memcpy(pre, P.col_pre.data(), sizeof(uint64_t) * fits(pre_cap, P.col_pre.size()));
     if (which == 1 && !P.direct_segs.empty())
         for (int r = 0; r < P.R; ++r) {
             if (in_window) { in_window[2 * r] = P.direct_in_start[r]; in_window[2 * r + 1] = P.direct_in_end[r]; }
@@ -561,6 +568,10 @@ void check_stall(OpEntry& e, const std::string& name) {
     std::vector<char> zeros(e.state.bytes, 0);
     HIP_TRY(hipMemcpy(e.state.p, zeros.data(), zeros.size(), hipMemcpyHostToDevice));
     e.epoch = 0;
+    const int n_ops = (int)e.prog.ops.size();
+    if (st.error_op > n_ops || st.error_dep < 1 || st.error_dep > n_ops)
+        throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting (its progress block names ops " +
+                                      std::to_string(st.error_op - 1) + " and " + std::to_string(st.error_dep - 1) + ", which the program does not have)"};
     const LinkedOp& a = e.prog.ops[st.error_op - 1];
     const LinkedOp& b = e.prog.ops[st.error_dep - 1];
     throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting: data op " + std::to_string(st.error_op - 1) +
@@ -726,6 +737,10 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
             }
         }
 
+        // the output must hold what the collective hands back; checked before anything is enqueued
+        if (ct == "reduce_scatter" && out_bytes < in_bytes / R) return fail(PCCL_ERR_INVALID, "reduce_scatter output is smaller than one chunk");
+        if (ct == "alltoall" && out_bytes < in_bytes / R * R) return fail(PCCL_ERR_INVALID, "alltoall output is smaller than the input");
+
         // layout of the staged data inside a rank buffer (reference engine_c.cc:468-548)
         size_t need = (size_t)P.buffer_elems * es;
         if (ct == "allgather") need = std::max(need, in_bytes * R);
@@ -748,12 +763,10 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
 
         if (ct == "reduce_scatter") {
             size_t chunk = in_bytes / R;
-            if (out_bytes < chunk) return fail(PCCL_ERR_INVALID, "reduce_scatter output is smaller than one chunk");
             for (int r = 0; r < R; ++r) { off.src[r] = (int64_t)r * (int64_t)chunk; off.dst[r] = 0; }
             rc = launch_stage(bufp, dst, off, R, chunk, s);
         } else if (ct == "alltoall") {
             size_t chunk = in_bytes / R;
-            if (out_bytes < chunk * R) return fail(PCCL_ERR_INVALID, "alltoall output is smaller than the input");
             rc = 0;
             for (int p = 0; p < R && rc == 0; ++p) {
                 for (int r = 0; r < R; ++r) {

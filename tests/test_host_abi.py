@@ -316,3 +316,46 @@ def test_alltoall_gather_plan():
     assert HostProgram([HostGraph.from_json(j) for j in jsons]).info()["num_gather_copies"] == 0
     jsons = graph_jsons("ring", "build_allreduce", 4, 4096, "bfloat16", "sm", 1)
     assert HostProgram([HostGraph.from_json(j) for j in jsons]).info()["num_gather_copies"] == 0
+
+
+def test_damaged_documents_are_errors_not_crashes():
+    """Truncated, corrupted and out-of-range graph documents come back as error codes (or load, and
+    then link or fail to link cleanly): nothing crosses the C ABI as a crash or an exception."""
+    import random
+    L = _lib.lib()
+    rng = random.Random(7)
+    stems = ["ring_ar_sm_w2_n2048_bf16_c1_rank0", "ring_ar_sm_w4_n4096_f32_c2_rank0", "tree_ar_sm_w8_n1024_f32_c1_rank0"]
+    paths = [os.path.join(ROOT, "tests/golden/graphs", s + ".json") for s in stems]
+    loaded = failed = 0
+    for path in paths:
+        text = open(path, "rb").read()
+        for _ in range(150):
+            b = bytearray(text)
+            kind = rng.randrange(4)
+            if kind == 0:
+                b = b[:rng.randrange(len(b))]
+            elif kind == 1:
+                for _ in range(rng.randrange(1, 6)):
+                    b[rng.randrange(len(b))] = rng.randrange(256)
+            elif kind == 2:
+                i = rng.randrange(len(b))
+                del b[i:i + rng.randrange(1, 40)]
+            else:
+                s = b.decode("latin1")
+                nums = list(re.finditer(r"\d+", s))
+                m = rng.choice(nums)
+                s = s[:m.start()] + rng.choice(["-1", "99999999999999999999", "2147483648", "1e9", "0.5", "9223372036854775807"]) + s[m.end():]
+                b = bytearray(s.encode("latin1"))
+            g = ctypes.c_void_p()
+            rc = L.pccl_graph_load_json(bytes(b), len(b), ctypes.byref(g))
+            if rc != 0:
+                failed += 1
+                assert rc < 0 and L.pccl_hip_last_error()
+                continue
+            loaded += 1
+            arr = (ctypes.c_void_p * 2)(g, g)
+            p = ctypes.c_void_p()
+            if L.pccl_program_link(arr, 2, ctypes.byref(p)) == 0:
+                L.pccl_program_free(p)
+            L.pccl_graph_free(g)
+    assert failed > 50 and loaded > 10
