@@ -183,6 +183,8 @@ def main() -> int:
     ap.add_argument("--num-blocks", type=int, default=-1)
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
                     help="engine option to set before the run (e.g. lds_slots=0, slot_threads=128); repeatable")
+    ap.add_argument("--rank-skew-bytes", type=int, default=0,
+                    help="carve the rank buffers out of one allocation, each this many bytes further in than its size")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--gpu-inputs", action="store_true",
@@ -228,7 +230,18 @@ def main() -> int:
     else:
         pristine = make_inputs(n, dev)
     log(f"inputs generated in {time.perf_counter() - t0:.1f} s")
-    bufs = [p.clone() for p in pristine]
+    if args.rank_skew_bytes:
+        # rank buffers carved out of one allocation, rank r starting r * (size + skew) bytes in: the
+        # same position of different ranks then falls on different memory channels
+        stride = n + args.rank_skew_bytes // 2
+        arena = torch.empty(R * stride, dtype=torch.bfloat16, device=dev)
+        bufs = [arena[r * stride:r * stride + n] for r in range(R)]
+        for b, p in zip(bufs, pristine):
+            b.copy_(p)
+        log("rank buffer addresses: " + " ".join(hex(b.data_ptr()) for b in bufs))
+    else:
+        bufs = [p.clone() for p in pristine]
+        log("rank buffer addresses: " + " ".join(hex(b.data_ptr()) for b in bufs))
 
     # the first execution in the process (tables just uploaded, nothing of the buffers in any cache)
     c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -54,6 +54,7 @@ struct ColumnLaunch {
                               // 64, 128 or 256: workgroup size of the slot runner (re-read values in LDS)
     int32_t num_ranks;        // slot runner: LDS slots per thread
     int32_t slot_direct;      // slot runner: 1 = first touches are loaded straight into LDS
+    int32_t xcd_run;          // run length of the tile-to-XCD mapping; filled in by the launcher
 };
 
 struct StepwiseLaunch {
