@@ -294,3 +294,63 @@ def test_prepared_calls(engine_factory):
         assert bits_equal(bufs[r], want[r])
     with pytest.raises(ValueError, match="expected 8 tensors"):
         eng.prepare("ar", bufs[:3])
+
+
+@pytest.mark.parametrize("mode", ["auto", "stepwise"])
+def test_executions_can_be_captured_into_a_graph_of_the_caller(engine_factory, mode):
+    """After a first eager execution (linking and table upload allocate) an execution is kernel
+    launches only, so a caller may capture it into a graph.  Every replay is checked against the
+    oracle, with eager work and synchronisations in between."""
+    world, n = 8, 1 << 16
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2)
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("ar", j, r)
+    eng.set_option("mode", mode)
+    x = seeded_inputs("randn", world, n, "bfloat16", seed=11)
+    want = oracle_buffers(jsons, x, "bfloat16")
+    src = [t.cuda() for t in x]
+    bufs = [torch.empty_like(t) for t in src]
+    for b, t in zip(bufs, src):
+        b.copy_(t)
+    eng.execute_inplace("ar", bufs, sync=True)          # eager: links, uploads, and is the reference run
+    for r in range(world):
+        assert bits_equal(bufs[r], want[r])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for b, t in zip(bufs, src):
+                b.copy_(t)
+            eng.execute_inplace("ar", bufs)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(4):
+        for b in bufs:
+            b.fill_(float(rep))                           # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for r in range(world):
+            assert bits_equal(bufs[r], want[r]), f"replay {rep}, rank {r}"
+
+
+def test_persistent_runner_refuses_stream_capture(engine_factory):
+    world, n = 4, 1 << 12
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("ar", j, r)
+    eng.set_option("mode", "persistent")
+    bufs = [torch.randn(n, device="cuda") for _ in range(world)]
+    eng.execute_inplace("ar", bufs, sync=True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            bufs[0].add_(0)                               # something capturable, so the graph is not empty
+            with pytest.raises(PcclError, match="cannot be captured"):
+                eng.execute_inplace("ar", bufs)
+    torch.cuda.current_stream().wait_stream(side)
+    eng.execute_inplace("ar", bufs, sync=True)            # eager executions still work afterwards
