@@ -456,12 +456,12 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
         L.num_items = (int)P.num_items; L.tile_elems = P.tile_elems; L.state = (StepState*)e.state.p;
         L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
         if (ctx->mode == Mode::Persistent) {
-            // The launch number is a kernel argument: a captured launch would replay the same number,
-            // find every flag of the previous replay already set and skip all its waits.
+            // The launch number is a kernel argument, which every replay of a recorded launch would
+            // repeat (finding all flags of the previous replay set): on a capturing stream the
+            // number comes from a device-side counter that a one-thread kernel advances first.
             hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-            if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
-                throw Error{PCCL_ERR_UNSUPPORTED, "the persistent runner cannot be captured into a HIP graph (its launch number is a kernel argument); use mode auto or stepwise on a capturing stream"};
-            L.epoch = ++e.epoch;                 // flags of this launch carry this value; never cleared
+            const bool capturing = hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
+            L.epoch = capturing ? 0 : ++e.epoch;
             L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
             rc = launch_persistent(L, ptrs, stream);   // sizes the grid to what is resident at once
             e.ran_persistent = true;

@@ -33,7 +33,7 @@ struct DevStepOp {
 
 struct StepState {      // device memory of the persistent runner
     uint32_t reserved0;
-    int32_t reserved;
+    int32_t graph_epoch;   // launch number of the last launch recorded into a graph (see StepwiseLaunch::epoch)
     int32_t error_op;   // 1 + index of the op whose bounded wait expired (0 = none); host clears it
     int32_t error_dep;  // 1 + index of the predecessor it was waiting for
     int32_t pad[28];
@@ -67,7 +67,8 @@ struct StepwiseLaunch {
     StepState* state;
     int32_t dtype;
     int32_t num_blocks;
-    int32_t epoch;            // persistent runner: value a completed item's flag takes in this launch
+    int32_t epoch;            // persistent runner: value a completed item's flag takes in this launch;
+                              // 0: take it from StepState::graph_epoch, which the launcher advances first
     uint32_t reserved1;
     uint64_t timeout_ticks;   // persistent runner: 100 MHz ticks a workgroup may run before a wait gives up
 };

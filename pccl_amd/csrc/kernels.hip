@@ -395,6 +395,13 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const DevGatherCopy* c
     }
 }
 
+// Launch numbers of recorded launches start here, far from the host's own count (1, 2, ...).
+constexpr int32_t kGraphEpochBase = 0x40000000;
+__global__ void advance_graph_epoch_kernel(StepState* state) {
+    const int32_t e = state->graph_epoch;
+    __hip_atomic_store(&state->graph_epoch, (e < kGraphEpochBase ? kGraphEpochBase : e) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* dst, int64_t nwords) {
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * kThreads) dst[i] = 0;
 }
@@ -479,6 +486,11 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     int32_t* ready = flags + L.num_items;                       // one per op
     const int tid = threadIdx.x;
     const uint64_t t_start = __builtin_amdgcn_s_memrealtime();
+    // The launch number that flags and ready words take: a kernel argument, or - for a launch
+    // recorded into a graph, whose arguments every replay repeats - the device-side counter that
+    // the one-thread kernel recorded in front of this one has just advanced.
+    const int32_t epoch = L.epoch != 0 ? L.epoch
+                                       : __hip_atomic_load(&L.state->graph_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tid == 0) s_stalled = 0;
     __syncthreads();
     // The loop is software-pipelined over the workgroup's items: the descriptor of the next item and
@@ -498,7 +510,7 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
         // never arrives.
         auto wait_for = [&](int32_t* word, int dep) {
             int nap = 1;
-            while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != L.epoch) {
+            while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != epoch) {
                 if (__builtin_amdgcn_s_memrealtime() - t_start > L.timeout_ticks) {
                     __hip_atomic_store(&L.state->error_dep, dep + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(&L.state->error_op, opi + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -520,7 +532,7 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
                 const int first = as_const(L.ops)[d].first_item, nt = as_const(L.ops)[d].ntiles;
                 for (int t = tid; t < nt; t += kThreads) wait_for(&flags[first + t], d);
             }
-        } else if (tid == 0 && op.ndeps > 0 && seen != L.epoch) {
+        } else if (tid == 0 && op.ndeps > 0 && seen != epoch) {
             // every other tile waits for the first tile's verdict, one word
             wait_for(&ready[opi], as_const(L.deps)[op.dep_start]);
         }
@@ -529,7 +541,7 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
         const int stalled = __builtin_amdgcn_readfirstlane(s_stalled);
         if (stalled) break;   // a predecessor never arrived: do not touch the data, just leave
         if (opens && tid == 0 && op.ntiles > 1 && op.ndeps > 0)
-            __hip_atomic_store(&ready[opi], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&ready[opi], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         DevStepOp nop = op;
         if (has_next) nop = load_const(L.ops + nopi);
         const int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
@@ -547,7 +559,7 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
         // whole device) before the workgroup meets and one thread publishes the item
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == 0) __hip_atomic_store(&flags[item], L.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) __hip_atomic_store(&flags[item], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();   // keeps the single-thread block away from the back edge (see above)
         if (!has_next) break;
         item = next; opi = nopi; op = nop; seen = nseen;
@@ -895,15 +907,19 @@ static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, h
     // that, the bound from the vector registers it reports and what the runtime says.  (A form of
     // this kernel that needed 100 scalar registers fitted only 7 times per CU while the runtime's
     // estimate said 8: the grid was one workgroup per CU too large and waits expired.)
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, persistent_kernel<DT>, kThreads, 0) != hipSuccess || per_cu <= 0) per_cu = 1;
-    hipFuncAttributes attr;
-    if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(persistent_kernel<DT>)) == hipSuccess && attr.numRegs > 0) {
-        const int by_vgpr = 512 / ((attr.numRegs + 7) / 8 * 8);
-        if (by_vgpr < per_cu) per_cu = by_vgpr;
+    static int cached_per_cu = 0;   // per instantiation; the queries are made once
+    int per_cu = cached_per_cu;
+    if (per_cu == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, persistent_kernel<DT>, kThreads, 0) != hipSuccess || per_cu <= 0) per_cu = 1;
+        hipFuncAttributes attr;
+        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(persistent_kernel<DT>)) == hipSuccess && attr.numRegs > 0) {
+            const int by_vgpr = 512 / ((attr.numRegs + 7) / 8 * 8);
+            if (by_vgpr < per_cu) per_cu = by_vgpr;
+        }
+        if (per_cu > 8) per_cu = 8;
+        if (per_cu < 1) per_cu = 1;
+        cached_per_cu = per_cu;
     }
-    if (per_cu > 8) per_cu = 8;
-    if (per_cu < 1) per_cu = 1;
     const int resident = current_cus() * per_cu;
     // Default: 4 workgroups per CU.  On the headline graph 3, 4 and 5 per CU take 3.05 to 3.07 ms,
     // 8 per CU 3.10 ms, 2 per CU 3.34 ms (32 KiB items).
@@ -917,6 +933,11 @@ static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, h
 
 int launch_persistent(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream) {
     hipStream_t s = (hipStream_t)stream;
+    if (L.epoch == 0) {   // the launch number comes from the device-side counter: advance it first
+        hipLaunchKernelGGL(advance_graph_epoch_kernel, dim3(1), dim3(1), 0, s, L.state);
+        hipError_t rc = hipGetLastError();
+        if (rc != hipSuccess) return (int)rc;
+    }
     switch (L.dtype) {
         case PCCL_F32: return launch_persistent_dt<PCCL_F32>(L, ptrs, s);
         case PCCL_F16: return launch_persistent_dt<PCCL_F16>(L, ptrs, s);
