@@ -45,6 +45,8 @@ CASES = [
     ("tree", 8, 8192, "float16", 1, "randn0.1"),
     ("ring", 8, 1 << 16, "float8_e4m3", 2, "randn"),       # fp8: add in f16, saturating narrow
     ("rhd", 8, 1 << 15, "float8_e5m2", 1, "randn"),
+    ("ring", 24, 24 * 2731, "bfloat16", 1, "randn"),       # more than 16 ranks and nothing read back:
+                                                           # column mode picks the register runner
 ]
 
 
