@@ -56,17 +56,17 @@ class DeviceProfile:
 
 H100_PROFILE = DeviceProfile()
 
-# One MI355X, virtual ranks in its HBM.  A chunk copy streams at 6.3 TB/s of traffic = 3.1 TB/s of
-# payload; a chunk reduce (two reads, one write) at 6.4 TB/s of traffic = 2.1 TB/s of payload =
-# 535 G four-byte elements per second; one more dependency level costs one more launch of the
+# One MI355X, virtual ranks in its HBM.  A chunk copy streams at 6.7 TB/s of traffic = 3.35 TB/s
+# of payload; a chunk reduce (two reads, one write) at 6.6 TB/s of traffic = 2.2 TB/s of payload =
+# 550 G four-byte elements per second; one more dependency level costs one more launch of the
 # level runner (about 4.5 us back to back).  tma.* run as the sm.* ops.
 MI355X_PROFILE = DeviceProfile(
     name="mi355x-vranks",
     launch_overhead_us=4.5,
-    bandwidth_gb_s={"sm": 3100.0, "tma": 3100.0, "host": 10.0},
-    reduce_throughput_gops={"sm": 535.0, "tma": 535.0},
+    bandwidth_gb_s={"sm": 3350.0, "tma": 3350.0, "host": 10.0},
+    reduce_throughput_gops={"sm": 550.0, "tma": 550.0},
     num_channels=8,
-    per_channel_bw_gb_s={"sm": 3100.0, "tma": 3100.0, "host": 10.0},
+    per_channel_bw_gb_s={"sm": 3350.0, "tma": 3350.0, "host": 10.0},
     channel_launch_overhead_us=0.0,
 )
 
