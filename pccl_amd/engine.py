@@ -129,7 +129,8 @@ class Engine:
     def execute_inplace(self, name: str, bufs: TensorList, sync: bool = False):
         """Zero-copy execution: ``bufs[r]`` is rank ``r``'s buffer and is updated in place."""
         bs = self._as_list(bufs, "bufs")
-        _lib.check(self._L.pccl_hip_execute_inplace(self._h, name.encode(), self._ptrs(bs), bs[0].nbytes,
+        # the library checks the program's extent against one size: the smallest buffer's
+        _lib.check(self._L.pccl_hip_execute_inplace(self._h, name.encode(), self._ptrs(bs), min(b.nbytes for b in bs),
                                                     _current_stream_ptr(self.device), int(sync)))
         return bs
 

@@ -137,6 +137,9 @@ def test_buffer_checks_and_mode_selection(engine_factory):
     small = [torch.zeros(n // 2, device="cuda") for _ in range(world)]
     with pytest.raises(PcclError, match="smaller than"):
         eng.execute_inplace("ar", small, sync=True)
+    one_small = [torch.zeros(n, device="cuda"), torch.zeros(n // 2, device="cuda")]   # any rank counts
+    with pytest.raises(PcclError, match="smaller than"):
+        eng.execute_inplace("ar", one_small, sync=True)
     # buffers that are only 4-byte aligned: auto falls back to the level runner, column refuses
     base = [torch.zeros(n + 4, device="cuda") for _ in range(world)]
     shifted = [b[1:n + 1] for b in base]
