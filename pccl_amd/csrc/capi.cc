@@ -399,9 +399,10 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
             const LinkedOp& L = P.ops[k];
             DevStepOp& d = so[k];
             d.off0 = L.off0; d.off1 = L.off1; d.off2 = L.off2; d.size = L.size;
-            d.self = L.rank; d.peer = L.peer; d.is_reduce = L.is_reduce; d.redop = L.redop;
+            d.who = (uint32_t)L.rank | (uint32_t)L.peer << 8 | (uint32_t)(L.is_reduce ? 1 : 0) << 16 | (uint32_t)L.redop << 24;
             d.first_item = P.step_ops[k].first_item; d.ntiles = P.step_ops[k].ntiles;
             d.dep_start = P.step_ops[k].dep_start; d.ndeps = P.step_ops[k].ndeps;
+            d.lead = P.step_ops[k].lead; d.pad_[0] = d.pad_[1] = 0;
             if (d.ndeps > 256) throw Error{PCCL_ERR_UNSUPPORTED, "a data op with more than 256 direct predecessors"};
             for (int t = 0; t < d.ntiles; ++t) item_op[(size_t)d.first_item + t] = (int32_t)k;
         }

@@ -5,6 +5,13 @@
 
 #include "../../include/pccl_hip.h"
 
+// accessors usable in kernels and in the host-only translation units
+#ifdef __HIPCC__
+#define PCCL_HD __host__ __device__
+#else
+#define PCCL_HD
+#endif
+
 namespace pccl_hip {
 
 // Rank-buffer base pointers handed to a kernel by value (kernarg segment).  Entry r is where
@@ -25,11 +32,20 @@ struct DevColSegment {
     uint64_t bcast_mask;     // ranks that receive the accumulator after the last instruction
 };
 
-struct DevStepOp {
+struct DevStepOp {    // 64 bytes: one 16-dword scalar load
     int64_t off0, off1, off2, size;  // elements
-    int32_t self, peer, is_reduce, redop;
+    uint32_t who;    // self rank | peer rank << 8 | is_reduce << 16 | reduce operator << 24
     int32_t first_item, ntiles, dep_start, ndeps;
+    int32_t lead;    // the op's items sit on a grid of tile_elems anchored `lead` elements in front of its
+                     // first element, chosen so that item boundaries fall on multiples of the tile size
+                     // in the destination buffer: only the first and last item of an op are ragged
+    int32_t pad_[2];
+    PCCL_HD int self() const { return who & 0xFF; }
+    PCCL_HD int peer() const { return (who >> 8) & 0xFF; }
+    PCCL_HD bool is_reduce() const { return (who >> 16) & 1; }
+    PCCL_HD int redop() const { return who >> 24; }
 };
+static_assert(sizeof(DevStepOp) == 64, "DevStepOp is read with one scalar load");
 
 struct StepState {      // device memory of the persistent runner
     uint32_t reserved0;

@@ -332,49 +332,57 @@ constexpr int64_t kPrimTileBytes = 4 * 1024;
 // The mapping is a bijection on [0, round_up(tiles, 8 * run)); the caller skips what falls beyond.
 constexpr int kXcds = 8;
 constexpr int kXcdRun = 256;
+// `run` is a power of two, so all of this is shifts and masks (a 64-bit division by a run-time
+// value would be some forty scalar instructions in front of every workgroup's first load).
 __host__ __device__ __forceinline__ int64_t span_tiles(int64_t tiles, int run) {
     const int64_t span = (int64_t)kXcds * run;
-    return (tiles + span - 1) / span * span;
+    return (tiles + span - 1) & ~(span - 1);
 }
 __device__ __forceinline__ int64_t xcd_tile(int64_t w, int run) {
-    const int64_t span = (int64_t)kXcds * run, in = w % span;
-    return w - in + (in % kXcds) * run + in / kXcds;
+    const int shift = __builtin_ctz((unsigned)run);
+    const int64_t in = w & ((int64_t)kXcds * run - 1);
+    return w - in + ((in & (kXcds - 1)) << shift) + (in >> 3);
 }
+static_assert(kXcds == 8 && (kXcdRun & (kXcdRun - 1)) == 0, "xcd_tile shifts by 3 and by log2(run)");
 
+// Tiles are anchored at multiples of 4 KiB of the destination address, not at the start of the
+// range: a range that starts at an odd address has ragged tiles at its two ends only.
 template <int DT>
 __global__ __launch_bounds__(kThreads) void reduce_kernel(const char* a, const char* b, char* c, int64_t n, int redop, int run) {
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int64_t TE = kPrimTileBytes / ES;
-    int64_t ntiles = (n + TE - 1) / TE;
+    const int64_t lead = (int64_t)((uintptr_t)c % kPrimTileBytes) / ES;
+    const int64_t ntiles = (n + lead + TE - 1) / TE;
     for (int64_t w = blockIdx.x; w < span_tiles(ntiles, run); w += gridDim.x) {
         const int64_t t = xcd_tile(w, run);
         if (t >= ntiles) continue;
-        int64_t e0 = t * TE, cnt = n - e0 < TE ? n - e0 : TE;
-        range_op<DT, true>(a + e0 * ES, b + e0 * ES, c + e0 * ES, cnt, redop, threadIdx.x, kThreads);
+        int64_t e0 = t * TE - lead, e1 = e0 + TE;
+        if (e0 < 0) e0 = 0;
+        if (e1 > n) e1 = n;
+        range_op<DT, true>(a + e0 * ES, b + e0 * ES, c + e0 * ES, e1 - e0, redop, threadIdx.x, kThreads);
+    }
+}
+
+__device__ __forceinline__ void copy_tiles(const char* src, char* dst, int64_t nbytes, int run) {
+    const int64_t lead = (int64_t)((uintptr_t)dst % kPrimTileBytes);
+    const int64_t ntiles = (nbytes + lead + kPrimTileBytes - 1) / kPrimTileBytes;
+    for (int64_t w = blockIdx.x; w < span_tiles(ntiles, run); w += gridDim.x) {
+        const int64_t t = xcd_tile(w, run);
+        if (t >= ntiles) continue;
+        int64_t b0 = t * kPrimTileBytes - lead, b1 = b0 + kPrimTileBytes;
+        if (b0 < 0) b0 = 0;
+        if (b1 > nbytes) b1 = nbytes;
+        range_copy_bytes(src + b0, dst + b0, b1 - b0, threadIdx.x, kThreads);
     }
 }
 
 __global__ __launch_bounds__(kThreads) void copy_kernel(const char* src, char* dst, int64_t nbytes, int run) {
-    int64_t ntiles = (nbytes + kPrimTileBytes - 1) / kPrimTileBytes;
-    for (int64_t w = blockIdx.x; w < span_tiles(ntiles, run); w += gridDim.x) {
-        const int64_t t = xcd_tile(w, run);
-        if (t >= ntiles) continue;
-        int64_t b0 = t * kPrimTileBytes, cnt = nbytes - b0 < kPrimTileBytes ? nbytes - b0 : kPrimTileBytes;
-        range_copy_bytes(src + b0, dst + b0, cnt, threadIdx.x, kThreads);
-    }
+    copy_tiles(src, dst, nbytes, run);
 }
 
 __global__ __launch_bounds__(kThreads) void stage_kernel(RankPtrs src, RankPtrs dst, StageOffsets off, int64_t nbytes, int run) {
-    int r = blockIdx.y;
-    const char* s = src.p[r] + off.src[r];
-    char* d = dst.p[r] + off.dst[r];
-    int64_t ntiles = (nbytes + kPrimTileBytes - 1) / kPrimTileBytes;
-    for (int64_t w = blockIdx.x; w < span_tiles(ntiles, run); w += gridDim.x) {
-        const int64_t t = xcd_tile(w, run);
-        if (t >= ntiles) continue;
-        int64_t b0 = t * kPrimTileBytes, cnt = nbytes - b0 < kPrimTileBytes ? nbytes - b0 : kPrimTileBytes;
-        range_copy_bytes(s + b0, d + b0, cnt, threadIdx.x, kThreads);
-    }
+    const int r = blockIdx.y;
+    copy_tiles(src.p[r] + off.src[r], dst.p[r] + off.dst[r], nbytes, run);
 }
 
 // A list of independent copies between rank tensors in one launch (the staged alltoall call composed
@@ -421,20 +429,30 @@ __global__ __launch_bounds__(kThreads) void level_kernel(StepwiseLaunch L, int i
     for (int64_t u = blockIdx.x; u < span_tiles(total, run); u += gridDim.x) {
         const int64_t w = xcd_tile(u, run);
         if (w >= total) continue;
-        int item = item_begin + (int)(w / subs);
-        int64_t sub = w % subs;
+        int item;
+        int64_t sub;
+        if ((subs & (subs - 1)) == 0) {   // the usual case: item sizes are powers of two
+            item = item_begin + (int)(w >> __builtin_ctz((unsigned)subs));
+            sub = w & (subs - 1);
+        } else {
+            item = item_begin + (int)(w / subs);
+            sub = w % subs;
+        }
         int opi = as_const(L.item_op)[item];
         DevStepOp op = load_const(L.ops + opi);
-        int64_t t0 = (int64_t)(item - op.first_item) * L.tile_elems;
-        int64_t tcnt = op.size - t0 < L.tile_elems ? op.size - t0 : L.tile_elems;
-        int64_t e0 = t0 + sub * SUB_ELEMS;
-        int64_t cnt = tcnt - sub * SUB_ELEMS;
+        // items and pieces sit on a grid anchored `lead` elements in front of the op (see DevStepOp)
+        int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems + sub * SUB_ELEMS - op.lead;
+        int64_t e1 = e0 + SUB_ELEMS;
+        const int64_t item_end = (int64_t)(item - op.first_item + 1) * L.tile_elems - op.lead;
+        if (e1 > item_end) e1 = item_end;
+        if (e1 > op.size) e1 = op.size;
+        if (e0 < 0) e0 = 0;
+        const int64_t cnt = e1 - e0;
         if (cnt <= 0) continue;
-        if (cnt > SUB_ELEMS) cnt = SUB_ELEMS;
-        char* self = ptrs.p[op.self];
-        const char* peer = ptrs.p[op.peer];
-        if (op.is_reduce)
-            range_op<DT, true>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
+        char* self = ptrs.p[op.self()];
+        const char* peer = ptrs.p[op.peer()];
+        if (op.is_reduce())
+            range_op<DT, true>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop(), tid, kThreads);
         else
             range_copy_bytes(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
     }
@@ -544,12 +562,15 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
             __hip_atomic_store(&ready[opi], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         DevStepOp nop = op;
         if (has_next) nop = load_const(L.ops + nopi);
-        const int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems;
-        const int64_t cnt = op.size - e0 < L.tile_elems ? op.size - e0 : L.tile_elems;
-        char* self = ptrs.p[op.self];
-        const char* peer = ptrs.p[op.peer];
-        if (op.is_reduce)
-            range_op<DT, true, MEM_COHERENT>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop, tid, kThreads);
+        int64_t e0 = (int64_t)(item - op.first_item) * L.tile_elems - op.lead;
+        int64_t e1 = e0 + L.tile_elems;
+        if (e0 < 0) e0 = 0;
+        if (e1 > op.size) e1 = op.size;
+        const int64_t cnt = e1 - e0;
+        char* self = ptrs.p[op.self()];
+        const char* peer = ptrs.p[op.peer()];
+        if (op.is_reduce())
+            range_op<DT, true, MEM_COHERENT>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, self + (op.off2 + e0) * ES, cnt, op.redop(), tid, kThreads);
         else
             range_copy_bytes<MEM_COHERENT>(peer + (op.off0 + e0) * ES, self + (op.off1 + e0) * ES, cnt * ES, tid, kThreads);
         int32_t nseen = 0;
@@ -982,7 +1003,7 @@ int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, s
     hipStream_t s = (hipStream_t)stream;
     const char* pa = (const char*)a; const char* pb = (const char*)b; char* pc = (char*)c;
     int es = (dtype == PCCL_F32 || dtype == PCCL_I32) ? 4 : (dtype == PCCL_F16 || dtype == PCCL_BF16) ? 2 : 1;
-    const int64_t ntiles = ((int64_t)n * es + kPrimTileBytes - 1) / kPrimTileBytes;
+    const int64_t ntiles = ((int64_t)n * es + kPrimTileBytes - 1) / kPrimTileBytes + 1;   // + 1: tiles are anchored at aligned addresses
     const int run = run_for_tiles(ntiles);
     int grid = grid_for_tiles(ntiles, run);
     switch (dtype) {
@@ -999,7 +1020,7 @@ int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, s
 
 int launch_copy_bytes(const void* src, void* dst, size_t nbytes, void* stream) {
     if (nbytes == 0) return 0;
-    const int64_t ntiles = ((int64_t)nbytes + kPrimTileBytes - 1) / kPrimTileBytes;
+    const int64_t ntiles = ((int64_t)nbytes + kPrimTileBytes - 1) / kPrimTileBytes + 1;   // + 1: tiles are anchored at aligned addresses
     const int run = run_for_tiles(ntiles);
     hipLaunchKernelGGL(copy_kernel, dim3(grid_for_tiles(ntiles, run)), dim3(kThreads), 0, (hipStream_t)stream, (const char*)src, (char*)dst, (int64_t)nbytes, run);
     return (int)hipGetLastError();
@@ -1007,7 +1028,7 @@ int launch_copy_bytes(const void* src, void* dst, size_t nbytes, void* stream) {
 
 int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& off, int R, size_t bytes, void* stream) {
     if (bytes == 0 || R <= 0) return 0;
-    int64_t ntiles = ((int64_t)bytes + kPrimTileBytes - 1) / kPrimTileBytes;
+    int64_t ntiles = ((int64_t)bytes + kPrimTileBytes - 1) / kPrimTileBytes + 1;   // + 1: tiles are anchored at aligned addresses
     const int run = run_for_tiles(ntiles);
     const int64_t cap = 1 << 24, want = span_tiles(ntiles, run);
     int gx = (int)(want < cap ? want : cap);   // a multiple of 8, so that blockIdx.x % 8 is the XCD in every row

@@ -393,7 +393,11 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
     for (int k = 0; k < D; ++k) {
         StepOpPlan& s = P.step_ops[k];
         s.first_item = (int)items;
-        s.ntiles = (int)((P.ops[k].size + P.tile_elems - 1) / P.tile_elems);
+        // the item grid is anchored at a multiple of the tile size in the destination buffer, so
+        // that an op with an odd start still has whole, aligned items everywhere but at its ends
+        const int64_t dst = P.ops[k].is_reduce ? P.ops[k].off2 : P.ops[k].off1;
+        s.lead = (int)(dst % P.tile_elems);
+        s.ntiles = (int)((P.ops[k].size + s.lead + P.tile_elems - 1) / P.tile_elems);
         s.dep_start = (int)P.step_deps.size();
         s.ndeps = (int)P.ops[k].deps.size();
         for (int d : P.ops[k].deps) P.step_deps.push_back(d);

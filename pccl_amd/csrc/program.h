@@ -57,6 +57,7 @@ struct ColSegment {
 
 struct StepOpPlan {
     int first_item = 0, ntiles = 0, dep_start = 0, ndeps = 0;
+    int lead = 0;   // elements between the item grid's anchor and the op's first element (< tile_elems)
 };
 
 struct Program {
