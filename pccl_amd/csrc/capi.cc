@@ -238,6 +238,7 @@ struct OpEntry {
     Program prog;
     DevBuf gather;                        // gather plan of an alltoall graph (DevGatherCopy records)
     int64_t gather_tiles = 0;
+    int gather_copy_tiles = 0;            // > 0: every copy of the gather plan has this many tiles
     DevBuf segs, direct_segs, instrs, pre, step_ops, step_deps, item_op, state;
     int64_t total_tiles = 0, direct_tiles = 0;
     int vecs_per_thread = 0;
@@ -389,6 +390,12 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
             tiles += (gc[i].bytes + 4095) / 4096;
         }
         e.gather_tiles = tiles;
+        // all copies the same number of tiles (an alltoall's equal chunks)?
+        const int64_t per = gc.size() > 1 ? gc[1].first_tile : tiles;
+        e.gather_copy_tiles = 0;
+        bool same = per > 0 && tiles == per * (int64_t)gc.size() && tiles <= INT32_MAX;
+        for (size_t i = 0; i < gc.size() && same; ++i) same = gc[i].first_tile == (int64_t)i * per;
+        if (same) e.gather_copy_tiles = (int)per;
         e.gather.upload(gc.data(), gc.size() * sizeof(DevGatherCopy));
     }
     // stepwise plan
@@ -743,7 +750,7 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
                 RankPtrs src{}, dst{};
                 for (int r = 0; r < R; ++r) { src.p[r] = (char*)inputs[r]; dst.p[r] = (char*)outputs[r]; }
                 if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, s));
-                int grc = launch_gather((const DevGatherCopy*)e.gather.p, (int)P.gather.size(), e.gather_tiles, src, dst, s);
+                int grc = launch_gather((const DevGatherCopy*)e.gather.p, (int)P.gather.size(), e.gather_tiles, e.gather_copy_tiles, src, dst, s);
                 if (grc) return fail(PCCL_ERR_HIP, std::string("gather launch failed: ") + hipGetErrorString((hipError_t)grc));
                 if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, s)); e.timed = true; }
                 ctx->last_stream = s;

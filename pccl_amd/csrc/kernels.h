@@ -100,7 +100,8 @@ int launch_copy_bytes(const void* src, void* dst, size_t nbytes, void* stream);
 // One direct copy of a gather plan: `bytes` from src.p[src_rank] + src_off to dst.p[dst_rank] + dst_off;
 // first_tile = tiles of all earlier copies (4 KiB tiles, one workgroup each).
 struct DevGatherCopy { int64_t src_off, dst_off, bytes, first_tile; int32_t src_rank, dst_rank; };
-int launch_gather(const DevGatherCopy* copies, int n, int64_t total_tiles, const RankPtrs& src, const RankPtrs& dst, void* stream);
+// copy_tiles > 0: every copy has that many tiles (copy = tile / copy_tiles); 0: search the prefix sums.
+int launch_gather(const DevGatherCopy* copies, int n, int64_t total_tiles, int copy_tiles, const RankPtrs& src, const RankPtrs& dst, void* stream);
 
 struct StageOffsets { int64_t src[PCCL_HIP_MAX_VRANKS]; int64_t dst[PCCL_HIP_MAX_VRANKS]; };
 int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& off, int R, size_t bytes, void* stream);

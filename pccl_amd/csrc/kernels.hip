@@ -387,14 +387,24 @@ __global__ __launch_bounds__(kThreads) void stage_kernel(RankPtrs src, RankPtrs 
 
 // A list of independent copies between rank tensors in one launch (the staged alltoall call composed
 // into direct copies): workgroup w finds its copy by binary search over the tile prefix sums.
-__global__ __launch_bounds__(kThreads) void gather_kernel(const DevGatherCopy* copies, int n, int64_t total_tiles, RankPtrs src, RankPtrs dst, int run) {
+// (When all copies have the same number of tiles - an alltoall's chunks - the search is one
+// division: a workgroup here moves 4 KiB, and the six dependent table reads of the search in front
+// of that cost 8 x 256 MiB 13 % of its time, 0.76 against 0.66 ms.  The level runner's one extra
+// table read, item -> op, is not worth replacing the same way: measured 0.5 % slower.)
+__global__ __launch_bounds__(kThreads) void gather_kernel(const DevGatherCopy* copies, int n, int64_t total_tiles, int copy_tiles, RankPtrs src, RankPtrs dst, int run) {
     for (int64_t u = blockIdx.x; u < span_tiles(total_tiles, run); u += gridDim.x) {
         const int64_t w = xcd_tile(u, run);
         if (w >= total_tiles) continue;
-        int lo = 0, hi = n;
-        while (hi - lo > 1) {
-            int mid = (lo + hi) >> 1;
-            if (as_const(copies)[mid].first_tile <= w) lo = mid; else hi = mid;
+        int lo = 0;
+        if (copy_tiles > 0) {
+            const uint32_t per = (uint32_t)copy_tiles;
+            lo = (per & (per - 1)) == 0 ? (int)((uint32_t)w >> __builtin_ctz(per)) : (int)((uint32_t)w / per);
+        } else {
+            int hi = n;
+            while (hi - lo > 1) {
+                int mid = (lo + hi) >> 1;
+                if (as_const(copies)[mid].first_tile <= w) lo = mid; else hi = mid;
+            }
         }
         const DevGatherCopy c = load_const(copies + lo);
         const int64_t b0 = (w - c.first_tile) * kPrimTileBytes;
@@ -1036,10 +1046,10 @@ int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& o
     return (int)hipGetLastError();
 }
 
-int launch_gather(const DevGatherCopy* copies, int n, int64_t total_tiles, const RankPtrs& src, const RankPtrs& dst, void* stream) {
+int launch_gather(const DevGatherCopy* copies, int n, int64_t total_tiles, int copy_tiles, const RankPtrs& src, const RankPtrs& dst, void* stream) {
     if (n <= 0 || total_tiles <= 0) return 0;
     const int run = run_for_tiles(total_tiles);
-    hipLaunchKernelGGL(gather_kernel, dim3(grid_for_tiles(total_tiles, run)), dim3(kThreads), 0, (hipStream_t)stream, copies, n, total_tiles, src, dst, run);
+    hipLaunchKernelGGL(gather_kernel, dim3(grid_for_tiles(total_tiles, run)), dim3(kThreads), 0, (hipStream_t)stream, copies, n, total_tiles, copy_tiles, src, dst, run);
     return (int)hipGetLastError();
 }
 
