@@ -343,3 +343,48 @@ def test_executions_can_be_captured_into_a_graph_of_the_caller(engine_factory, m
     eng.execute_inplace("ar", bufs, sync=True)
     for r in range(world):
         assert bits_equal(bufs[r], want[r]), f"eager execution after the replays, rank {r}"
+
+
+def test_calls_from_several_threads(engine_factory):
+    """One context, four host threads, each with its own stream and tensors, two operations: the
+    context's mutex serialises registration, linking and launches; results stay exact."""
+    import threading
+    world, n = 4, 1 << 14
+    eng = engine_factory(world)
+    specs = {"ar_f32": ("float32", 1), "ar_bf16": ("bfloat16", 2)}
+    want, inputs = {}, {}
+    for name, (dtype, ch) in specs.items():
+        jsons = graph_jsons("ring", "build_allreduce", world, n, dtype, "sm", ch)
+        for r, j in enumerate(jsons):
+            eng.register_operation_json(name, j, r)
+        inputs[name] = seeded_inputs("randn", world, n, dtype, seed=21)
+        want[name] = oracle_buffers(jsons, inputs[name], dtype)
+    errors = []
+
+    def worker(k):
+        try:
+            name = list(specs)[k % 2]
+            stream = torch.cuda.Stream()
+            src = [t.cuda() for t in inputs[name]]
+            with torch.cuda.stream(stream):
+                for it in range(25):
+                    bufs = [t.clone() for t in src]
+                    if it % 2:
+                        eng.execute_inplace(name, bufs)
+                        got = bufs
+                    else:
+                        got = eng.execute_operation_async(name, bufs)
+                    stream.synchronize()
+                    for r in range(world):
+                        if not bits_equal(got[r], want[name][r]):
+                            raise AssertionError(f"thread {k}, iteration {it}, rank {r}")
+        except Exception as e:   # noqa: BLE001 - reported by the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a worker thread did not finish"
+    assert not errors, errors
