@@ -236,7 +236,9 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
  * sync != 0 waits for it. */
 int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inputs,
                      void* const* outputs, size_t in_bytes, size_t out_bytes, void* stream, int sync);
-/* Zero-copy variant: bufs[r] IS rank buffer r (buf_bytes each, 16-byte aligned); no staging. */
+/* Zero-copy variant: bufs[r] IS rank buffer r (every one at least buf_bytes long); no staging.
+ * Buffers that are not 16-byte aligned are run by the level runner instead of the column runner.
+ * No counterpart in the reference, whose rank buffers belong to the engine. */
 int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
                              void* stream, int sync);
 /* Engine::syncOp / Engine::resetSignals (reference csrc/engine_c.cc:562-593). */
