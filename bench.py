@@ -260,6 +260,14 @@ def main() -> int:
         rel = ((bufs[0][:1 << 20].float() - ref32).abs() / ref32.abs().clamp_min(1.0)).max().item()
         verify = {"ranks_identical": bool(same), "matches_ring_order_bf16": bool(exact),
                   "max_rel_err_vs_fp32_sum_first_1Mi": round(rel, 5), "output_sha256": sha256_of(bufs[0])}
+        # at the headline size with the prescribed inputs: the hashes committed with the tests (the
+        # output hash is what the CPU oracle computes at full size, tests/golden/make_headline_sha256.py)
+        golden_path = os.path.join(ROOT, "tests", "golden", "headline_sha256.json")
+        if n == N and channels == CHANNELS and not args.gpu_inputs and os.path.exists(golden_path):
+            golden = json.load(open(golden_path))
+            verify["input_rank0_matches_committed_sha256"] = sha256_of(pristine[0]) == golden["input_sha256_per_rank"][0]
+            verify["output_matches_committed_oracle_sha256"] = verify["output_sha256"] == golden["output_sha256"]
+            exact = exact and verify["input_rank0_matches_committed_sha256"] and verify["output_matches_committed_oracle_sha256"]
         log(f"verify: {verify}")
         del want
         if not (same and exact):
