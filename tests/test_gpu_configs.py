@@ -161,3 +161,21 @@ def test_config2_headline_shape_in_all_modes_agree(engine_factory):
             for k in range(1, world):
                 acc = x[(c + k) % world][lo:lo + per_rank] + acc
             assert same_bits(results["column"][lo:lo + per_rank], acc)
+
+
+def test_config3_full_size_against_the_cpu_oracle(engine_factory):
+    """Configuration 3 at its full size (16 x 64 MiB f32, two channels) with the prescribed inputs
+    from the CPU generator, the GPU result compared bit for bit with the CPU oracle's (about a
+    gigabyte of buffers; the oracle needs a few seconds for it)."""
+    from helpers import bits_equal, oracle_buffers, seeded_inputs
+    world, n = 16, 16_777_216
+    print("config 3 at full size against the oracle", flush=True)
+    jsons = graph_jsons("rhd", "build_allreduce", world, n, "float32", "sm", 2)
+    x = seeded_inputs("uniform", world, n, "float32", seed=0)
+    want = oracle_buffers(jsons, x, "float32")
+    engine = engine_factory(world)
+    register(engine, "c3_oracle", jsons, "auto")
+    bufs = [t.cuda() for t in x]
+    engine.execute_inplace("c3_oracle", bufs, sync=True)
+    for r in range(world):
+        assert bits_equal(bufs[r], want[r]), f"rank {r}"
