@@ -238,3 +238,22 @@ def test_algorithm_selector():                 # reference pccl/dsl/algorithms/s
         assert type(got) is type(cands[costs.index(min(costs))])
     # log-step schedules have the shorter critical path for small messages on 8 ranks
     assert type(select_algorithm_cost_based(0, 8, 8192, 1024)) is not RingAllreduce
+
+
+def test_superopt_upgrades_sm_to_tma():        # reference tests/test_superopt.py:813-851
+    """The executor upgrades of the reference's superoptimisation pass: no cuda_sm data executor is
+    left, the document keeps its fields, and the result is the document the tma template gives."""
+    from pccl_amd.dsl import Compiler
+    world, n = 4, 4096
+    for r in range(world):
+        sm = RingAllreduce().build_allreduce(r, world, n, dtype="bfloat16", executor="sm", num_channels=2)
+        tma = RingAllreduce().build_allreduce(r, world, n, dtype="bfloat16", executor="tma", num_channels=2)
+        doc = Compiler(enable_superopt=True, topology=None).compile_to_dict(sm)
+        assert doc["version"] == 2 and doc["operations"]
+        data = {op["executor"] for op in doc["operations"] if op["primitive"] not in ("notify", "wait_notify", "noop")}
+        assert data == {"cuda_tma"}
+        required = {"index", "executor", "primitive", "channel", "dependencies", "next_ops", "params"}
+        assert all(required <= set(op) for op in doc["operations"])
+        assert doc == Compiler().compile_to_dict(tma)
+    plain = Compiler().compile_to_dict(RingAllreduce().build_allreduce(0, world, n, dtype="bfloat16", executor="sm"))
+    assert {op["executor"] for op in plain["operations"]} == {"cuda_sm"}
