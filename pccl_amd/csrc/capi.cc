@@ -435,6 +435,56 @@ OpEntry& find_entry(pccl_hip_ctx* ctx, const char* name) {
     return it->second;
 }
 
+// The level runner: one launch per dependency level, or - option level_graph - the launches of an
+// execution replayed as one HIP graph.  The graph holds only kernel nodes (no memset nodes), is
+// captured on a private stream and is bound to one set of rank pointers (kernel arguments are
+// frozen at capture time); a handful are kept per operation, the least recently used is dropped.
+int launch_levels(pccl_hip_ctx* ctx, OpEntry& e, const StepwiseLaunch& L, const RankPtrs& ptrs, char* const* rank_bufs,
+                  hipStream_t stream) {
+    const size_t nlevels = e.level_item_begin.size() - 1;
+    auto launch_all = [&](hipStream_t s) {
+        int rc = 0;
+        for (size_t l = 0; l < nlevels && rc == 0; ++l)
+            rc = launch_level(L, e.level_item_begin[l], e.level_item_begin[l + 1], ptrs, s);
+        return rc;
+    };
+    if (!ctx->level_graph || e.graph_failed || nlevels < 2) return launch_all(stream);
+
+    std::vector<char*> key(rank_bufs, rank_bufs + ctx->R);
+    OpEntry::LevelGraph* hit = nullptr;
+    for (auto& g : e.level_graphs) if (g.key == key) hit = &g;
+    if (!hit) {
+        if (!ctx->capture_stream) HIP_TRY(hipStreamCreateWithFlags(&ctx->capture_stream, hipStreamNonBlocking));
+        OpEntry::LevelGraph g;
+        g.key = key;
+        hipError_t st = hipStreamBeginCapture(ctx->capture_stream, hipStreamCaptureModeThreadLocal);
+        if (st == hipSuccess) {
+            const int lrc = launch_all(ctx->capture_stream);
+            st = hipStreamEndCapture(ctx->capture_stream, &g.graph);
+            if (st == hipSuccess && lrc != 0) st = (hipError_t)lrc;
+        }
+        if (st == hipSuccess) st = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
+        if (st != hipSuccess) {   // capture does not work here: launch level by level from now on
+            if (g.exec) (void)hipGraphExecDestroy(g.exec);
+            if (g.graph) (void)hipGraphDestroy(g.graph);
+            (void)hipGetLastError();
+            e.graph_failed = true;
+            return launch_all(stream);
+        }
+        if (e.level_graphs.size() >= 4) {
+            size_t old = 0;
+            for (size_t i = 1; i < e.level_graphs.size(); ++i) if (e.level_graphs[i].used < e.level_graphs[old].used) old = i;
+            (void)hipGraphExecDestroy(e.level_graphs[old].exec);
+            (void)hipGraphDestroy(e.level_graphs[old].graph);
+            e.level_graphs.erase(e.level_graphs.begin() + old);
+        }
+        e.level_graphs.push_back(g);
+        hit = &e.level_graphs.back();
+    }
+    hit->used = ++e.graph_clock;
+    return (int)hipGraphLaunch(hit->exec, stream);
+}
+
 // Enqueue the program on `stream` over the rank buffers `rank_bufs` (R pointers).
 void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t buf_bytes, hipStream_t stream) {
     const Program& P = e.prog;
@@ -483,53 +533,7 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
             rc = launch_persistent(L, ptrs, stream);   // sizes the grid to what is resident at once
             e.ran_persistent = true;
         } else {
-            rc = 0;
-            const size_t nlevels = e.level_item_begin.size() - 1;
-            bool done = false;
-            if (ctx->level_graph && !e.graph_failed && nlevels >= 2) {
-                // one graph launch instead of one kernel launch per level; the graph holds only
-                // kernel nodes (no memset nodes) and is bound to this set of rank pointers
-                std::vector<char*> key(rank_bufs, rank_bufs + ctx->R);
-                OpEntry::LevelGraph* hit = nullptr;
-                for (auto& g : e.level_graphs) if (g.key == key) hit = &g;
-                if (!hit) {
-                    if (!ctx->capture_stream) HIP_TRY(hipStreamCreateWithFlags(&ctx->capture_stream, hipStreamNonBlocking));
-                    OpEntry::LevelGraph g;
-                    g.key = key;
-                    hipError_t st = hipStreamBeginCapture(ctx->capture_stream, hipStreamCaptureModeThreadLocal);
-                    if (st == hipSuccess) {
-                        int lrc = 0;
-                        for (size_t l = 0; l < nlevels && lrc == 0; ++l)
-                            lrc = launch_level(L, e.level_item_begin[l], e.level_item_begin[l + 1], ptrs, ctx->capture_stream);
-                        st = hipStreamEndCapture(ctx->capture_stream, &g.graph);
-                        if (st == hipSuccess && lrc != 0) st = (hipError_t)lrc;
-                    }
-                    if (st == hipSuccess) st = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
-                    if (st != hipSuccess) {
-                        if (g.exec) (void)hipGraphExecDestroy(g.exec);
-                        if (g.graph) (void)hipGraphDestroy(g.graph);
-                        (void)hipGetLastError();
-                        e.graph_failed = true;
-                    } else {
-                        if (e.level_graphs.size() >= 4) {   // forget the least recently used
-                            size_t old = 0;
-                            for (size_t i = 1; i < e.level_graphs.size(); ++i) if (e.level_graphs[i].used < e.level_graphs[old].used) old = i;
-                            (void)hipGraphExecDestroy(e.level_graphs[old].exec);
-                            (void)hipGraphDestroy(e.level_graphs[old].graph);
-                            e.level_graphs.erase(e.level_graphs.begin() + old);
-                        }
-                        e.level_graphs.push_back(g);
-                        hit = &e.level_graphs.back();
-                    }
-                }
-                if (hit) {
-                    hit->used = ++e.graph_clock;
-                    rc = (int)hipGraphLaunch(hit->exec, stream);
-                    done = true;
-                }
-            }
-            for (size_t l = 0; !done && l < nlevels && rc == 0; ++l)
-                rc = launch_level(L, e.level_item_begin[l], e.level_item_begin[l + 1], ptrs, stream);
+            rc = launch_levels(ctx, e, L, ptrs, rank_bufs, stream);
         }
     }
     if (rc != 0) throw Error{PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)};

@@ -123,201 +123,250 @@ static void count_column_traffic(const Program& P, const ColSegment& seg, int es
             if ((P.col_pre[seg.pre_start + w] >> (8 * j) & 0xFF) != 0xFF) *slot_loads += bytes;
 }
 
-Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOptions& opt) {
-    const int R = (int)graphs.size();
-    if (R <= 0 || R > PCCL_HIP_MAX_VRANKS) throw Error{PCCL_ERR_INVALID, "number of virtual ranks must be 1.." + std::to_string(PCCL_HIP_MAX_VRANKS)};
+// The linker: R per-rank graphs in, one Program out.  Each step is a method; they run in the order
+// `run` calls them and hand their results on through the members.
+namespace {
+
+class Linker {
+  public:
+    Linker(const std::vector<const RankGraph*>& graphs_, const LinkOptions& opt_)
+        : graphs(graphs_), opt(opt_), R((int)graphs_.size()) {}
+
+    Program run() {
+        read_headers();
+        check_ranks();
+        simulate_semaphores();
+        build_reachability();
+        collect_data_ops();
+        check_races();
+        keep_conflict_dependencies();
+        order_ops();
+        plan_steps();
+        plan_gather();
+        plan_column();
+        plan_direct();
+        return std::move(P);
+    }
+
+  private:
+    const std::vector<const RankGraph*>& graphs;
+    const LinkOptions& opt;
+    const int R;
     Program P;
-    P.R = R;
-    bool have_dtype = false;
-    std::vector<int> base(R + 1, 0);
-    for (int r = 0; r < R; ++r) {
-        if (!graphs[r]) throw Error{PCCL_ERR_LINK, "virtual rank " + std::to_string(r) + " has no registered graph"};
-        const RankGraph& g = *graphs[r];
-        base[r + 1] = base[r] + (int)g.ops.size();
-        if (g.has_dtype) {
-            if (have_dtype && g.dtype != P.dtype) throw Error{PCCL_ERR_LINK, "ranks disagree on tensor_info.dtype"};
-            P.dtype = g.dtype; have_dtype = true;
+    std::vector<int> base;          // node id of rank r's op i = base[r] + i
+    int N = 0;                      // ops of all ranks, signals included
+    int es = 0;                     // element size in bytes
+    std::vector<Node> nodes;        // happens-before graph over all ops
+    std::vector<int> exec_order;    // one execution order the semaphores allow (a topological order)
+    std::map<std::pair<int, int>, std::vector<int>> notify_seq, wait_seq;   // per (rank, signal id), for the ambiguity check
+    bool closure = false;           // reach[] is available (the graph is small enough for N^2 bits)
+    std::vector<Bitset> reach;      // reach[v] = nodes that happen before v
+    std::vector<int> data_of;       // node id -> provisional data-op index (-1: a signal or noop)
+    std::vector<int> data_nodes;    // provisional data-op index -> node id
+    int D = 0;                      // number of data ops
+    std::vector<LinkedOp> ops;      // data ops in execution order, before the final sort
+    std::vector<std::vector<ColInstr>> raw_progs;   // column plan: per segment, before finish_column_program
+
+
+    void read_headers() {
+        if (R <= 0 || R > PCCL_HIP_MAX_VRANKS) throw Error{PCCL_ERR_INVALID, "number of virtual ranks must be 1.." + std::to_string(PCCL_HIP_MAX_VRANKS)};
+        P.R = R;
+        bool have_dtype = false;
+        base.assign(R + 1, 0);
+        for (int r = 0; r < R; ++r) {
+            if (!graphs[r]) throw Error{PCCL_ERR_LINK, "virtual rank " + std::to_string(r) + " has no registered graph"};
+            const RankGraph& g = *graphs[r];
+            base[r + 1] = base[r] + (int)g.ops.size();
+            if (g.has_dtype) {
+                if (have_dtype && g.dtype != P.dtype) throw Error{PCCL_ERR_LINK, "ranks disagree on tensor_info.dtype"};
+                P.dtype = g.dtype; have_dtype = true;
+            }
+            if (r == 0) { P.collective_type = g.collective_type; P.tensor_elems = g.tensor_elems; }
+            else if (g.collective_type != P.collective_type) throw Error{PCCL_ERR_LINK, "ranks disagree on collective_type"};
+            P.buffer_elems = std::max(P.buffer_elems, g.max_extent());
+            P.tensor_elems = std::max(P.tensor_elems, g.tensor_elems);
         }
-        if (r == 0) { P.collective_type = g.collective_type; P.tensor_elems = g.tensor_elems; }
-        else if (g.collective_type != P.collective_type) throw Error{PCCL_ERR_LINK, "ranks disagree on collective_type"};
-        P.buffer_elems = std::max(P.buffer_elems, g.max_extent());
-        P.tensor_elems = std::max(P.tensor_elems, g.tensor_elems);
+        N = base[R];
+        P.num_all_ops = N;
+        es = elem_size(P.dtype);
     }
-    const int N = base[R];
-    P.num_all_ops = N;
-    const int es = elem_size(P.dtype);
 
-    // ---- static checks on ranks
-    for (int r = 0; r < R; ++r)
-        for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
-            const GraphOp& o = graphs[r]->ops[i];
-            bool uses_peer = o.kind == OpKind::Reduce || o.kind == OpKind::Copy || o.kind == OpKind::Notify;
-            if (uses_peer && (o.peer < 0 || o.peer >= R))
-                throw Error{PCCL_ERR_LINK, op_name(*graphs[r], r, (int)i) + " names rank " + std::to_string(o.peer) + " but only " + std::to_string(R) + " virtual ranks exist"};
-        }
-
-    // ---- simulate the semaphores (same discipline as the reference's dependency-counter runner:
-    //      per rank and channel a FIFO of ready ops, one at a time; a wait blocks its channel)
-    std::vector<Node> nodes(N);
-    for (int r = 0; r < R; ++r)
-        for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
-            Node& n = nodes[base[r] + i];
-            n.rank = r; n.pos = (int)i;
-            for (int d : graphs[r]->ops[i].deps) n.preds.push_back(base[r] + d);
-        }
-    std::vector<int> remaining(N);
-    std::vector<std::deque<int>> queues((size_t)R * PCCL_HIP_MAX_CHANNELS);
-    for (int r = 0; r < R; ++r)
-        for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
-            remaining[base[r] + i] = graphs[r]->ops[i].num_deps_declared;
-            if (remaining[base[r] + i] == 0) queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + graphs[r]->ops[i].channel].push_back((int)i);
-        }
-    // per (target rank, id): notify nodes not yet consumed, in arrival order
-    std::map<std::pair<int, int>, std::deque<int>> pending;
-    std::map<std::pair<int, int>, std::vector<int>> notify_seq, wait_seq;  // for the ambiguity check
-    std::vector<int> exec_order;
-    exec_order.reserve(N);
-    int done = 0;
-    while (done < N) {
-        bool progressed = false;
+    void check_ranks() {
         for (int r = 0; r < R; ++r)
-            for (int c = 0; c < PCCL_HIP_MAX_CHANNELS; ++c) {
-                auto& q = queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + c];
-                while (!q.empty()) {
-                    int i = q.front();
-                    const GraphOp& o = graphs[r]->ops[i];
-                    int id = base[r] + i;
-                    if (o.kind == OpKind::Wait) {
-                        auto key = std::make_pair(r, (int)o.off0);
-                        auto it = pending.find(key);
-                        if (it == pending.end() || it->second.empty()) break;  // blocked
-                        nodes[id].preds.push_back(it->second.front());
-                        it->second.pop_front();
-                        wait_seq[key].push_back(id);
-                    } else if (o.kind == OpKind::Notify) {
-                        auto key = std::make_pair(o.peer, (int)o.off0);
-                        pending[key].push_back(id);
-                        notify_seq[key].push_back(id);
-                    }
-                    q.pop_front();
-                    exec_order.push_back(id);
-                    ++done; progressed = true;
-                    for (int nx : o.nexts)
-                        if (--remaining[base[r] + nx] == 0)
-                            queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + graphs[r]->ops[nx].channel].push_back(nx);
-                }
+            for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
+                const GraphOp& o = graphs[r]->ops[i];
+                bool uses_peer = o.kind == OpKind::Reduce || o.kind == OpKind::Copy || o.kind == OpKind::Notify;
+                if (uses_peer && (o.peer < 0 || o.peer >= R))
+                    throw Error{PCCL_ERR_LINK, op_name(*graphs[r], r, (int)i) + " names rank " + std::to_string(o.peer) + " but only " + std::to_string(R) + " virtual ranks exist"};
             }
-        if (!progressed) {
-            std::string blocked;
-            int shown = 0;
-            for (int r = 0; r < R && shown < 4; ++r)
-                for (int c = 0; c < PCCL_HIP_MAX_CHANNELS && shown < 4; ++c) {
+    }
+
+    // Simulate the semaphores with the discipline of the reference's dependency-counter runner: per
+    // rank and channel a FIFO of ready ops, one at a time; a wait blocks its channel.
+    void simulate_semaphores() {
+        nodes.assign(N, Node{});
+        for (int r = 0; r < R; ++r)
+            for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
+                Node& n = nodes[base[r] + i];
+                n.rank = r; n.pos = (int)i;
+                for (int d : graphs[r]->ops[i].deps) n.preds.push_back(base[r] + d);
+            }
+        std::vector<int> remaining(N);
+        std::vector<std::deque<int>> queues((size_t)R * PCCL_HIP_MAX_CHANNELS);
+        for (int r = 0; r < R; ++r)
+            for (size_t i = 0; i < graphs[r]->ops.size(); ++i) {
+                remaining[base[r] + i] = graphs[r]->ops[i].num_deps_declared;
+                if (remaining[base[r] + i] == 0) queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + graphs[r]->ops[i].channel].push_back((int)i);
+            }
+        // per (target rank, id): notify nodes not yet consumed, in arrival order
+        std::map<std::pair<int, int>, std::deque<int>> pending;
+        exec_order.reserve(N);
+        int done = 0;
+        while (done < N) {
+            bool progressed = false;
+            for (int r = 0; r < R; ++r)
+                for (int c = 0; c < PCCL_HIP_MAX_CHANNELS; ++c) {
                     auto& q = queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + c];
-                    if (!q.empty()) { blocked += (shown ? "; " : "") + op_name(*graphs[r], r, q.front()) + " waits on signal " + std::to_string(graphs[r]->ops[q.front()].off0); ++shown; }
+                    while (!q.empty()) {
+                        int i = q.front();
+                        const GraphOp& o = graphs[r]->ops[i];
+                        int id = base[r] + i;
+                        if (o.kind == OpKind::Wait) {
+                            auto key = std::make_pair(r, (int)o.off0);
+                            auto it = pending.find(key);
+                            if (it == pending.end() || it->second.empty()) break;  // blocked
+                            nodes[id].preds.push_back(it->second.front());
+                            it->second.pop_front();
+                            wait_seq[key].push_back(id);
+                        } else if (o.kind == OpKind::Notify) {
+                            auto key = std::make_pair(o.peer, (int)o.off0);
+                            pending[key].push_back(id);
+                            notify_seq[key].push_back(id);
+                        }
+                        q.pop_front();
+                        exec_order.push_back(id);
+                        ++done; progressed = true;
+                        for (int nx : o.nexts)
+                            if (--remaining[base[r] + nx] == 0)
+                                queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + graphs[r]->ops[nx].channel].push_back(nx);
+                    }
                 }
-            if (blocked.empty()) blocked = "ops with unmet dependencies (cyclic or dangling dependency lists)";
-            throw Error{PCCL_ERR_LINK, "deadlock: " + std::to_string(done) + " of " + std::to_string(N) + " ops can run; blocked: " + blocked};
-        }
-    }
-    for (auto& kv : pending) if (!kv.second.empty()) P.residual_signals++;
-
-    // ---- reachability (happens-before) over all ops, in execution order (a topological order)
-    const bool closure = (size_t)N <= kClosureLimit;
-    std::vector<Bitset> reach;  // reach[v] = nodes that happen before v
-    if (closure) {
-        reach.assign(N, Bitset(N));
-        for (int id : exec_order)
-            for (int p : nodes[id].preds) { reach[id].or_with(reach[p]); reach[id].set(p); }
-        auto ordered_seq = [&](const std::vector<int>& seq) {
-            for (size_t k = 1; k < seq.size(); ++k)
-                if (!reach[seq[k]].test(seq[k - 1])) return false;
-            return true;
-        };
-        for (auto& kv : notify_seq)
-            if (!ordered_seq(kv.second))
-                throw Error{PCCL_ERR_LINK, "signal " + std::to_string(kv.first.second) + " of rank " + std::to_string(kv.first.first) + " is notified by ops that are not ordered with each other: the pairing of notifies and waits is ambiguous"};
-        for (auto& kv : wait_seq)
-            if (!ordered_seq(kv.second))
-                throw Error{PCCL_ERR_LINK, "signal " + std::to_string(kv.first.second) + " of rank " + std::to_string(kv.first.first) + " is awaited by ops that are not ordered with each other: the pairing of notifies and waits is ambiguous"};
-    }
-
-    // ---- data ops and their nearest data predecessors
-    std::vector<int> data_of(N, -1);  // node id -> provisional data-op index
-    std::vector<int> data_nodes;
-    for (int id : exec_order) {
-        const GraphOp& o = graphs[nodes[id].rank]->ops[nodes[id].pos];
-        if (o.kind == OpKind::Reduce || o.kind == OpKind::Copy) { data_of[id] = (int)data_nodes.size(); data_nodes.push_back(id); }
-    }
-    const int D = (int)data_nodes.size();
-    // frontier[v] = set of data nodes that are the nearest data ancestors of v (through signals/noops)
-    std::vector<std::vector<int>> frontier(N);
-    for (int id : exec_order) {
-        std::vector<int>& f = frontier[id];
-        for (int p : nodes[id].preds) {
-            if (data_of[p] >= 0) f.push_back(p);
-            else f.insert(f.end(), frontier[p].begin(), frontier[p].end());
-        }
-        std::sort(f.begin(), f.end());
-        f.erase(std::unique(f.begin(), f.end()), f.end());
-        if (closure && f.size() > 1) {  // drop ancestors of other members
-            std::vector<int> keep;
-            for (int a : f) {
-                bool redundant = false;
-                for (int b : f) if (a != b && reach[b].test(a)) { redundant = true; break; }
-                if (!redundant) keep.push_back(a);
+            if (!progressed) {
+                std::string blocked;
+                int shown = 0;
+                for (int r = 0; r < R && shown < 4; ++r)
+                    for (int c = 0; c < PCCL_HIP_MAX_CHANNELS && shown < 4; ++c) {
+                        auto& q = queues[(size_t)r * PCCL_HIP_MAX_CHANNELS + c];
+                        if (!q.empty()) { blocked += (shown ? "; " : "") + op_name(*graphs[r], r, q.front()) + " waits on signal " + std::to_string(graphs[r]->ops[q.front()].off0); ++shown; }
+                    }
+                if (blocked.empty()) blocked = "ops with unmet dependencies (cyclic or dangling dependency lists)";
+                throw Error{PCCL_ERR_LINK, "deadlock: " + std::to_string(done) + " of " + std::to_string(N) + " ops can run; blocked: " + blocked};
             }
-            f.swap(keep);
         }
+        for (auto& kv : pending) if (!kv.second.empty()) P.residual_signals++;
     }
-    std::vector<LinkedOp> ops(D);
-    for (int k = 0; k < D; ++k) {
-        int id = data_nodes[k];
-        const GraphOp& o = graphs[nodes[id].rank]->ops[nodes[id].pos];
-        LinkedOp& L = ops[k];
-        L.rank = nodes[id].rank; L.channel = o.channel; L.graph_pos = nodes[id].pos; L.index = o.index;
-        L.is_reduce = o.kind == OpKind::Reduce; L.redop = o.redop; L.peer = o.peer;
-        L.off0 = o.off0; L.off1 = o.off1; L.off2 = o.off2; L.size = o.size;
-        for (int p : frontier[id]) L.deps.push_back(data_of[p]);
-        int lvl = 0;
-        for (int d : L.deps) lvl = std::max(lvl, ops[d].level + 1);
-        L.level = lvl;
-        P.num_levels = std::max(P.num_levels, lvl + 1);
-        P.algorithmic_bytes += (L.is_reduce ? 3 : 2) * L.size * es;
-        // an op whose own source and destination ranges overlap without coinciding has no
-        // defined element order
-        auto partial = [&](int64_t s, int64_t d) { return s != d && s < d + L.size && d < s + L.size; };
-        if (L.size > 0) {
-            if (L.is_reduce && partial(L.off1, L.off2)) throw Error{PCCL_ERR_LINK, op_name(*graphs[L.rank], L.rank, L.graph_pos) + ": src and dst ranges overlap without coinciding"};
-            if (L.peer == L.rank && partial(L.off0, L.dst_off())) throw Error{PCCL_ERR_LINK, op_name(*graphs[L.rank], L.rank, L.graph_pos) + ": reads and writes overlapping ranges of its own buffer"};
+
+    // Reachability (happens-before) over all ops, in execution order.
+    void build_reachability() {
+        closure = (size_t)N <= kClosureLimit;
+        if (closure) {
+            reach.assign(N, Bitset(N));
+            for (int id : exec_order)
+                for (int p : nodes[id].preds) { reach[id].or_with(reach[p]); reach[id].set(p); }
+            auto ordered_seq = [&](const std::vector<int>& seq) {
+                for (size_t k = 1; k < seq.size(); ++k)
+                    if (!reach[seq[k]].test(seq[k - 1])) return false;
+                return true;
+            };
+            for (auto& kv : notify_seq)
+                if (!ordered_seq(kv.second))
+                    throw Error{PCCL_ERR_LINK, "signal " + std::to_string(kv.first.second) + " of rank " + std::to_string(kv.first.first) + " is notified by ops that are not ordered with each other: the pairing of notifies and waits is ambiguous"};
+            for (auto& kv : wait_seq)
+                if (!ordered_seq(kv.second))
+                    throw Error{PCCL_ERR_LINK, "signal " + std::to_string(kv.first.second) + " of rank " + std::to_string(kv.first.first) + " is awaited by ops that are not ordered with each other: the pairing of notifies and waits is ambiguous"};
         }
     }
 
-    // ---- race check: conflicting accesses to one rank buffer must be ordered
-    if (opt.check_races && closure && D > 1) {
-        struct Acc { int rank; int64_t s, e; bool write; int op; };
-        std::vector<Acc> acc;
+    // The data ops and their nearest data predecessors (signals and noops contracted).
+    void collect_data_ops() {
+        data_of.assign(N, -1);
+        for (int id : exec_order) {
+            const GraphOp& o = graphs[nodes[id].rank]->ops[nodes[id].pos];
+            if (o.kind == OpKind::Reduce || o.kind == OpKind::Copy) { data_of[id] = (int)data_nodes.size(); data_nodes.push_back(id); }
+        }
+        D = (int)data_nodes.size();
+        // frontier[v] = set of data nodes that are the nearest data ancestors of v (through signals/noops)
+        std::vector<std::vector<int>> frontier(N);
+        for (int id : exec_order) {
+            std::vector<int>& f = frontier[id];
+            for (int p : nodes[id].preds) {
+                if (data_of[p] >= 0) f.push_back(p);
+                else f.insert(f.end(), frontier[p].begin(), frontier[p].end());
+            }
+            std::sort(f.begin(), f.end());
+            f.erase(std::unique(f.begin(), f.end()), f.end());
+            if (closure && f.size() > 1) {  // drop ancestors of other members
+                std::vector<int> keep;
+                for (int a : f) {
+                    bool redundant = false;
+                    for (int b : f) if (a != b && reach[b].test(a)) { redundant = true; break; }
+                    if (!redundant) keep.push_back(a);
+                }
+                f.swap(keep);
+            }
+        }
+        ops.assign(D, LinkedOp{});
         for (int k = 0; k < D; ++k) {
-            const LinkedOp& L = ops[k];
-            if (L.size <= 0) continue;
-            acc.push_back({L.peer, L.off0, L.off0 + L.size, false, k});
-            if (L.is_reduce) acc.push_back({L.rank, L.off1, L.off1 + L.size, false, k});
-            acc.push_back({L.rank, L.dst_off(), L.dst_off() + L.size, true, k});
-        }
-        std::sort(acc.begin(), acc.end(), [](const Acc& a, const Acc& b) { return a.rank != b.rank ? a.rank < b.rank : a.s < b.s; });
-        size_t pairs = 0;
-        bool complete = true;
-        for (size_t i = 0; i < acc.size() && complete; ++i)
-            for (size_t j = i + 1; j < acc.size() && acc[j].rank == acc[i].rank && acc[j].s < acc[i].e; ++j) {
-                if (++pairs > kPairLimit) { complete = false; break; }
-                if (!(acc[i].write || acc[j].write) || acc[i].op == acc[j].op) continue;
-                int a = data_nodes[acc[i].op], b = data_nodes[acc[j].op];
-                if (!reach[a].test(b) && !reach[b].test(a)) {
-                    const LinkedOp &A = ops[acc[i].op], &B = ops[acc[j].op];
-                    throw Error{PCCL_ERR_LINK, "data race on rank " + std::to_string(acc[i].rank) + " elements [" + std::to_string(std::max(acc[i].s, acc[j].s)) + ", " + std::to_string(std::min(acc[i].e, acc[j].e)) + "): " +
-                                                   op_name(*graphs[A.rank], A.rank, A.graph_pos) + " and " + op_name(*graphs[B.rank], B.rank, B.graph_pos) + " are not ordered by any notify/wait chain"};
-                }
+            int id = data_nodes[k];
+            const GraphOp& o = graphs[nodes[id].rank]->ops[nodes[id].pos];
+            LinkedOp& L = ops[k];
+            L.rank = nodes[id].rank; L.channel = o.channel; L.graph_pos = nodes[id].pos; L.index = o.index;
+            L.is_reduce = o.kind == OpKind::Reduce; L.redop = o.redop; L.peer = o.peer;
+            L.off0 = o.off0; L.off1 = o.off1; L.off2 = o.off2; L.size = o.size;
+            for (int p : frontier[id]) L.deps.push_back(data_of[p]);
+            int lvl = 0;
+            for (int d : L.deps) lvl = std::max(lvl, ops[d].level + 1);
+            L.level = lvl;
+            P.num_levels = std::max(P.num_levels, lvl + 1);
+            P.algorithmic_bytes += (L.is_reduce ? 3 : 2) * L.size * es;
+            // an op whose own source and destination ranges overlap without coinciding has no
+            // defined element order
+            auto partial = [&](int64_t s, int64_t d) { return s != d && s < d + L.size && d < s + L.size; };
+            if (L.size > 0) {
+                if (L.is_reduce && partial(L.off1, L.off2)) throw Error{PCCL_ERR_LINK, op_name(*graphs[L.rank], L.rank, L.graph_pos) + ": src and dst ranges overlap without coinciding"};
+                if (L.peer == L.rank && partial(L.off0, L.dst_off())) throw Error{PCCL_ERR_LINK, op_name(*graphs[L.rank], L.rank, L.graph_pos) + ": reads and writes overlapping ranges of its own buffer"};
             }
-        P.race_checked = complete;
+        }
+    }
+
+    // Conflicting accesses to one rank buffer must be ordered by some notify / wait chain.
+    void check_races() {
+        if (opt.check_races && closure && D > 1) {
+            struct Acc { int rank; int64_t s, e; bool write; int op; };
+            std::vector<Acc> acc;
+            for (int k = 0; k < D; ++k) {
+                const LinkedOp& L = ops[k];
+                if (L.size <= 0) continue;
+                acc.push_back({L.peer, L.off0, L.off0 + L.size, false, k});
+                if (L.is_reduce) acc.push_back({L.rank, L.off1, L.off1 + L.size, false, k});
+                acc.push_back({L.rank, L.dst_off(), L.dst_off() + L.size, true, k});
+            }
+            std::sort(acc.begin(), acc.end(), [](const Acc& a, const Acc& b) { return a.rank != b.rank ? a.rank < b.rank : a.s < b.s; });
+            size_t pairs = 0;
+            bool complete = true;
+            for (size_t i = 0; i < acc.size() && complete; ++i)
+                for (size_t j = i + 1; j < acc.size() && acc[j].rank == acc[i].rank && acc[j].s < acc[i].e; ++j) {
+                    if (++pairs > kPairLimit) { complete = false; break; }
+                    if (!(acc[i].write || acc[j].write) || acc[i].op == acc[j].op) continue;
+                    int a = data_nodes[acc[i].op], b = data_nodes[acc[j].op];
+                    if (!reach[a].test(b) && !reach[b].test(a)) {
+                        const LinkedOp &A = ops[acc[i].op], &B = ops[acc[j].op];
+                        throw Error{PCCL_ERR_LINK, "data race on rank " + std::to_string(acc[i].rank) + " elements [" + std::to_string(std::max(acc[i].s, acc[j].s)) + ", " + std::to_string(std::min(acc[i].e, acc[j].e)) + "): " +
+                                                       op_name(*graphs[A.rank], A.rank, A.graph_pos) + " and " + op_name(*graphs[B.rank], B.rank, B.graph_pos) + " are not ordered by any notify/wait chain"};
+                    }
+                }
+            P.race_checked = complete;
+        }
     }
 
     // ---- keep only the orderings that matter: B must follow A exactly when A happens before B
@@ -325,86 +374,92 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
     //      disjoint ranges (e.g. the ragged pieces of one schedule step) is not a dependency, so
     //      such ops share a level and run in one launch.  Any execution that respects these edges
     //      gives the results of every order the notify/wait chains allow.
-    if (opt.conflict_deps && closure && D > 1 && D <= 8192) {
-        auto overlaps = [](int64_t s0, int64_t n0, int64_t s1, int64_t n1) { return s0 < s1 + n1 && s1 < s0 + n0; };
-        auto conflict = [&](const LinkedOp& A, const LinkedOp& B) {
-            if (A.size <= 0 || B.size <= 0) return false;
-            // writes of A against every access of B, and writes of B against reads of A
-            if (A.rank == B.rank && overlaps(A.dst_off(), A.size, B.dst_off(), B.size)) return true;
-            if (A.rank == B.peer && overlaps(A.dst_off(), A.size, B.off0, B.size)) return true;
-            if (B.is_reduce && A.rank == B.rank && overlaps(A.dst_off(), A.size, B.off1, B.size)) return true;
-            if (B.rank == A.peer && overlaps(B.dst_off(), B.size, A.off0, A.size)) return true;
-            if (A.is_reduce && A.rank == B.rank && overlaps(B.dst_off(), B.size, A.off1, A.size)) return true;
-            return false;
-        };
-        std::vector<Bitset> kept(D, Bitset(D));   // data ops ordered before k through kept edges
-        P.num_levels = 0;
-        for (int k = 0; k < D; ++k) {             // ops[] is in execution (topological) order
-            LinkedOp& B = ops[k];
-            B.deps.clear();
-            for (int a = k - 1; a >= 0; --a) {    // latest first, so covered ancestors are skipped
-                if (kept[k].test(a)) continue;
-                if (!reach[data_nodes[k]].test(data_nodes[a]) || !conflict(ops[a], B)) continue;
-                B.deps.push_back(a);
-                kept[k].or_with(kept[a]);
-                kept[k].set(a);
+    void keep_conflict_dependencies() {
+        if (opt.conflict_deps && closure && D > 1 && D <= 8192) {
+            auto overlaps = [](int64_t s0, int64_t n0, int64_t s1, int64_t n1) { return s0 < s1 + n1 && s1 < s0 + n0; };
+            auto conflict = [&](const LinkedOp& A, const LinkedOp& B) {
+                if (A.size <= 0 || B.size <= 0) return false;
+                // writes of A against every access of B, and writes of B against reads of A
+                if (A.rank == B.rank && overlaps(A.dst_off(), A.size, B.dst_off(), B.size)) return true;
+                if (A.rank == B.peer && overlaps(A.dst_off(), A.size, B.off0, B.size)) return true;
+                if (B.is_reduce && A.rank == B.rank && overlaps(A.dst_off(), A.size, B.off1, B.size)) return true;
+                if (B.rank == A.peer && overlaps(B.dst_off(), B.size, A.off0, A.size)) return true;
+                if (A.is_reduce && A.rank == B.rank && overlaps(B.dst_off(), B.size, A.off1, A.size)) return true;
+                return false;
+            };
+            std::vector<Bitset> kept(D, Bitset(D));   // data ops ordered before k through kept edges
+            P.num_levels = 0;
+            for (int k = 0; k < D; ++k) {             // ops[] is in execution (topological) order
+                LinkedOp& B = ops[k];
+                B.deps.clear();
+                for (int a = k - 1; a >= 0; --a) {    // latest first, so covered ancestors are skipped
+                    if (kept[k].test(a)) continue;
+                    if (!reach[data_nodes[k]].test(data_nodes[a]) || !conflict(ops[a], B)) continue;
+                    B.deps.push_back(a);
+                    kept[k].or_with(kept[a]);
+                    kept[k].set(a);
+                }
+                int lvl = 0;
+                for (int d : B.deps) lvl = std::max(lvl, ops[d].level + 1);
+                B.level = lvl;
+                P.num_levels = std::max(P.num_levels, lvl + 1);
             }
-            int lvl = 0;
-            for (int d : B.deps) lvl = std::max(lvl, ops[d].level + 1);
-            B.level = lvl;
-            P.num_levels = std::max(P.num_levels, lvl + 1);
         }
     }
 
-    // ---- final order: (level, rank, channel, graph position); remap deps
-    std::vector<int> perm(D);
-    std::iota(perm.begin(), perm.end(), 0);
-    std::stable_sort(perm.begin(), perm.end(), [&](int a, int b) {
-        const LinkedOp &A = ops[a], &B = ops[b];
-        if (A.level != B.level) return A.level < B.level;
-        if (A.rank != B.rank) return A.rank < B.rank;
-        if (A.channel != B.channel) return A.channel < B.channel;
-        return A.graph_pos < B.graph_pos;
-    });
-    std::vector<int> inv(D);
-    for (int k = 0; k < D; ++k) inv[perm[k]] = k;
-    P.ops.resize(D);
-    for (int k = 0; k < D; ++k) {
-        P.ops[k] = ops[perm[k]];
-        for (int& d : P.ops[k].deps) d = inv[d];
-        std::sort(P.ops[k].deps.begin(), P.ops[k].deps.end());
+    // Final order: (level, rank, channel, graph position); dependencies renumbered to it.
+    void order_ops() {
+        std::vector<int> perm(D);
+        std::iota(perm.begin(), perm.end(), 0);
+        std::stable_sort(perm.begin(), perm.end(), [&](int a, int b) {
+            const LinkedOp &A = ops[a], &B = ops[b];
+            if (A.level != B.level) return A.level < B.level;
+            if (A.rank != B.rank) return A.rank < B.rank;
+            if (A.channel != B.channel) return A.channel < B.channel;
+            return A.graph_pos < B.graph_pos;
+        });
+        std::vector<int> inv(D);
+        for (int k = 0; k < D; ++k) inv[perm[k]] = k;
+        P.ops.resize(D);
+        for (int k = 0; k < D; ++k) {
+            P.ops[k] = ops[perm[k]];
+            for (int& d : P.ops[k].deps) d = inv[d];
+            std::sort(P.ops[k].deps.begin(), P.ops[k].deps.end());
+        }
     }
 
-    // ---- stepwise plan
-    int64_t tile_bytes = opt.step_tile_bytes;
-    if (tile_bytes <= 0) {
-        // automatic: 32 KiB items (the fastest on large programs), halved down to 4 KiB while an
-        // average level has fewer than 1024 items - a small program is bound by the latency of its
-        // chain of levels, and needs its few bytes spread over many workgroups
-        int64_t bytes = 0;
-        for (const LinkedOp& L : P.ops) bytes += L.size * es;
-        const int64_t per_level = bytes / std::max(1, P.num_levels);
-        tile_bytes = 32 * 1024;
-        while (tile_bytes > 4096 && per_level / tile_bytes < 1024) tile_bytes >>= 1;
+    // The stepwise plan: every op cut into work items.
+    void plan_steps() {
+        int64_t tile_bytes = opt.step_tile_bytes;
+        if (tile_bytes <= 0) {
+            // automatic: 32 KiB items (the fastest on large programs), halved down to 4 KiB while an
+            // average level has fewer than 1024 items - a small program is bound by the latency of its
+            // chain of levels, and needs its few bytes spread over many workgroups
+            int64_t bytes = 0;
+            for (const LinkedOp& L : P.ops) bytes += L.size * es;
+            const int64_t per_level = bytes / std::max(1, P.num_levels);
+            tile_bytes = 32 * 1024;
+            while (tile_bytes > 4096 && per_level / tile_bytes < 1024) tile_bytes >>= 1;
+        }
+        P.tile_elems = std::max<int64_t>(tile_bytes / es, 1024);
+        P.step_ops.resize(D);
+        int64_t items = 0;
+        for (int k = 0; k < D; ++k) {
+            StepOpPlan& s = P.step_ops[k];
+            s.first_item = (int)items;
+            // the item grid is anchored at a multiple of the tile size in the destination buffer, so
+            // that an op with an odd start still has whole, aligned items everywhere but at its ends
+            const int64_t dst = P.ops[k].is_reduce ? P.ops[k].off2 : P.ops[k].off1;
+            s.lead = (int)(dst % P.tile_elems);
+            s.ntiles = (int)((P.ops[k].size + s.lead + P.tile_elems - 1) / P.tile_elems);
+            s.dep_start = (int)P.step_deps.size();
+            s.ndeps = (int)P.ops[k].deps.size();
+            for (int d : P.ops[k].deps) P.step_deps.push_back(d);
+            items += s.ntiles;
+            if (items > INT32_MAX) throw Error{PCCL_ERR_UNSUPPORTED, "program has more than 2^31 work items"};
+        }
+        P.num_items = items;
     }
-    P.tile_elems = std::max<int64_t>(tile_bytes / es, 1024);
-    P.step_ops.resize(D);
-    int64_t items = 0;
-    for (int k = 0; k < D; ++k) {
-        StepOpPlan& s = P.step_ops[k];
-        s.first_item = (int)items;
-        // the item grid is anchored at a multiple of the tile size in the destination buffer, so
-        // that an op with an odd start still has whole, aligned items everywhere but at its ends
-        const int64_t dst = P.ops[k].is_reduce ? P.ops[k].off2 : P.ops[k].off1;
-        s.lead = (int)(dst % P.tile_elems);
-        s.ntiles = (int)((P.ops[k].size + s.lead + P.tile_elems - 1) / P.tile_elems);
-        s.dep_start = (int)P.step_deps.size();
-        s.ndeps = (int)P.ops[k].deps.size();
-        for (int d : P.ops[k].deps) P.step_deps.push_back(d);
-        items += s.ntiles;
-        if (items > INT32_MAX) throw Error{PCCL_ERR_UNSUPPORTED, "program has more than 2^31 work items"};
-    }
-    P.num_items = items;
 
     // ---- gather plan: an alltoall graph whose ops are all copies out of regions nobody writes.
     // Staged semantics (reference engine_c.cc:524-543): input r sits at [0, n) of buffer r, the
@@ -413,134 +468,148 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
     // every output element, the input element it comes from - no buffer needed.  Abandoned (the
     // call then stages through the rank buffers) if any output element would come from scratch the
     // program never wrote, or if an op writes something another op reads or writes.
-    if (P.collective_type == "alltoall" && D > 0 && P.tensor_elems > 0 && P.tensor_elems % R == 0) {
-        const int64_t n = P.tensor_elems, chunk = n / R;
-        bool ok = true;
-        for (const LinkedOp& L : P.ops) if (L.is_reduce) ok = false;
-        // sources inside the input region, destinations outside it and mutually disjoint per rank
-        std::vector<std::vector<std::pair<int64_t, int>>> writes(R);   // (dst offset, op) per rank
-        for (int k = 0; k < D && ok; ++k) {
-            const LinkedOp& L = P.ops[k];
-            if (L.size <= 0) continue;
-            if (L.off0 < 0 || L.off0 + L.size > n || L.off1 < n) ok = false;
-            writes[L.rank].push_back({L.off1, k});
-        }
-        for (int r = 0; r < R && ok; ++r) {
-            std::sort(writes[r].begin(), writes[r].end());
-            for (size_t i = 1; i < writes[r].size(); ++i) {
-                const LinkedOp& prev = P.ops[writes[r][i - 1].second];
-                if (prev.off1 + prev.size > writes[r][i].first) ok = false;
+    void plan_gather() {
+        if (P.collective_type == "alltoall" && D > 0 && P.tensor_elems > 0 && P.tensor_elems % R == 0) {
+            const int64_t n = P.tensor_elems, chunk = n / R;
+            bool ok = true;
+            for (const LinkedOp& L : P.ops) if (L.is_reduce) ok = false;
+            // sources inside the input region, destinations outside it and mutually disjoint per rank
+            std::vector<std::vector<std::pair<int64_t, int>>> writes(R);   // (dst offset, op) per rank
+            for (int k = 0; k < D && ok; ++k) {
+                const LinkedOp& L = P.ops[k];
+                if (L.size <= 0) continue;
+                if (L.off0 < 0 || L.off0 + L.size > n || L.off1 < n) ok = false;
+                writes[L.rank].push_back({L.off1, k});
             }
-        }
-        for (int r = 0; r < R && ok; ++r)
-            for (int p = 0; p < R && ok; ++p) {
-                if (p == r) { P.gather.push_back({r, r, (int64_t)p * chunk, (int64_t)r * chunk, chunk}); continue; }
-                int64_t x = n + (int64_t)p * chunk;
-                const int64_t x_end = x + chunk;
-                while (x < x_end && ok) {        // walk the scratch chunk through the ops that wrote it
-                    const LinkedOp* hit = nullptr;
-                    for (auto& w : writes[r]) {
-                        const LinkedOp& L = P.ops[w.second];
-                        if (L.off1 <= x && x < L.off1 + L.size) { hit = &L; break; }
-                    }
-                    if (!hit) { ok = false; break; }
-                    const int64_t len = std::min(x_end, hit->off1 + hit->size) - x;
-                    P.gather.push_back({r, hit->peer, (int64_t)p * chunk + (x - (n + (int64_t)p * chunk)), hit->off0 + (x - hit->off1), len});
-                    x += len;
+            for (int r = 0; r < R && ok; ++r) {
+                std::sort(writes[r].begin(), writes[r].end());
+                for (size_t i = 1; i < writes[r].size(); ++i) {
+                    const LinkedOp& prev = P.ops[writes[r][i - 1].second];
+                    if (prev.off1 + prev.size > writes[r][i].first) ok = false;
                 }
             }
-        if (!ok) P.gather.clear();
+            for (int r = 0; r < R && ok; ++r)
+                for (int p = 0; p < R && ok; ++p) {
+                    if (p == r) { P.gather.push_back({r, r, (int64_t)p * chunk, (int64_t)r * chunk, chunk}); continue; }
+                    int64_t x = n + (int64_t)p * chunk;
+                    const int64_t x_end = x + chunk;
+                    while (x < x_end && ok) {        // walk the scratch chunk through the ops that wrote it
+                        const LinkedOp* hit = nullptr;
+                        for (auto& w : writes[r]) {
+                            const LinkedOp& L = P.ops[w.second];
+                            if (L.off1 <= x && x < L.off1 + L.size) { hit = &L; break; }
+                        }
+                        if (!hit) { ok = false; break; }
+                        const int64_t len = std::min(x_end, hit->off1 + hit->size) - x;
+                        P.gather.push_back({r, hit->peer, (int64_t)p * chunk + (x - (n + (int64_t)p * chunk)), hit->off0 + (x - hit->off1), len});
+                        x += len;
+                    }
+                }
+            if (!ok) P.gather.clear();
+        }
     }
 
-    // ---- column plan
-    P.position_aligned = D > 0;
-    for (auto& L : P.ops) if (!L.position_aligned()) { P.position_aligned = false; break; }
-    if (P.position_aligned) {
-        std::vector<int64_t> cuts;
-        for (auto& L : P.ops) if (L.size > 0) { cuts.push_back(L.off0); cuts.push_back(L.off0 + L.size); }
-        std::sort(cuts.begin(), cuts.end());
-        cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
-        // ops covering each elementary interval, in program order
-        std::vector<std::vector<int>> cover(cuts.size() > 0 ? cuts.size() - 1 : 0);
-        for (int k = 0; k < D; ++k) {
-            const LinkedOp& L = P.ops[k];
-            if (L.size <= 0) continue;
-            size_t a = std::lower_bound(cuts.begin(), cuts.end(), L.off0) - cuts.begin();
-            size_t b = std::lower_bound(cuts.begin(), cuts.end(), L.off0 + L.size) - cuts.begin();
-            for (size_t i = a; i < b; ++i) cover[i].push_back(k);
+    // The column program of one segment: the ops covering it in program order, values forwarded
+    // through the accumulator where one op's result is the next one's operand, dead stores dropped,
+    // final stores marked (not yet finished: see finish_column_program).
+    std::vector<ColInstr> segment_program(const std::vector<int>& covering) const {
+        std::vector<ColInstr> prog;
+        uint64_t written = 0;  // ranks an earlier instruction of this program wrote
+        for (size_t n = 0; n < covering.size(); ++n) {
+            const LinkedOp& L = P.ops[covering[n]];
+            ColInstr in{};
+            in.self = (uint8_t)L.rank; in.peer = (uint8_t)L.peer; in.redop = (uint8_t)L.redop; in.store = 1;
+            bool prev_is_peer = n > 0 && prog.back().self == in.peer;
+            bool prev_is_self = n > 0 && prog.back().self == in.self;
+            in.a_src = prev_is_peer ? SRC_ACC : SRC_MEM;
+            in.b_src = !L.is_reduce ? SRC_NONE : prev_is_self ? SRC_ACC : SRC_MEM;
+            if (in.a_src == SRC_MEM) in.a_first = !(written >> in.peer & 1);
+            if (in.b_src == SRC_MEM) in.b_first = !(written >> in.self & 1);
+            written |= 1ull << in.self;
+            prog.push_back(in);
         }
-        // instruction signature of an op list (what the device program depends on)
-        auto sig = [&](const std::vector<int>& v) {
-            std::vector<int> s;
-            for (int k : v) { const LinkedOp& L = P.ops[k]; s.push_back(L.rank | L.peer << 8 | (int)L.is_reduce << 16 | L.redop << 17); }
-            return s;
-        };
-        std::vector<int> prev_sig;
-        std::vector<std::vector<ColInstr>> raw_progs;   // per segment, before finish_column_program
-        for (size_t i = 0; i < cover.size(); ++i) {
-            if (cover[i].empty()) { prev_sig.clear(); continue; }
-            std::vector<int> s = sig(cover[i]);
-            if (!P.segs.empty() && P.segs.back().end == cuts[i] && s == prev_sig) { P.segs.back().end = cuts[i + 1]; continue; }
-            prev_sig = s;
-            ColSegment seg;
-            seg.start = cuts[i]; seg.end = cuts[i + 1];
-            seg.prog_start = (int)P.col_instrs.size();
-            // build + optimise the column program
-            std::vector<ColInstr> prog;
-            uint64_t written = 0;  // ranks an earlier instruction of this program wrote
-            for (size_t n = 0; n < cover[i].size(); ++n) {
-                const LinkedOp& L = P.ops[cover[i][n]];
-                ColInstr in{};
-                in.self = (uint8_t)L.rank; in.peer = (uint8_t)L.peer; in.redop = (uint8_t)L.redop; in.store = 1;
-                bool prev_is_peer = n > 0 && prog.back().self == in.peer;
-                bool prev_is_self = n > 0 && prog.back().self == in.self;
-                in.a_src = prev_is_peer ? SRC_ACC : SRC_MEM;
-                in.b_src = !L.is_reduce ? SRC_NONE : prev_is_self ? SRC_ACC : SRC_MEM;
-                if (in.a_src == SRC_MEM) in.a_first = !(written >> in.peer & 1);
-                if (in.b_src == SRC_MEM) in.b_first = !(written >> in.self & 1);
-                written |= 1ull << in.self;
-                prog.push_back(in);
-            }
-            // dead stores: overwritten before any later instruction reads that rank from memory
-            for (size_t n = 0; n < prog.size(); ++n) {
-                for (size_t m = n + 1; m < prog.size(); ++m) {
-                    bool reads = (prog[m].a_src != SRC_ACC && prog[m].peer == prog[n].self) ||
-                                 (prog[m].b_src == SRC_MEM && prog[m].self == prog[n].self);
-                    if (reads) break;
-                    if (prog[m].self == prog[n].self) { prog[n].store = 0; break; }
-                }
-            }
-            // a store nothing in this program reads back from memory is final: mark it streaming
-            for (size_t n = 0; n < prog.size(); ++n) {
-                if (!prog[n].store) continue;
-                bool reread = false;
-                for (size_t m = n + 1; m < prog.size() && !reread; ++m)
-                    reread = (prog[m].a_src != SRC_ACC && prog[m].peer == prog[n].self) ||
+        // dead stores: overwritten before any later instruction reads that rank from memory
+        for (size_t n = 0; n < prog.size(); ++n) {
+            for (size_t m = n + 1; m < prog.size(); ++m) {
+                bool reads = (prog[m].a_src != SRC_ACC && prog[m].peer == prog[n].self) ||
                              (prog[m].b_src == SRC_MEM && prog[m].self == prog[n].self);
-                if (!reread) prog[n].store = 2;
+                if (reads) break;
+                if (prog[m].self == prog[n].self) { prog[n].store = 0; break; }
             }
-            seg.prog_len = (int)prog.size();
-            raw_progs.push_back(prog);            // the direct plan below starts from the unfinished form
-            finish_column_program(P, seg, prog);
-            P.col_instrs.insert(P.col_instrs.end(), prog.begin(), prog.end());
-            P.segs.push_back(seg);
         }
-        for (auto& seg : P.segs)
-            count_column_traffic(P, seg, es, &P.column_load_bytes, &P.column_store_bytes, &P.slot_load_bytes, &P.slot_store_bytes);
+        // a store nothing in this program reads back from memory is final: mark it streaming
+        for (size_t n = 0; n < prog.size(); ++n) {
+            if (!prog[n].store) continue;
+            bool reread = false;
+            for (size_t m = n + 1; m < prog.size() && !reread; ++m)
+                reread = (prog[m].a_src != SRC_ACC && prog[m].peer == prog[n].self) ||
+                         (prog[m].b_src == SRC_MEM && prog[m].self == prog[n].self);
+            if (!reread) prog[n].store = 2;
+        }
+        return prog;
+    }
 
-        // ---- direct plan: the same programs with the caller's input tensors as the source of
-        // every first-touch load and the output tensors as the destination of every store, so
-        // that no staging copy is needed.  The staged semantics are "place input r in buffer r at
-        // its window, run, hand back the output window of buffer r" (reference engine_c.cc:468-548):
-        //   allreduce / untyped   in [0,n)                out [0,n)
-        //   reduce_scatter        in [0,n)                out [r*n/R, (r+1)*n/R)
-        //   allgather             in [r*n/R, (r+1)*n/R)   out [0,n)
-        // For the result to be identical, a (rank, position) inside the output window that the
-        // program never writes is passed through from the input (one copy instruction with
-        // peer = self), a final store outside the output window is dropped (nobody can observe
-        // it), and the plan is abandoned (staging is used instead) if any access would need
-        // memory outside the windows: a first touch outside the input window, or a value that is
-        // written outside the output window and read back later.
+    // The column plan: when every op reads and writes the same element positions, the program
+    // decomposes by position into segments with one column program each.
+    void plan_column() {
+        P.position_aligned = D > 0;
+        for (auto& L : P.ops) if (!L.position_aligned()) { P.position_aligned = false; break; }
+        if (P.position_aligned) {
+            std::vector<int64_t> cuts;
+            for (auto& L : P.ops) if (L.size > 0) { cuts.push_back(L.off0); cuts.push_back(L.off0 + L.size); }
+            std::sort(cuts.begin(), cuts.end());
+            cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+            // ops covering each elementary interval, in program order
+            std::vector<std::vector<int>> cover(cuts.size() > 0 ? cuts.size() - 1 : 0);
+            for (int k = 0; k < D; ++k) {
+                const LinkedOp& L = P.ops[k];
+                if (L.size <= 0) continue;
+                size_t a = std::lower_bound(cuts.begin(), cuts.end(), L.off0) - cuts.begin();
+                size_t b = std::lower_bound(cuts.begin(), cuts.end(), L.off0 + L.size) - cuts.begin();
+                for (size_t i = a; i < b; ++i) cover[i].push_back(k);
+            }
+            // instruction signature of an op list (what the device program depends on)
+            auto sig = [&](const std::vector<int>& v) {
+                std::vector<int> s;
+                for (int k : v) { const LinkedOp& L = P.ops[k]; s.push_back(L.rank | L.peer << 8 | (int)L.is_reduce << 16 | L.redop << 17); }
+                return s;
+            };
+            std::vector<int> prev_sig;
+            for (size_t i = 0; i < cover.size(); ++i) {
+                if (cover[i].empty()) { prev_sig.clear(); continue; }
+                std::vector<int> s = sig(cover[i]);
+                if (!P.segs.empty() && P.segs.back().end == cuts[i] && s == prev_sig) { P.segs.back().end = cuts[i + 1]; continue; }
+                prev_sig = s;
+                ColSegment seg;
+                seg.start = cuts[i]; seg.end = cuts[i + 1];
+                seg.prog_start = (int)P.col_instrs.size();
+                std::vector<ColInstr> prog = segment_program(cover[i]);
+                seg.prog_len = (int)prog.size();
+                raw_progs.push_back(prog);            // the direct plan below starts from the unfinished form
+                finish_column_program(P, seg, prog);
+                P.col_instrs.insert(P.col_instrs.end(), prog.begin(), prog.end());
+                P.segs.push_back(seg);
+            }
+            for (auto& seg : P.segs)
+                count_column_traffic(P, seg, es, &P.column_load_bytes, &P.column_store_bytes, &P.slot_load_bytes, &P.slot_store_bytes);
+        }
+    }
+
+    // ---- direct plan: the same programs with the caller's input tensors as the source of
+    // every first-touch load and the output tensors as the destination of every store, so
+    // that no staging copy is needed.  The staged semantics are "place input r in buffer r at
+    // its window, run, hand back the output window of buffer r" (reference engine_c.cc:468-548):
+    //   allreduce / untyped   in [0,n)                out [0,n)
+    //   reduce_scatter        in [0,n)                out [r*n/R, (r+1)*n/R)
+    //   allgather             in [r*n/R, (r+1)*n/R)   out [0,n)
+    // For the result to be identical, a (rank, position) inside the output window that the
+    // program never writes is passed through from the input (one copy instruction with
+    // peer = self), a final store outside the output window is dropped (nobody can observe
+    // it), and the plan is abandoned (staging is used instead) if any access would need
+    // memory outside the windows: a first touch outside the input window, or a value that is
+    // written outside the output window and read back later.
+    void plan_direct() {
+        if (!P.position_aligned) return;
         const int64_t n = P.tensor_elems;
         const std::string& ct = P.collective_type;
         const bool ar = ct.empty() || ct == "allreduce";
@@ -566,12 +635,12 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                 const int64_t a = cuts2[i], b = cuts2[i + 1];
                 if (a < 0 || b > n) continue;
                 while (si < base_segs.size() && base_segs[si].end <= a) ++si;
-                const ColSegment* base = (si < base_segs.size() && base_segs[si].start <= a && b <= base_segs[si].end) ? &base_segs[si] : nullptr;
+                const ColSegment* under = (si < base_segs.size() && base_segs[si].start <= a && b <= base_segs[si].end) ? &base_segs[si] : nullptr;
                 auto in_window = [&](int r) { return P.direct_in_start[r] <= a && b <= P.direct_in_end[r]; };
                 auto out_window = [&](int r) { return P.direct_out_start[r] <= a && b <= P.direct_out_end[r]; };
                 std::vector<ColInstr> prog;
                 uint64_t written = 0;
-                if (base)
+                if (under)
                     for (size_t k = 0; k < raw_progs[si].size() && valid; ++k) {
                         ColInstr in = raw_progs[si][k];
                         if (in.a_src == SRC_MEM) valid = in.a_first ? in_window(in.peer) : out_window(in.peer);
@@ -615,7 +684,14 @@ Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOpti
                 count_column_traffic(P, seg, es, &P.direct_load_bytes, &P.direct_store_bytes, &P.direct_slot_load_bytes, &P.direct_slot_store_bytes);
         }
     }
-    return P;
+};
+
+}  // namespace
+
+Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOptions& opt) {
+    if (graphs.empty() || graphs.size() > (size_t)PCCL_HIP_MAX_VRANKS)
+        throw Error{PCCL_ERR_INVALID, "number of virtual ranks must be 1.." + std::to_string(PCCL_HIP_MAX_VRANKS)};
+    return Linker(graphs, opt).run();
 }
 
 }  // namespace pccl_hip
