@@ -584,6 +584,82 @@ bool run_direct(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
     return true;
 }
 
+// An alltoall as direct copies from the input tensors to the output tensors, when the program
+// composes into such copies (the gather plan) and no output overlaps an input or another output.
+bool run_gather(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* const* outputs,
+                size_t in_bytes, size_t out_bytes, hipStream_t s) {
+    const Program& P = e.prog;
+    const int R = ctx->R;
+    const size_t es = elem_size(P.dtype);
+    if (P.collective_type != "alltoall" || !ctx->fuse_staging || !e.gather.p || ctx->mode != Mode::Auto ||
+        in_bytes != (size_t)P.tensor_elems * es || out_bytes < in_bytes)
+        return false;
+    for (int r = 0; r < R; ++r)
+        for (int q = 0; q < R; ++q) {
+            const uintptr_t o = (uintptr_t)outputs[r], i = (uintptr_t)inputs[q];
+            if (o < i + in_bytes && i < o + in_bytes) return false;
+            if (q != r && o < (uintptr_t)outputs[q] + in_bytes && (uintptr_t)outputs[q] < o + in_bytes) return false;
+        }
+    RankPtrs src{}, dst{};
+    for (int r = 0; r < R; ++r) { src.p[r] = (char*)inputs[r]; dst.p[r] = (char*)outputs[r]; }
+    if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, s));
+    int rc = launch_gather((const DevGatherCopy*)e.gather.p, (int)P.gather.size(), e.gather_tiles, e.gather_copy_tiles, src, dst, s);
+    if (rc) throw Error{PCCL_ERR_HIP, std::string("gather launch failed: ") + hipGetErrorString((hipError_t)rc)};
+    if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, s)); e.timed = true; }
+    return true;
+}
+
+// The reference's staging (engine_c.cc:468-548): inputs into the rank buffers, the program, the
+// results out of the rank buffers, laid out per collective type.
+void run_staged(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* const* outputs,
+                size_t in_bytes, size_t out_bytes, hipStream_t s) {
+    const Program& P = e.prog;
+    const int R = ctx->R;
+    const size_t es = elem_size(P.dtype);
+    const std::string& ct = P.collective_type;
+    // the output must hold what the collective hands back; checked before anything is enqueued
+    if (ct == "reduce_scatter" && out_bytes < in_bytes / R) throw Error{PCCL_ERR_INVALID, "reduce_scatter output is smaller than one chunk"};
+    if (ct == "alltoall" && out_bytes < in_bytes / R * R) throw Error{PCCL_ERR_INVALID, "alltoall output is smaller than the input"};
+
+    size_t need = (size_t)P.buffer_elems * es;
+    if (ct == "allgather") need = std::max(need, in_bytes * R);
+    else need = std::max(need, in_bytes);
+    if (ct == "alltoall") need = std::max(need, 2 * in_bytes);
+    else if (ct != "reduce_scatter") need = std::max(need, out_bytes);
+    ensure_buffers(ctx, need);
+
+    RankPtrs src{}, dst{}, bufp{};
+    StageOffsets off{};
+    for (int r = 0; r < R; ++r) {
+        src.p[r] = (char*)inputs[r]; bufp.p[r] = ctx->bufs[r]; dst.p[r] = (char*)outputs[r];
+        off.src[r] = 0;
+        off.dst[r] = ct == "allgather" ? (int64_t)r * (int64_t)in_bytes : 0;
+    }
+    int rc = launch_stage(src, bufp, off, R, in_bytes, s);
+    if (rc) throw Error{PCCL_ERR_HIP, std::string("input staging: ") + hipGetErrorString((hipError_t)rc)};
+
+    run_program(ctx, e, ctx->bufs.data(), ctx->buf_bytes, s);
+
+    const size_t chunk = in_bytes / R;
+    if (ct == "reduce_scatter") {           // chunk r of buffer r
+        for (int r = 0; r < R; ++r) { off.src[r] = (int64_t)r * (int64_t)chunk; off.dst[r] = 0; }
+        rc = launch_stage(bufp, dst, off, R, chunk, s);
+    } else if (ct == "alltoall") {          // own chunk from the input region, the others from the scratch region
+        rc = 0;
+        for (int p = 0; p < R && rc == 0; ++p) {
+            for (int r = 0; r < R; ++r) {
+                off.src[r] = p == r ? (int64_t)r * (int64_t)chunk : (int64_t)in_bytes + (int64_t)p * (int64_t)chunk;
+                off.dst[r] = (int64_t)p * (int64_t)chunk;
+            }
+            rc = launch_stage(bufp, dst, off, R, chunk, s);
+        }
+    } else {                                // allreduce and untyped graphs: the head of the buffer
+        for (int r = 0; r < R; ++r) { off.src[r] = 0; off.dst[r] = 0; }
+        rc = launch_stage(bufp, dst, off, R, out_bytes, s);
+    }
+    if (rc) throw Error{PCCL_ERR_HIP, std::string("output staging: ") + hipGetErrorString((hipError_t)rc)};
+}
+
 // After the stream has drained: did a bounded wait of the persistent runner expire?
 void check_stall(OpEntry& e, const std::string& name) {
     if (!e.ran_persistent || !e.state.p) return;
@@ -725,87 +801,13 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
         link_entry(ctx, e);
-        const Program& P = e.prog;
-        const int R = ctx->R;
-        const size_t es = elem_size(P.dtype);
-        const std::string& ct = P.collective_type;
         hipStream_t s = (hipStream_t)stream;
-        for (int r = 0; r < R; ++r)
+        for (int r = 0; r < ctx->R; ++r)
             if (!inputs[r] || !outputs[r]) return fail(PCCL_ERR_INVALID, "null tensor for virtual rank " + std::to_string(r));
-
-        if (run_direct(ctx, e, inputs, outputs, in_bytes, out_bytes, s)) {
-            ctx->last_stream = s;
-            if (sync) HIP_TRY(hipStreamSynchronize(s));
-            return 0;
-        }
-
-        // alltoall as direct copies from the input tensors to the output tensors, when the program
-        // composes into such copies and no output overlaps an input
-        if (ct == "alltoall" && ctx->fuse_staging && e.gather.p && ctx->mode == Mode::Auto &&
-            in_bytes == (size_t)P.tensor_elems * es && out_bytes >= in_bytes) {
-            bool disjoint = true;
-            for (int r = 0; r < R && disjoint; ++r)
-                for (int q = 0; q < R && disjoint; ++q) {
-                    const uintptr_t o = (uintptr_t)outputs[r], i = (uintptr_t)inputs[q];
-                    if (o < i + in_bytes && i < o + in_bytes) disjoint = false;
-                    if (q != r && o < (uintptr_t)outputs[q] + in_bytes && (uintptr_t)outputs[q] < o + in_bytes) disjoint = false;
-                }
-            if (disjoint) {
-                RankPtrs src{}, dst{};
-                for (int r = 0; r < R; ++r) { src.p[r] = (char*)inputs[r]; dst.p[r] = (char*)outputs[r]; }
-                if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, s));
-                int grc = launch_gather((const DevGatherCopy*)e.gather.p, (int)P.gather.size(), e.gather_tiles, e.gather_copy_tiles, src, dst, s);
-                if (grc) return fail(PCCL_ERR_HIP, std::string("gather launch failed: ") + hipGetErrorString((hipError_t)grc));
-                if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, s)); e.timed = true; }
-                ctx->last_stream = s;
-                if (sync) HIP_TRY(hipStreamSynchronize(s));
-                return 0;
-            }
-        }
-
-        // the output must hold what the collective hands back; checked before anything is enqueued
-        if (ct == "reduce_scatter" && out_bytes < in_bytes / R) return fail(PCCL_ERR_INVALID, "reduce_scatter output is smaller than one chunk");
-        if (ct == "alltoall" && out_bytes < in_bytes / R * R) return fail(PCCL_ERR_INVALID, "alltoall output is smaller than the input");
-
-        // layout of the staged data inside a rank buffer (reference engine_c.cc:468-548)
-        size_t need = (size_t)P.buffer_elems * es;
-        if (ct == "allgather") need = std::max(need, in_bytes * R);
-        else need = std::max(need, in_bytes);
-        if (ct == "alltoall") need = std::max(need, 2 * in_bytes);
-        else if (ct != "reduce_scatter") need = std::max(need, out_bytes);
-        ensure_buffers(ctx, need);
-
-        RankPtrs src{}, dst{}, bufp{};
-        StageOffsets off{};
-        for (int r = 0; r < R; ++r) {
-            src.p[r] = (char*)inputs[r]; bufp.p[r] = ctx->bufs[r]; dst.p[r] = (char*)outputs[r];
-            off.src[r] = 0;
-            off.dst[r] = ct == "allgather" ? (int64_t)r * (int64_t)in_bytes : 0;
-        }
-        int rc = launch_stage(src, bufp, off, R, in_bytes, s);
-        if (rc) return fail(PCCL_ERR_HIP, std::string("input staging: ") + hipGetErrorString((hipError_t)rc));
-
-        run_program(ctx, e, ctx->bufs.data(), ctx->buf_bytes, s);
-
-        if (ct == "reduce_scatter") {
-            size_t chunk = in_bytes / R;
-            for (int r = 0; r < R; ++r) { off.src[r] = (int64_t)r * (int64_t)chunk; off.dst[r] = 0; }
-            rc = launch_stage(bufp, dst, off, R, chunk, s);
-        } else if (ct == "alltoall") {
-            size_t chunk = in_bytes / R;
-            rc = 0;
-            for (int p = 0; p < R && rc == 0; ++p) {
-                for (int r = 0; r < R; ++r) {
-                    off.src[r] = p == r ? (int64_t)r * (int64_t)chunk : (int64_t)in_bytes + (int64_t)p * (int64_t)chunk;
-                    off.dst[r] = (int64_t)p * (int64_t)chunk;
-                }
-                rc = launch_stage(bufp, dst, off, R, chunk, s);
-            }
-        } else {
-            for (int r = 0; r < R; ++r) { off.src[r] = 0; off.dst[r] = 0; }
-            rc = launch_stage(bufp, dst, off, R, out_bytes, s);
-        }
-        if (rc) return fail(PCCL_ERR_HIP, std::string("output staging: ") + hipGetErrorString((hipError_t)rc));
+        // on the caller's tensors where the program allows it, else through the rank buffers
+        if (!run_direct(ctx, e, inputs, outputs, in_bytes, out_bytes, s) &&
+            !run_gather(ctx, e, inputs, outputs, in_bytes, out_bytes, s))
+            run_staged(ctx, e, inputs, outputs, in_bytes, out_bytes, s);
         ctx->last_stream = s;
         if (sync) { HIP_TRY(hipStreamSynchronize(s)); check_stall(e, name); }
         return 0;
