@@ -49,6 +49,7 @@ class Engine:
         _lib.check(self._L.pccl_hip_create(ctypes.byref(h), device, num_vranks))
         self._h = h
         self._posted: Dict[str, Dict[int, tuple]] = {}
+        self._elem_bytes: Dict[str, int] = {}      # per operation: element size of the graph's dtype
         self._views = [RankView(self, r) for r in range(num_vranks)]
 
     def close(self) -> None:
@@ -67,6 +68,7 @@ class Engine:
         """Register rank ``rank``'s graph file; with ``rank=None`` ``filename`` must contain
         ``{rank}`` and all virtual ranks are registered.  Returns False when a file cannot be
         loaded (like the reference's ``regOp``); a bad primitive or dtype raises."""
+        self._elem_bytes.pop(name, None)
         ranks = [rank] if rank is not None else list(range(self.num_vranks))
         if rank is None and "{rank}" not in filename:
             raise ValueError("register_operation without rank needs a '{rank}' placeholder in filename")
@@ -82,6 +84,7 @@ class Engine:
         return True
 
     def register_operation_json(self, name: str, text: str, rank: int) -> bool:
+        self._elem_bytes.pop(name, None)
         data = text.encode()
         _lib.check(self._L.pccl_hip_register_json(self._h, name.encode(), rank, data, len(data)))
         return True
@@ -104,6 +107,19 @@ class Engine:
                 raise ValueError(f"{what}: tensors must be contiguous")
         return ts
 
+    _DTYPE_BYTES = {0: 4, 1: 2, 2: 2, 3: 1, 4: 1, 5: 4}    # pccl_dtype -> bytes per element
+
+    def _check_dtype(self, name: str, ts: List[torch.Tensor], what: str) -> None:
+        """The library sees bytes, and the reference checks nothing (engine_c.cc:304-320): a tensor
+        whose elements are not the size of the graph's dtype is certainly a mistake, so say so."""
+        es = self._elem_bytes.get(name)
+        if es is None:
+            es = self._elem_bytes[name] = self._DTYPE_BYTES[self.op_info(name)["dtype"]]
+        for x in ts:
+            if x.element_size() != es:
+                raise ValueError(f"{what}: {x.dtype} has {x.element_size()}-byte elements, "
+                                 f"operation '{name}' was compiled for {es}-byte elements")
+
     def _ptrs(self, ts: List[torch.Tensor]):
         return (ctypes.c_void_p * len(ts))(*[x.data_ptr() for x in ts])
 
@@ -111,6 +127,8 @@ class Engine:
         nb_in, nb_out = inputs[0].nbytes, outputs[0].nbytes
         if any(x.nbytes != nb_in for x in inputs) or any(x.nbytes != nb_out for x in outputs):
             raise ValueError("all ranks must pass tensors of the same size")
+        self._check_dtype(name, inputs, "inputs")
+        self._check_dtype(name, outputs, "outputs")
         _lib.check(self._L.pccl_hip_execute(self._h, name.encode(), self._ptrs(inputs), self._ptrs(outputs),
                                             nb_in, nb_out, _current_stream_ptr(self.device), int(sync)))
 
@@ -129,6 +147,7 @@ class Engine:
     def execute_inplace(self, name: str, bufs: TensorList, sync: bool = False):
         """Zero-copy execution: ``bufs[r]`` is rank ``r``'s buffer and is updated in place."""
         bs = self._as_list(bufs, "bufs")
+        self._check_dtype(name, bs, "bufs")
         # the library checks the program's extent against one size: the smallest buffer's
         _lib.check(self._L.pccl_hip_execute_inplace(self._h, name.encode(), self._ptrs(bs), min(b.nbytes for b in bs),
                                                     _current_stream_ptr(self.device), int(sync)))
@@ -144,6 +163,9 @@ class Engine:
         outs = None if outputs is None else self._as_list(outputs, "outputs")
         if any(x.nbytes != ins[0].nbytes for x in ins) or (outs and any(x.nbytes != outs[0].nbytes for x in outs)):
             raise ValueError("all ranks must pass tensors of the same size")
+        self._check_dtype(name, ins, "inputs")
+        if outs:
+            self._check_dtype(name, outs, "outputs")
         return PreparedCall(self, name, ins, outs)
 
     def sync_operation(self, name: str) -> None:

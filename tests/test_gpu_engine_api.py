@@ -388,3 +388,21 @@ def test_calls_from_several_threads(engine_factory):
         t.join(timeout=100)
     assert not any(t.is_alive() for t in threads), "a worker thread did not finish"
     assert not errors, errors
+
+
+def test_tensors_of_the_wrong_element_size_are_refused(engine_factory):
+    world, n = 2, 2048
+    eng = engine_factory(world)
+    for r, j in enumerate(graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm")):
+        eng.register_operation_json("ar_bf16_only", j, r)
+    wrong = [torch.zeros(n, device="cuda", dtype=torch.float32) for _ in range(world)]
+    with pytest.raises(ValueError, match="4-byte elements"):
+        eng.execute_inplace("ar_bf16_only", wrong)
+    with pytest.raises(ValueError, match="4-byte elements"):
+        eng.execute_operation("ar_bf16_only", wrong)
+    right = [torch.ones(n, device="cuda", dtype=torch.bfloat16) for _ in range(world)]
+    eng.execute_inplace("ar_bf16_only", right, sync=True)
+    assert torch.all(right[0].float() == 2)
+    as_int16 = [t.view(torch.int16) for t in right]          # same element size: the bytes are what counts
+    eng.execute_inplace("ar_bf16_only", as_int16, sync=True)
+    assert torch.all(right[1].float() == 4)
