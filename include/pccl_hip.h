@@ -29,7 +29,10 @@ typedef enum {
     PCCL_ERR_PARSE = -3,       /* malformed graph document, unknown primitive or dtype */
     PCCL_ERR_LINK = -4,        /* ranks missing, deadlock, unbalanced signals, data race */
     PCCL_ERR_HIP = -5,         /* a HIP runtime call failed */
-    PCCL_ERR_UNSUPPORTED = -6  /* valid request this build does not implement */
+    PCCL_ERR_UNSUPPORTED = -6, /* valid request this build does not implement */
+    PCCL_ERR_NOT_A_GRAPH = -7  /* a readable JSON document without an 'operations' array, or with an
+                                * operation lacking index / executor / primitive: the two cases in which
+                                * the reference's loader returns false (csrc/engine/graph_builder.cc:22-41) */
 } pccl_status;
 
 /* Element types, numbered like the reference's DataType (csrc/plugins/cuda/kernel/compute.h:13-19);

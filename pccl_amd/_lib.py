@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libpccl_hip.so")
 MAX_VRANKS = 64
 MAX_CHANNELS = 8
 
-OK, ERR_INVALID, ERR_NOT_FOUND, ERR_PARSE, ERR_LINK, ERR_HIP, ERR_UNSUPPORTED = 0, -1, -2, -3, -4, -5, -6
+OK, ERR_INVALID, ERR_NOT_FOUND, ERR_PARSE, ERR_LINK, ERR_HIP, ERR_UNSUPPORTED, ERR_NOT_A_GRAPH = 0, -1, -2, -3, -4, -5, -6, -7
 
 DTYPE_ID = {"float32": 0, "float16": 1, "bfloat16": 2, "float8_e4m3": 3, "float8_e5m2": 4, "int32": 5}
 REDOP_ID = {"sum": 0, "max": 1, "min": 2}

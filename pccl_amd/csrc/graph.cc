@@ -89,7 +89,7 @@ RankGraph load_graph_json(const char* text, size_t len) {
         throw Error{PCCL_ERR_PARSE, e.what()};
     }
     if (!doc.is_object() || !doc.contains("operations") || !doc.at("operations").is_array())
-        throw Error{PCCL_ERR_PARSE, "graph document has no 'operations' array"};
+        throw Error{PCCL_ERR_NOT_A_GRAPH, "graph document has no 'operations' array"};
 
     RankGraph g;
     std::string dtype_name;
@@ -116,7 +116,7 @@ RankGraph load_graph_json(const char* text, size_t len) {
         for (size_t pos = 0; pos < ops.size(); ++pos) {
             const json::Value& op = ops[pos];
             if (!op.is_object() || !op.contains("index") || !op.contains("executor") || !op.contains("primitive"))
-                throw Error{PCCL_ERR_PARSE, "operation " + std::to_string(pos) + " lacks index/executor/primitive"};
+                throw Error{PCCL_ERR_NOT_A_GRAPH, "operation " + std::to_string(pos) + " lacks index/executor/primitive"};
             GraphOp& o = g.ops[pos];
             o.index = (int)op.at("index").as_int("index");
             by_index.emplace_back(o.index, (int)pos);

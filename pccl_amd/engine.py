@@ -75,10 +75,7 @@ class Engine:
         for r in ranks:
             path = filename.format(rank=r) if "{rank}" in filename else filename
             rc = self._L.pccl_hip_register_file(self._h, name.encode(), r, path.encode())
-            if rc in (_lib.ERR_NOT_FOUND,):
-                return False
-            if rc == _lib.ERR_PARSE and "lacks index/executor/primitive" in self.last_error() or \
-               rc == _lib.ERR_PARSE and "no 'operations'" in self.last_error():
+            if rc in (_lib.ERR_NOT_FOUND, _lib.ERR_NOT_A_GRAPH):   # where the reference's loader returns false
                 return False
             _lib.check(rc)
         return True

@@ -11,7 +11,7 @@ import pytest
 
 from helpers import ROOT, graph_jsons, oracle
 from pccl_amd import _lib
-from pccl_amd._lib import (ERR_INVALID, ERR_LINK, ERR_NOT_FOUND, ERR_PARSE, ERR_UNSUPPORTED, HostGraph,
+from pccl_amd._lib import (ERR_INVALID, ERR_LINK, ERR_NOT_A_GRAPH, ERR_NOT_FOUND, ERR_PARSE, ERR_UNSUPPORTED, HostGraph,
                            HostProgram, PcclError)
 from pccl_amd.dsl import CommunicationOp, compile_to_json_string
 
@@ -106,9 +106,9 @@ def test_load_errors():
         HostGraph.from_file("/nonexistent/graph.json")
     assert e.value.code == ERR_NOT_FOUND                       # reference: regOp returns false
     d = _doc(); del d["operations"]
-    assert _load_err(d).code == ERR_PARSE                       # reference: returns false
+    assert _load_err(d).code == ERR_NOT_A_GRAPH                 # reference: returns false
     d = _doc(); del d["operations"][3]["primitive"]
-    assert "index/executor/primitive" in str(_load_err(d))
+    assert "index/executor/primitive" in str(_load_err(d)) and _load_err(d).code == ERR_NOT_A_GRAPH   # false there too
     d = _doc(); d["operations"][2]["primitive"] = "sm.scatter"
     assert "unknown primitive" in str(_load_err(d))             # reference: throws
     d = _doc(); d["tensor_info"]["dtype"] = "float64"
