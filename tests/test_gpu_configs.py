@@ -163,6 +163,35 @@ def test_config2_headline_shape_in_all_modes_agree(engine_factory):
             assert same_bits(results["column"][lo:lo + per_rank], acc)
 
 
+def test_largest_rank_buffers_the_graph_format_allows(engine_factory):
+    """Offsets and sizes in a graph are 32-bit element counts (reference include/engine/fused_step.h:11-14),
+    so the largest rank buffer is 2^31 - 1 elements.  A two-rank f32 ring on 2^31 - 2 elements (8 GiB per
+    rank, chunks of 2^30 - 1 elements, so the second chunk starts 4 bytes short of 4 GiB and off 16-byte
+    alignment) puts byte offsets beyond 2^32 through every runner.  Integer-valued inputs make the sum
+    exact, and with two ranks the order of the one addition does not matter."""
+    world, n = 2, (1 << 31) - 2
+    print(f"largest buffers: ring R={world} n={n} f32, column / stepwise / persistent / staged", flush=True)
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)
+    x = dev_inputs("randint", world, n, "float32")
+    want = x[0] + x[1]
+    engine = engine_factory(world)
+    for mode in ("column", "stepwise", "persistent"):
+        print(f"  mode={mode}", flush=True)
+        register(engine, f"big_{mode}", jsons, mode)
+        bufs = [t.clone() for t in x]
+        engine.execute_inplace(f"big_{mode}", bufs, sync=True)
+        for r in range(world):
+            assert same_bits(bufs[r], want), f"mode {mode}, rank {r}"
+        del bufs
+    print("  staged call", flush=True)
+    register(engine, "big_staged", jsons, "auto")
+    outs = [torch.full((n,), -1.0, device="cuda") for _ in range(world)]
+    engine.execute_operation("big_staged", x, outs)
+    for r in range(world):
+        assert same_bits(outs[r], want), f"staged call, rank {r}"
+    assert engine.op_info("big_staged")["algorithmic_bytes"] == 5 * n * 4
+
+
 def test_config3_full_size_against_the_cpu_oracle(engine_factory):
     """Configuration 3 at its full size (16 x 64 MiB f32, two channels) with the prescribed inputs
     from the CPU generator, the GPU result compared bit for bit with the CPU oracle's (about a

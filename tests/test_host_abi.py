@@ -190,6 +190,22 @@ def _link(jsons):
     return HostProgram([HostGraph.from_json(j) for j in jsons])
 
 
+def test_element_counts_are_32_bit_like_the_reference_descriptors():
+    """Offsets and sizes are ints in the reference's trigger and fused step (include/engine/fused_step.h:11-14,
+    cuda_executor.cu:63-72): a graph whose op reaches 2^31 elements is refused at load time, one that
+    stays a single element below loads, links and keeps its descriptor forms exact."""
+    n = (1 << 31) - 2
+    jsons = graph_jsons("ring", "build_allreduce", 2, n, "float32", "sm", 1)
+    g = HostGraph.from_json(jsons[0])
+    trig, cnt = g.triggers()
+    assert max(trig[i].offset_0 + trig[i].size for i in range(cnt) if trig[i].primitive_type in (1, 3, 64, 65, 8)) <= n
+    assert any(trig[i].offset_0 == n // 2 and trig[i].size == n // 2 for i in range(cnt))
+    assert _link(jsons).info()["algorithmic_bytes"] == 5 * n * 4
+    with pytest.raises(PcclError) as e:
+        HostGraph.from_json(graph_jsons("ring", "build_allreduce", 2, 1 << 32, "float32", "sm", 1)[0])
+    assert e.value.code == ERR_PARSE and "32-bit element range" in str(e.value)
+
+
 def test_program_info_closed_forms():
     world, n = 8, 8192 * 4
     info = _link(graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 4)).info()
