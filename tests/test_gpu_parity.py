@@ -214,6 +214,40 @@ def _ring_partial(kind, rank, world, n):
     return compile_to_json_string(op.get_graph())
 
 
+@pytest.mark.parametrize("mode", ["auto", "column", "stepwise", "persistent"])
+@pytest.mark.parametrize("what", ["no operations", "zero-size data ops"])
+def test_empty_graphs_and_zero_size_ops_leave_the_data_alone(engine_factory, what, mode):
+    """A graph without operations, and a ring whose reduces and copies all have size 0 (its notify /
+    wait chain intact), register and run; nothing is moved.  In the reference's call shape the input
+    is staged into the rank buffer and the output read back from it (engine_c.cc:524-543), so the
+    output equals the input; in place the buffers keep their contents.  The oracle agrees."""
+    import json
+    world, n = 4, 4096
+    docs = [json.loads(t) for t in graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)]
+    for d in docs:
+        if what == "no operations":
+            d["operations"] = []
+        else:
+            for op in d["operations"]:
+                for key in ("size", "count"):
+                    if key in op.get("params", {}):
+                        op["params"][key] = 0
+    jsons = [json.dumps(d) for d in docs]
+    inputs = seeded_inputs("randn", world, n, "float32", seed=11)
+    expect = oracle_buffers(jsons, inputs, "float32")
+    for r in range(world):
+        assert bits_equal(expect[r], inputs[r])
+    engine = engine_factory(world)
+    got, info = run_gpu(engine, jsons, inputs, mode, inplace=True)
+    assert info["algorithmic_bytes"] == 0
+    for r in range(world):
+        assert bits_equal(got[r], inputs[r]), f"in place, rank {r}"
+    got, _ = run_gpu(engine, jsons, inputs, mode)
+    for r in range(world):
+        assert bits_equal(got[r], inputs[r]), f"staged, rank {r}"
+    engine.set_option("mode", "auto")
+
+
 @pytest.mark.parametrize("fuse", [1, 0])
 @pytest.mark.parametrize("kind", ["reduce", "copy"])
 def test_partial_ring_graphs_pass_untouched_chunks_through(engine_factory, kind, fuse):
