@@ -229,7 +229,13 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * "slot_threads" = 0 | 64 | 128 | 256 (workgroup size of that runner, 0 = from the rank count);
  * "slot_direct" = "1" | "0" (first touches loaded straight into LDS, or through registers);
  * "level_graph" = "0" | "1" (the level runner launches level by level, or replays the launches of an
- * execution as one HIP graph captured per set of rank pointers). */
+ * execution as one HIP graph captured per set of rank pointers);
+ * "trace_ranges" = "0" | "1" (host-side roctx ranges around the stages of a call, under the names of
+ * the reference's NVTX ranges, include/common/nvtx.h:7-16, csrc/engine_c.cc:468-489,
+ * csrc/plugins/cuda/cuda_device.cc:313-319: "d2d_input_copy", "execute", "d2d_output_copy", and
+ * inside "execute" "fused_kernel" for the column runner or "executor_kernel" for the level and
+ * persistent runners; the marker library is loaded at run time and PCCL_ERR_UNSUPPORTED is returned
+ * if there is none; the environment variable PCCL_TRACE_RANGES=1 sets it for new contexts). */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
 
 /* Engine::exeOp / exeOpAsync (reference csrc/engine_c.cc:269-560): for every virtual rank r copy

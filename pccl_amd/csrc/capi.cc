@@ -1,4 +1,5 @@
 // C ABI: host-only graph tools and the device executor context.
+#include <dlfcn.h>
 #include <hip/hip_runtime_api.h>
 
 #include <cstdio>
@@ -45,6 +46,41 @@ int guarded(F&& f) {
         hipError_t e_ = (expr);                                                                         \
         if (e_ != hipSuccess) throw Error{PCCL_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)}; \
     } while (0)
+
+// Host-side ranges for a profiler's timeline, under the names of the reference's NVTX ranges
+// (include/common/nvtx.h:7-16; engine_c.cc:468,485,489; cuda_device.cc:313,319).  The marker
+// library is looked up at run time, the first time a context asks for ranges; without it (or
+// without the option) a range costs one branch.
+struct MarkerApi {
+    int (*push)(const char*) = nullptr;
+    int (*pop)() = nullptr;
+};
+
+const MarkerApi& marker_api() {
+    static const MarkerApi api = [] {
+        MarkerApi m;
+        for (const char* lib : {"librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4", "libroctx64.so"}) {
+            void* h = dlopen(lib, RTLD_NOW | RTLD_GLOBAL);
+            if (!h) continue;
+            m.push = (int (*)(const char*))dlsym(h, "roctxRangePushA");
+            m.pop = (int (*)())dlsym(h, "roctxRangePop");
+            if (m.push && m.pop) break;
+            m = MarkerApi{};
+        }
+        return m;
+    }();
+    return api;
+}
+
+class TraceRange {
+  public:
+    TraceRange(bool wanted, const char* name) : on_(wanted && marker_api().push) { if (on_) marker_api().push(name); }
+    ~TraceRange() { if (on_) marker_api().pop(); }
+    TraceRange(const TraceRange&) = delete;
+    TraceRange& operator=(const TraceRange&) = delete;
+  private:
+    bool on_;
+};
 
 void fill_info(const Program& p, pccl_program_info* out) {
     std::memset(out, 0, sizeof(*out));
@@ -290,6 +326,7 @@ struct pccl_hip_ctx {
     int vecs_per_thread = 1;
     bool check_races = true;
     bool timing = false;
+    bool trace_ranges = false;            // emit profiler ranges around the stages of a call
     bool lds_slots = true;                // column runner keeps re-read values in LDS slots
     int slot_threads = 0;                 // slot runner workgroup size (0: chosen from the rank count)
     bool slot_direct = true;              // slot runner fetches first touches straight into LDS
@@ -508,6 +545,7 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
         throw Error{PCCL_ERR_UNSUPPORTED, P.position_aligned ? "column mode needs 16-byte aligned rank buffers" : "column mode needs every data op to read and write the same element positions"};
     if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
     int rc;
+    TraceRange range(ctx->trace_ranges, column ? "fused_kernel" : "executor_kernel");
     if (column) {
         ColumnLaunch L{};
         L.segs = (const DevColSegment*)e.segs.p; L.num_segs = (int)P.segs.size();
@@ -578,6 +616,7 @@ bool run_direct(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
     L.slot_threads = e.slot_threads; L.num_ranks = ctx->R; L.slot_direct = ctx->slot_direct;
     L.total_tiles = e.direct_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
     L.num_blocks = ctx->num_blocks;
+    TraceRange exe(ctx->trace_ranges, "execute"), range(ctx->trace_ranges, "fused_kernel");
     int rc = launch_column(L, ptrs, stream);
     if (rc != 0) throw Error{PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)};
     if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, stream)); e.timed = true; }
@@ -603,6 +642,7 @@ bool run_gather(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
     RankPtrs src{}, dst{};
     for (int r = 0; r < R; ++r) { src.p[r] = (char*)inputs[r]; dst.p[r] = (char*)outputs[r]; }
     if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, s));
+    TraceRange exe(ctx->trace_ranges, "execute"), range(ctx->trace_ranges, "fused_kernel");
     int rc = launch_gather((const DevGatherCopy*)e.gather.p, (int)P.gather.size(), e.gather_tiles, e.gather_copy_tiles, src, dst, s);
     if (rc) throw Error{PCCL_ERR_HIP, std::string("gather launch failed: ") + hipGetErrorString((hipError_t)rc)};
     if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, s)); e.timed = true; }
@@ -635,11 +675,19 @@ void run_staged(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
         off.src[r] = 0;
         off.dst[r] = ct == "allgather" ? (int64_t)r * (int64_t)in_bytes : 0;
     }
-    int rc = launch_stage(src, bufp, off, R, in_bytes, s);
+    int rc;
+    {
+        TraceRange range(ctx->trace_ranges, "d2d_input_copy");
+        rc = launch_stage(src, bufp, off, R, in_bytes, s);
+    }
     if (rc) throw Error{PCCL_ERR_HIP, std::string("input staging: ") + hipGetErrorString((hipError_t)rc)};
 
-    run_program(ctx, e, ctx->bufs.data(), ctx->buf_bytes, s);
+    {
+        TraceRange range(ctx->trace_ranges, "execute");
+        run_program(ctx, e, ctx->bufs.data(), ctx->buf_bytes, s);
+    }
 
+    TraceRange range(ctx->trace_ranges, "d2d_output_copy");
     const size_t chunk = in_bytes / R;
     if (ct == "reduce_scatter") {           // chunk r of buffer r
         for (int r = 0; r < R; ++r) { off.src[r] = (int64_t)r * (int64_t)chunk; off.dst[r] = 0; }
@@ -714,6 +762,7 @@ int pccl_hip_create(pccl_hip_ctx** out, int device, int num_vranks) {
         ctx->bufs.assign(num_vranks, nullptr);
         if (const char* nb = std::getenv("PCCL_NUM_BLOCKS")) ctx->num_blocks = std::atoi(nb);
         if (std::getenv("PCCL_DISABLE_FUSED")) ctx->mode = Mode::Stepwise;
+        if (const char* tr = std::getenv("PCCL_TRACE_RANGES")) ctx->trace_ranges = std::atoi(tr) != 0;
         *out = ctx.release();
         return 0;
     });
@@ -763,6 +812,10 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             else return fail(PCCL_ERR_INVALID, "mode must be auto, column, stepwise or persistent");
         } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
         else if (k == "timing") ctx->timing = std::atoi(value) != 0;
+        else if (k == "trace_ranges") {
+            ctx->trace_ranges = std::atoi(value) != 0;
+            if (ctx->trace_ranges && !marker_api().push) { ctx->trace_ranges = false; return fail(PCCL_ERR_UNSUPPORTED, "trace_ranges: no roctx marker library could be loaded"); }
+        }
         else if (k == "fuse_staging") ctx->fuse_staging = std::atoi(value) != 0;
         else if (k == "wait_timeout_ms") { ctx->wait_timeout_ms = std::atoi(value); if (ctx->wait_timeout_ms < 0) ctx->wait_timeout_ms = 0; }   // 0: give up on the first predecessor that is not ready
         else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
@@ -823,7 +876,10 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
         OpEntry& e = find_entry(ctx, name);
         link_entry(ctx, e);
         hipStream_t s = (hipStream_t)stream;
-        run_program(ctx, e, (char* const*)bufs, buf_bytes, s);
+        {
+            TraceRange exe(ctx->trace_ranges, "execute");
+            run_program(ctx, e, (char* const*)bufs, buf_bytes, s);
+        }
         ctx->last_stream = s;
         if (sync) { HIP_TRY(hipStreamSynchronize(s)); check_stall(e, name); }
         return 0;

@@ -190,6 +190,34 @@ def test_kernel_timing_option(engine_factory):
     assert 0.0 < ms < 50.0
 
 
+def test_profiler_ranges_option(engine_factory):
+    """The reference wraps the stages of a call in NVTX ranges (engine_c.cc:468-489, cuda_device.cc:313-319);
+    here they are roctx ranges behind an option.  Without a profiler attached they must change nothing:
+    staged and in-place calls in every mode give the bits they give without them."""
+    world, n = 4, 1 << 14
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 2)
+    x = seeded_inputs("randn", world, n, "float32", seed=21)
+    want = oracle_buffers(jsons, x, "float32")
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("ranges", j, r)
+    eng.set_option("trace_ranges", 1)
+    try:
+        for mode in ("auto", "stepwise", "persistent"):
+            eng.set_option("mode", mode)
+            for fuse in (1, 0):
+                eng.set_option("fuse_staging", fuse)
+                outs = eng.execute_operation("ranges", [t.cuda() for t in x])
+                bufs = [t.cuda() for t in x]
+                eng.execute_inplace("ranges", bufs, sync=True)
+                for r in range(world):
+                    assert bits_equal(outs[r].cpu(), want[r]) and bits_equal(bufs[r].cpu(), want[r]), (mode, fuse, r)
+    finally:
+        eng.set_option("trace_ranges", 0)
+        eng.set_option("fuse_staging", 1)
+        eng.set_option("mode", "auto")
+
+
 def test_registration_from_trigger_arrays(engine_factory):
     """What a C++ engine that parses the JSON itself would hand over: the 32-byte triggers and the
     88-byte metadata records (reference proxy_trigger.h:8-16, primitive.h:8-17)."""
