@@ -3,6 +3,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -28,11 +29,35 @@ int fail(int code, const std::string& msg) {
     return code;
 }
 
+// Log lines on stderr, levels and the PCCL_LOG_LEVEL switch as in the reference
+// (csrc/common/logging.cc:6-35, default WARN); stdout stays free for the caller's own output.
+enum LogLevel { LOG_TRACE, LOG_DEBUG, LOG_INFO, LOG_WARN, LOG_ERROR, LOG_CRITICAL };
+
+int log_threshold() {
+    static const int level = [] {
+        const char* v = std::getenv("PCCL_LOG_LEVEL");
+        const std::string s = v ? v : "";
+        const char* names[] = {"TRACE", "DEBUG", "INFO", "WARN", "ERROR", "CRITICAL"};
+        for (int i = 0; i < 6; ++i)
+            if (s == names[i]) return i;
+        return (int)LOG_WARN;
+    }();
+    return level;
+}
+
+void log_line(int level, const std::string& msg) {
+    if (level < log_threshold()) return;
+    const char* tags[] = {"trace", "debug", "info", "warning", "error", "critical"};
+    std::fprintf(stderr, "[pccl] [%s] %s\n", tags[level], msg.c_str());
+}
+
 template <class F>
 int guarded(F&& f) {
     try {
         return f();
     } catch (const Error& e) {
+        // the caller gets the message with the status code; the log repeats it only on request
+        log_line(e.code == PCCL_ERR_HIP ? LOG_ERROR : LOG_INFO, "call failed (" + std::to_string(e.code) + "): " + e.msg);
         return fail(e.code, e.msg);
     } catch (const std::bad_alloc&) {
         return fail(PCCL_ERR_INVALID, "out of host memory");
@@ -464,6 +489,15 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
     HIP_TRY(hipEventCreate(&e.ev0));
     HIP_TRY(hipEventCreate(&e.ev1));
     e.linked = true;
+    if (log_threshold() <= LOG_INFO)   // the reference's "Fused step executor enabled" line (engine_c.cc:357)
+        log_line(LOG_INFO, "linked " + std::to_string(ctx->R) + " rank graphs: " + std::to_string(P.ops.size()) + " data ops on " +
+                               std::to_string(P.num_levels) + " levels, " + std::to_string(P.num_items) + " work items of " +
+                               std::to_string(P.tile_elems * es) + " bytes; " +
+                               (P.position_aligned ? "position aligned, " + std::to_string(P.segs.size()) + " column segments, " +
+                                                         (e.slot_threads > 0 ? "slot runner with " + std::to_string(e.slot_threads) + " threads"
+                                                                             : std::string("register runner"))
+                                                   : std::string("not position aligned: level / persistent runner")) +
+                               (P.gather.empty() ? "" : "; alltoall gather plan of " + std::to_string(P.gather.size()) + " copies"));
 }
 
 OpEntry& find_entry(pccl_hip_ctx* ctx, const char* name) {
@@ -739,6 +773,9 @@ int register_graph(pccl_hip_ctx* ctx, const char* name, int vrank, RankGraph&& g
     if (e.graphs.empty()) e.graphs.resize(ctx->R);
     if (e.linked) { HIP_TRY(hipDeviceSynchronize()); e.release(); }  // re-registration replaces the op
     e.graphs[vrank] = std::make_unique<RankGraph>(std::move(g));
+    if (log_threshold() <= LOG_INFO)   // reference engine_c.cc:168,199
+        log_line(LOG_INFO, std::string("operation '") + name + "' registered for virtual rank " + std::to_string(vrank) + ": " +
+                               std::to_string(e.graphs[vrank]->ops.size()) + " ops");
     return 0;
 }
 
@@ -763,6 +800,8 @@ int pccl_hip_create(pccl_hip_ctx** out, int device, int num_vranks) {
         if (const char* nb = std::getenv("PCCL_NUM_BLOCKS")) ctx->num_blocks = std::atoi(nb);
         if (std::getenv("PCCL_DISABLE_FUSED")) ctx->mode = Mode::Stepwise;
         if (const char* tr = std::getenv("PCCL_TRACE_RANGES")) ctx->trace_ranges = std::atoi(tr) != 0;
+        if (log_threshold() <= LOG_INFO)   // reference engine_c.cc:84,163
+            log_line(LOG_INFO, "engine context on device " + std::to_string(device) + " with " + std::to_string(num_vranks) + " virtual ranks");
         *out = ctx.release();
         return 0;
     });

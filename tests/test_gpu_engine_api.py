@@ -218,6 +218,33 @@ def test_profiler_ranges_option(engine_factory):
         eng.set_option("mode", "auto")
 
 
+def test_info_log_lines_of_registration_and_linking():
+    """The reference logs engine start, registration and the runner it picked at INFO
+    (engine_c.cc:84,163,168,199,357); the same three moments are logged here, on stderr."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys; sys.path[:0] = [%r, %r]\n"
+        "import torch\n"
+        "from helpers import graph_jsons\n"
+        "from pccl_amd.engine import Engine\n"
+        "e = Engine(2, 0)\n"
+        "for r, j in enumerate(graph_jsons('ring', 'build_allreduce', 2, 4096, 'float32', 'sm', 1)):\n"
+        "    e.register_operation_json('logged', j, r)\n"
+        "b = [torch.ones(4096, device='cuda') for _ in range(2)]\n"
+        "e.execute_inplace('logged', b, sync=True)\n"
+        "print('sum', float(b[0][0]))\n"
+        "e.close()\n") % (root, os.path.join(root, "tests"))
+    env = dict(os.environ, PCCL_LOG_LEVEL="INFO")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip().splitlines()[-1] == "sum 2.0"
+    assert "[pccl] [info] engine context on device 0 with 2 virtual ranks" in out.stderr
+    assert "[pccl] [info] operation 'logged' registered for virtual rank 1: " in out.stderr
+    assert "[pccl] [info] linked 2 rank graphs: 4 data ops on 2 levels" in out.stderr and "slot runner with 256 threads" in out.stderr
+
+
 def test_registration_from_trigger_arrays(engine_factory):
     """What a C++ engine that parses the JSON itself would hand over: the 32-byte triggers and the
     88-byte metadata records (reference proxy_trigger.h:8-16, primitive.h:8-17)."""

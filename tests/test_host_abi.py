@@ -206,6 +206,23 @@ def test_element_counts_are_32_bit_like_the_reference_descriptors():
     assert e.value.code == ERR_PARSE and "32-bit element range" in str(e.value)
 
 
+def test_log_level_switch():
+    """PCCL_LOG_LEVEL as in the reference (csrc/common/logging.cc:6-35): nothing below WARN by default;
+    INFO repeats the message of a failing call on stderr, stdout stays untouched."""
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r); from pccl_amd._lib import HostGraph, PcclError\n"
+            "try: HostGraph.from_json('{}')\n"
+            "except PcclError as e: print('code', e.code)\n") % ROOT
+    for level, expect in ((None, False), ("INFO", True), ("ERROR", False), ("nonsense", False)):
+        env = {k: v for k, v in os.environ.items() if k != "PCCL_LOG_LEVEL"}
+        if level:
+            env["PCCL_LOG_LEVEL"] = level
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+        assert out.stdout.strip() == f"code {ERR_NOT_A_GRAPH}"
+        assert ("[pccl] [info] call failed (-7)" in out.stderr) == expect, (level, out.stderr)
+
+
 def test_program_info_closed_forms():
     world, n = 8, 8192 * 4
     info = _link(graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 4)).info()
