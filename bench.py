@@ -147,7 +147,14 @@ def cpu_baseline(sample_elems: int, channels: int, reps: int = 3):
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), "")
+    except OSError:
+        pass
     return {"value": round(stats.bytes / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "cpu_model": model, "host_cpus_visible": os.cpu_count(),
             "sample": f"same ring graph (R={R}, {channels} channels, bf16) at {sample_elems} elements "
                       f"per rank ({sample_elems * 2 >> 20} MiB), {stats.bytes} algorithmic bytes, median of "
                       f"{reps} runs after 1 warm-up, {med * 1e3:.1f} ms"}
