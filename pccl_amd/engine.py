@@ -100,6 +100,8 @@ class Engine:
         for x in ts:
             if not x.is_cuda:
                 raise ValueError(f"{what}: tensors must live on the GPU")
+            if x.device != self.device:
+                raise ValueError(f"{what}: tensor on {x.device}, the engine runs on {self.device}")
             if not x.is_contiguous():
                 raise ValueError(f"{what}: tensors must be contiguous")
         return ts
