@@ -561,7 +561,7 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
                 for (int t = tid; t < nt; t += kThreads) wait_for(&flags[first + t], d);
             }
         } else if (tid == 0 && op.ndeps > 0 && seen != epoch) {
-            // every other tile waits for the first tile's verdict, one word
+            // every other tile waits for the first tile's answer, one word
             wait_for(&ready[opi], as_const(L.deps)[op.dep_start]);
         }
         __syncthreads();   // everything this workgroup waited for has been seen; the data accesses
