@@ -187,9 +187,16 @@ typedef PCCL_GLOBAL u32x4* gvec_ptr;
 __device__ __forceinline__ u32x4 ldv(const char* p) { return *(gvec_cptr)(p); }
 __device__ __forceinline__ void stv(char* p, u32x4 v) { *(gvec_ptr)(p) = v; }
 // Streaming variants for data touched once.  Two forms, both measured on MI355X:
-//  * pointer form, non-temporal (nt): used by the column runners, whose per-store scalar work
-//    matters (building a buffer descriptor per store cost the 32-rank tree 5 %, and the ring is
-//    the same either way);
+//  * pointer form: used by the column runners, whose per-store scalar work matters (building a
+//    buffer descriptor per store cost the 32-rank tree 5 %, and the ring is the same either way).
+//    Loads are non-temporal (nt; agent scope on top changes nothing for them).  Stores are nt sc1
+//    like those of the buffer form below: programs that mostly write gain from the agent-scope bit
+//    (8-rank allgather as one launch on the caller's tensors, 512 MB per rank 0.91 -> 0.81 ms,
+//    16 MB per rank 31 -> 24 us), programs that read as much as they write are the same either way
+//    (headline ring, halving-doubling, tree, reduce_scatter).  The compiler has no builtin for a
+//    pointer store with that bit, hence the asm; the s_nop gives the one wait state that a 128-bit
+//    store needs before a vector instruction may overwrite its data registers, which the compiler
+//    inserts for stores it knows and cannot for this one;
 //  * raw buffer operations (wave-uniform base in a resource descriptor, 32-bit byte offset per
 //    lane) marked non-temporal AND agent scope (nt sc1): used by everything built on range_op.
 //    Headline graph with the level runner: cached 3.22 ms, sc1 3.18, nt 3.06 (as global or as
@@ -197,7 +204,9 @@ __device__ __forceinline__ void stv(char* p, u32x4 v) { *(gvec_ptr)(p) = v; }
 //    makes the access coherent across the XCDs' L2s (a store is written through before it is
 //    acknowledged, a load does not hit a stale line), which the persistent runner relies on.
 __device__ __forceinline__ u32x4 ldv_nt(const char* p) { return __builtin_nontemporal_load((gvec_cptr)(p)); }
-__device__ __forceinline__ void stv_nt(char* p, u32x4 v) { __builtin_nontemporal_store(v, (gvec_ptr)(p)); }
+__device__ __forceinline__ void stv_nt(char* p, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 0" : : "v"((gvec_ptr)(p)), "v"(v) : "memory");
+}
 constexpr int kAuxStream = 16 | 2;   // sc1 | nt
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const char* uniform_base) {
     return __builtin_amdgcn_make_buffer_rsrc((void*)uniform_base, 0, 0x7FFFFFFF, 0x00020000);
