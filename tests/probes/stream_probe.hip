@@ -8,7 +8,11 @@
 //            vectors, either back in place (an in-place execution) or to R other buffers (a staged
 //            call run on the caller's tensors); 4 GiB of buffers in every case
 //
-// Usage: stream_probe [width|streams|all]; prints one line per case.  Tiles are dealt to the XCDs in
+//   ceilings what the memory system gives a kernel that only reads 4 GiB, only writes 4 GiB, or
+//            copies 2 GiB to another 2 GiB, one 16-byte access per lane and 4 KiB tile, with plain
+//            non-temporal stores and with non-temporal agent-scope (nt sc1) stores
+//
+// Usage: stream_probe [width|streams|ceilings|all]; prints one line per case.  Tiles are dealt to the XCDs in
 // runs of 256 like the library's kernels do.
 #include <hip/hip_runtime.h>
 
@@ -73,6 +77,27 @@ __global__ __launch_bounds__(256) void touch(Ptrs in, Ptrs out, int64_t tiles) {
     for (int r = 0; r < R; ++r) { v[r].x += 1; __builtin_nontemporal_store(v[r], (u32x4*)(out.p[r] + off)); }
 }
 
+// MODE 0: read only (the sum of what a lane read is stored only if it equals a value it cannot
+// have, so that the loads stay); 1: write only; 2: copy.  SC1: stores as raw buffer stores marked
+// nt sc1 (wave-uniform base, 32-bit lane offset), else plain non-temporal pointer stores.
+template <int MODE, bool SC1>
+__global__ __launch_bounds__(256) void ceiling(const char* src, char* dst, int64_t tiles, uint32_t never) {
+    const int64_t tile = xcd_tile(blockIdx.x);
+    if (tile >= tiles) return;
+    const int lane_off = threadIdx.x * 16;
+    u32x4 v = u32x4{1, 2, 3, 4};
+    if constexpr (MODE != 1) v = __builtin_nontemporal_load((const u32x4*)(src + tile * 4096 + lane_off));
+    if constexpr (MODE == 0) {
+        if ((v.x ^ v.y ^ v.z ^ v.w) != never) return;
+    }
+    char* d = dst + tile * 4096;
+    if constexpr (SC1) {
+        __builtin_amdgcn_raw_buffer_store_b128(v, __builtin_amdgcn_make_buffer_rsrc((void*)d, 0, 0x7FFFFFFF, 0x00020000), lane_off, 0, 16 | 2);
+    } else {
+        __builtin_nontemporal_store(v, (u32x4*)(d + lane_off));
+    }
+}
+
 static unsigned grid_for(int64_t tiles) {
     const int64_t span = (int64_t)8 * kRun;
     return (unsigned)((tiles + span - 1) / span * span);
@@ -125,6 +150,16 @@ static void streams_case(bool in_place) {
     }
 }
 
+template <int MODE, bool SC1>
+static void ceiling_case(const char* src, char* dst, size_t bytes, const char* label) {
+    const int64_t tiles = (int64_t)(bytes / 4096);
+    // the buffers hold zeros, so the exclusive-or of a lane's four words is never 0xDEADBEEF
+    const float ms = timed_ms([&] { hipLaunchKernelGGL((ceiling<MODE, SC1>), dim3(grid_for(tiles)), dim3(256), 0, 0, src, dst, tiles, 0xDEADBEEFu); }, 10);
+    const double moved = MODE == 2 ? 2.0 * bytes : 1.0 * bytes;
+    std::printf("ceiling %-34s %.4f ms, %.0f GB/s\n", label, ms, moved / ms / 1e6);
+    std::fflush(stdout);
+}
+
 int main(int argc, char** argv) {
     const char* what = argc > 1 ? argv[1] : "all";
     const bool all = std::strcmp(what, "all") == 0;
@@ -150,6 +185,21 @@ int main(int argc, char** argv) {
             streams_case<16>(in_place);
             streams_case<32>(in_place);
         }
+    }
+    if (all || std::strcmp(what, "ceilings") == 0) {
+        const size_t bytes = (size_t)4 << 30;
+        char *a = nullptr, *b = nullptr;
+        CHECK(hipMalloc((void**)&a, bytes));
+        CHECK(hipMalloc((void**)&b, bytes));
+        CHECK(hipMemset(a, 0, bytes));
+        CHECK(hipMemset(b, 0, bytes));
+        ceiling_case<0, false>(a, b, bytes, "read 4 GiB:");
+        ceiling_case<1, false>(a, b, bytes, "write 4 GiB, nt stores:");
+        ceiling_case<1, true>(a, b, bytes, "write 4 GiB, nt sc1 stores:");
+        ceiling_case<2, false>(a, b, bytes / 2, "copy 2 GiB, nt stores:");
+        ceiling_case<2, true>(a, b, bytes / 2, "copy 2 GiB, nt sc1 stores:");
+        CHECK(hipFree(a));
+        CHECK(hipFree(b));
     }
     CHECK(hipDeviceSynchronize());
     return 0;
