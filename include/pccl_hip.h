@@ -153,6 +153,11 @@ typedef struct {
                                    into (0 = no such plan, the call stages through the rank buffers) */
     int64_t staged_load_bytes;  /* the same for a staged call that runs on the caller's tensors */
     int64_t staged_store_bytes; /* (0 when the graph has no such plan and staging copies are used) */
+    int32_t race_checked;       /* 1: every pair of conflicting accesses was checked for an ordering; 0: the
+                                   check was switched off or the program is too large for it */
+    int32_t order_checked;      /* 1: the pairing of notifies and waits was checked for ambiguity; 0: the
+                                   program has too many ops for the check (the pairing of one valid execution
+                                   order is then used unverified) */
 } pccl_program_info;
 
 /* One data op of the linked program, for inspection and tests. */

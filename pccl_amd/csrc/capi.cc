@@ -125,6 +125,25 @@ void fill_info(const Program& p, pccl_program_info* out) {
     out->num_gather_copies = (int)p.gather.size();
     out->staged_load_bytes = p.direct_load_bytes;
     out->staged_store_bytes = p.direct_store_bytes;
+    out->race_checked = p.race_checked;
+    out->order_checked = p.order_checked;
+}
+
+// What a linked program does differently from the reference, said once at link time (WARN, the
+// default threshold).  The reference keeps its counting semaphores across executions and across
+// operations (zeroed only by resetSignals, csrc/engine_c.cc:576-593; a wait passes on any count
+// above zero, csrc/plugins/cuda/cuda_executor.cu:425-445): a notify nobody awaits would there be
+// carried into the next execution, here every execution starts from zero.
+void warn_about(const Program& p, const std::string& what, bool races_wanted) {
+    if (p.residual_signals != 0)
+        log_line(LOG_WARN, what + ": " + std::to_string(p.residual_signals) + " semaphore(s) are left above zero by one execution "
+                               "(a notify without a wait); the reference would carry those counts into the next execution, "
+                               "this executor starts every execution from zero");
+    if (!p.order_checked)
+        log_line(LOG_WARN, what + ": " + std::to_string(p.num_all_ops) + " ops are too many for the notify/wait ambiguity check and the "
+                               "data-race check; the pairing of one valid execution order is used unverified");
+    else if (races_wanted && !p.race_checked && p.ops.size() > 1)
+        log_line(LOG_WARN, what + ": the data-race check gave up (too many overlapping accesses); conflicting accesses are not verified to be ordered");
 }
 
 }  // namespace
@@ -219,6 +238,7 @@ int pccl_program_link(const pccl_graph* const* graphs, int num_vranks, pccl_prog
         for (int r = 0; r < num_vranks; ++r) gs.push_back(graphs[r] ? &graphs[r]->g : nullptr);
         auto p = std::make_unique<pccl_program>();
         p->p = link_program(gs, LinkOptions{});
+        warn_about(p->p, "linked program", true);
         *out = p.release();
         return 0;
     });
@@ -366,8 +386,22 @@ struct pccl_hip_ctx {
 
 namespace {
 
-void ensure_buffers(pccl_hip_ctx* ctx, size_t bytes) {
+bool is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
+}
+
+// Set-up work (linking, table uploads, growing the rank buffers) allocates and synchronises, which
+// would invalidate a capture in progress on the caller's stream: refuse instead.
+void refuse_setup_under_capture(hipStream_t s, const char* what) {
+    if (is_capturing(s))
+        throw Error{PCCL_ERR_INVALID, std::string("the stream is capturing and this call would have to ") + what +
+                                          ": execute the operation once outside the capture first"};
+}
+
+void ensure_buffers(pccl_hip_ctx* ctx, size_t bytes, hipStream_t stream) {
     if (bytes <= ctx->buf_bytes) return;
+    refuse_setup_under_capture(stream, "grow the engine's rank buffers");
     // every registered op aliases the same rank buffers (as in the reference, engine_c.cc:191-196)
     HIP_TRY(hipDeviceSynchronize());
     for (char*& b : ctx->bufs) { if (b) (void)hipFree(b); b = nullptr; }
@@ -381,8 +415,9 @@ void ensure_buffers(pccl_hip_ctx* ctx, size_t bytes) {
     ctx->buf_bytes = rounded;
 }
 
-void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
+void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, bool check_stream = false) {
     if (e.linked) return;
+    if (check_stream) refuse_setup_under_capture(stream, "link the operation and upload its plan tables");
     std::vector<const RankGraph*> gs;
     for (int r = 0; r < ctx->R; ++r) gs.push_back(e.graphs[r].get());
     LinkOptions opt;
@@ -489,6 +524,7 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e) {
     HIP_TRY(hipEventCreate(&e.ev0));
     HIP_TRY(hipEventCreate(&e.ev1));
     e.linked = true;
+    warn_about(P, "operation linked over " + std::to_string(ctx->R) + " virtual ranks", ctx->check_races);
     if (log_threshold() <= LOG_INFO)   // the reference's "Fused step executor enabled" line (engine_c.cc:357)
         log_line(LOG_INFO, "linked " + std::to_string(ctx->R) + " rank graphs: " + std::to_string(P.ops.size()) + " data ops on " +
                                std::to_string(P.num_levels) + " levels, " + std::to_string(P.num_items) + " work items of " +
@@ -519,7 +555,7 @@ int launch_levels(pccl_hip_ctx* ctx, OpEntry& e, const StepwiseLaunch& L, const 
             rc = launch_level(L, e.level_item_begin[l], e.level_item_begin[l + 1], ptrs, s);
         return rc;
     };
-    if (!ctx->level_graph || e.graph_failed || nlevels < 2) return launch_all(stream);
+    if (!ctx->level_graph || e.graph_failed || nlevels < 2 || is_capturing(stream)) return launch_all(stream);
 
     std::vector<char*> key(rank_bufs, rank_bufs + ctx->R);
     OpEntry::LevelGraph* hit = nullptr;
@@ -598,9 +634,7 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
             // The launch number is a kernel argument, which every replay of a recorded launch would
             // repeat (finding all flags of the previous replay set): on a capturing stream the
             // number comes from a device-side counter that a one-thread kernel advances first.
-            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-            const bool capturing = hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
-            L.epoch = capturing ? 0 : ++e.epoch;
+            L.epoch = is_capturing(stream) ? 0 : ++e.epoch;
             L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
             rc = launch_persistent(L, ptrs, stream);   // sizes the grid to what is resident at once
             e.ran_persistent = true;
@@ -700,7 +734,7 @@ void run_staged(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
     else need = std::max(need, in_bytes);
     if (ct == "alltoall") need = std::max(need, 2 * in_bytes);
     else if (ct != "reduce_scatter") need = std::max(need, out_bytes);
-    ensure_buffers(ctx, need);
+    ensure_buffers(ctx, need, s);
 
     RankPtrs src{}, dst{}, bufp{};
     StageOffsets off{};
@@ -892,8 +926,8 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
         std::lock_guard<std::mutex> lock(ctx->mu);
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
-        link_entry(ctx, e);
         hipStream_t s = (hipStream_t)stream;
+        link_entry(ctx, e, s, true);
         for (int r = 0; r < ctx->R; ++r)
             if (!inputs[r] || !outputs[r]) return fail(PCCL_ERR_INVALID, "null tensor for virtual rank " + std::to_string(r));
         // on the caller's tensors where the program allows it, else through the rank buffers
@@ -913,8 +947,8 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
         std::lock_guard<std::mutex> lock(ctx->mu);
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
-        link_entry(ctx, e);
         hipStream_t s = (hipStream_t)stream;
+        link_entry(ctx, e, s, true);
         {
             TraceRange exe(ctx->trace_ranges, "execute");
             run_program(ctx, e, (char* const*)bufs, buf_bytes, s);

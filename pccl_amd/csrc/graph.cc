@@ -255,6 +255,20 @@ RankGraph graph_from_triggers(const pccl_trigger* trig, const pccl_primitive_met
         o.off0 = trig[i].offset_0; o.off1 = trig[i].offset_1; o.off2 = trig[i].offset_2;
         o.size = trig[i].size;
         o.redop = PCCL_SUM;  // the reference runtime has no other operator
+        // the same ranges the JSON loader enforces: a negative offset or size would make the
+        // kernels address memory in front of a rank buffer
+        if (o.kind == OpKind::Reduce || o.kind == OpKind::Copy) {
+            const std::string where = "op " + std::to_string(i) + ": ";
+            if (o.off0 < 0 || o.off1 < 0 || o.size < 0 || (o.kind == OpKind::Reduce && o.off2 < 0))
+                throw Error{PCCL_ERR_PARSE, where + "negative offset or size in a data trigger"};
+            const int64_t reach = std::max(o.off0, std::max(o.off1, o.kind == OpKind::Reduce ? o.off2 : 0)) + o.size;
+            if (reach > INT32_MAX)
+                throw Error{PCCL_ERR_PARSE, where + "offset + size out of the 32-bit element range"};
+            if (o.kind == OpKind::Copy) o.off2 = 0;   // unused by copies: whatever the array held there
+        } else if (o.kind == OpKind::Notify || o.kind == OpKind::Wait) {
+            if (o.off0 < 0 || o.off0 >= PCCL_HIP_NUM_SIGNALS)
+                throw Error{PCCL_ERR_PARSE, "op " + std::to_string(i) + ": signal_id " + std::to_string(o.off0) + " outside 0.." + std::to_string(PCCL_HIP_NUM_SIGNALS - 1)};
+        }
         o.channel = meta[i].channel;
         if (o.channel < 0 || o.channel >= PCCL_HIP_MAX_CHANNELS) throw Error{PCCL_ERR_PARSE, "channel out of range"};
         o.num_deps_declared = meta[i].num_dependencies;

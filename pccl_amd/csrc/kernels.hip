@@ -8,6 +8,8 @@
 // float sum of two 8-bit-significand values is exact or rounds innocuously (24 >= 2*8+2).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "kernels.h"
 
 namespace pccl_hip {
@@ -872,23 +874,28 @@ __global__ __launch_bounds__(kThreads) void column_slot_kernel(ColumnLaunch L, R
 
 // ------------------------------------------------------------------------------- launchers
 
-static int g_cu_count[16] = {0};
+// Per-device facts, queried once.  Contexts on different threads may ask at the same time: the
+// slots are atomics and every thread that finds one empty computes the same value.
+constexpr int kMaxDevices = 16;
+static std::atomic<int> g_cu_count[kMaxDevices];
+
+static int current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    return dev;
+}
 
 int device_cu_count(int device) {
-    if (device < 0 || device >= 16) device = 0;
-    if (!g_cu_count[device]) {
-        int n = 0;
+    if (device < 0 || device >= kMaxDevices) device = 0;
+    int n = g_cu_count[device].load(std::memory_order_relaxed);
+    if (!n) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
-        g_cu_count[device] = n;
+        g_cu_count[device].store(n, std::memory_order_relaxed);
     }
-    return g_cu_count[device];
+    return n;
 }
 
-static int current_cus() {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
-    return device_cu_count(dev);
-}
+static int current_cus() { return device_cu_count(current_device()); }
 
 // Run length of the tile-to-XCD mapping for a launch over `ntiles` tiles: kXcdRun, halved while the
 // launch is too small to give every XCD a whole run (small launches then start no idle workgroups).
@@ -947,8 +954,9 @@ static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, h
     // that, the bound from the vector registers it reports and what the runtime says.  (A form of
     // this kernel that needed 100 scalar registers fitted only 7 times per CU while the runtime's
     // estimate said 8: the grid was one workgroup per CU too large and waits expired.)
-    static int cached_per_cu = 0;   // per instantiation; the queries are made once
-    int per_cu = cached_per_cu;
+    static std::atomic<int> cached_per_cu[kMaxDevices];   // per instantiation and device; the queries are made once
+    const int dev = current_device();
+    int per_cu = cached_per_cu[dev].load(std::memory_order_relaxed);
     if (per_cu == 0) {
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, persistent_kernel<DT>, kThreads, 0) != hipSuccess || per_cu <= 0) per_cu = 1;
         hipFuncAttributes attr;
@@ -958,7 +966,7 @@ static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, h
         }
         if (per_cu > 8) per_cu = 8;
         if (per_cu < 1) per_cu = 1;
-        cached_per_cu = per_cu;
+        cached_per_cu[dev].store(per_cu, std::memory_order_relaxed);
     }
     const int resident = current_cus() * per_cu;
     // Default: 4 workgroups per CU.  On the headline graph 3, 4 and 5 per CU take 3.05 to 3.07 ms,

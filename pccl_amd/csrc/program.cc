@@ -269,6 +269,7 @@ class Linker {
     // Reachability (happens-before) over all ops, in execution order.
     void build_reachability() {
         closure = (size_t)N <= kClosureLimit;
+        P.order_checked = closure;
         if (closure) {
             reach.assign(N, Bitset(N));
             for (int id : exec_order)
@@ -341,6 +342,7 @@ class Linker {
 
     // Conflicting accesses to one rank buffer must be ordered by some notify / wait chain.
     void check_races() {
+        if (opt.check_races && closure && D <= 1) P.race_checked = true;   // nothing to conflict with
         if (opt.check_races && closure && D > 1) {
             struct Acc { int rank; int64_t s, e; bool write; int op; };
             std::vector<Acc> acc;

@@ -71,7 +71,8 @@ struct Program {
     int residual_signals = 0;
     int64_t buffer_elems = 0;
     int64_t algorithmic_bytes = 0;
-    bool race_checked = false;
+    bool race_checked = false;    // the data-race check ran over every pair of conflicting accesses
+    bool order_checked = false;   // the notify / wait pairing was checked for ambiguity (skipped above kClosureLimit ops)
 
     // column plan (valid when position_aligned)
     bool position_aligned = false;

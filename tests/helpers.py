@@ -43,9 +43,12 @@ def pipelined_ring_allreduce(rank: int, world: int, n: int, dtype: str, depth: i
 
     paired_signals=False numbers the signals exactly as the reference's bandwidth script does
     (tests/bench_allreduce_tma_bw.py:119-186: one running counter over waits and notifies).  That
-    numbering makes step s+1 wait on an id nobody notifies; the reference's kernels get past such a
-    wait through their spin bail-out (cuda_executor.cu:946-961), exact semaphore semantics report a
-    deadlock.  paired_signals=True is the same schedule with the wait of step t+1 on the id step t
+    numbering makes step s+1 wait on an id nobody notifies.  The reference's wait spins until the
+    count is above zero and has no bail-out (cuda_executor.cu:946-961; only the other blocks'
+    channel barrier at :997-1003 gives up, after 4 M spins), so there the schedule can only finish
+    on counts that earlier executions left in the signal array, which is never cleared between
+    executions (engine_c.cc:576-593); exact semaphore semantics from zero report a deadlock.
+    paired_signals=True is the same schedule with the wait of step t+1 on the id step t
     of the previous rank notifies, which is executable."""
     chunk = n // world
     prev_rank, next_rank = (rank - 1) % world, (rank + 1) % world

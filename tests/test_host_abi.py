@@ -149,6 +149,42 @@ def test_graph_from_triggers_round_trip():
         assert bytes(trig[i])[:28] == bytes(t2[i])[:28]
 
 
+def test_trigger_arrays_are_range_checked_like_documents():
+    """The trigger path (what a DevicePlugin adapter hands over) refuses what the JSON path refuses:
+    negative offsets and sizes, ranges past 2^31 - 1 elements, signal ids outside the signal array.
+    Host only: such a graph must never reach a kernel."""
+    text = graph_jsons("ring", "build_allreduce", 2, 2048, "float32", "sm", 1)[0]
+    g = HostGraph.from_json(text)
+    meta, _ = g.meta()
+
+    def damaged(pick, **fields):
+        trig, n = g.triggers()
+        i = next(k for k in range(n) if pick(trig[k]))
+        for name, value in fields.items():
+            setattr(trig[i], name, value)
+        with pytest.raises(PcclError) as e:
+            HostGraph.from_triggers(trig, meta, "allreduce")
+        assert e.value.code == ERR_PARSE, str(e.value)
+        return str(e.value)
+
+    is_copy = lambda t: t.primitive_type == 6
+    is_reduce = lambda t: t.primitive_type == 1
+    is_signal = lambda t: t.primitive_type in (21, 22)
+    assert "negative" in damaged(is_copy, offset_1=-100000, size=1024)
+    assert "negative" in damaged(is_copy, offset_0=-1)
+    assert "negative" in damaged(is_copy, size=-5)
+    assert "negative" in damaged(is_reduce, offset_2=-16)
+    assert "32-bit element range" in damaged(is_copy, offset_1=2**31 - 1000, size=1024)
+    assert "32-bit element range" in damaged(is_reduce, offset_2=2**31 - 1, size=2)
+    assert "signal_id" in damaged(is_signal, offset_0=4096)
+    assert "signal_id" in damaged(is_signal, offset_0=-1)
+    # untouched arrays still load, and a copy's unused third offset is ignored
+    trig, n = g.triggers()
+    i = next(k for k in range(n) if is_copy(trig[k]))
+    trig[i].offset_2 = -7
+    assert HostGraph.from_triggers(trig, meta, "allreduce").num_ops == n
+
+
 # ------------------------------------------------------------------------------- fused steps
 
 def test_fused_steps_two_rank_ring():
@@ -313,15 +349,59 @@ def test_linker_rejects_partially_overlapping_in_place_op():
 
 def test_residual_signals_are_counted():
     jsons = _two_rank(lambda op, me, other: op.notify(signal_id=9, target_rank=other))   # never awaited
-    assert _link(jsons).info()["residual_signals"] == 2
+    info = _link(jsons).info()
+    assert info["residual_signals"] == 2
+    assert info["race_checked"] == 1 and info["order_checked"] == 1
+
+
+def test_linker_warns_where_an_execution_would_differ_from_the_reference():
+    """A notify without a wait leaves its semaphore above zero; the reference carries that count into
+    the next execution (signals are only zeroed by resetSignals, csrc/engine_c.cc:576-593, and a wait
+    passes on any count above zero, cuda_executor.cu:425-445), this executor starts from zero every
+    time: said at WARN level when the program is linked.  A balanced graph links silently.  A program
+    too large for the ambiguity and race checks says that they were skipped."""
+    import subprocess
+    import sys
+    code = ("import sys, json; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+            "from pccl_amd._lib import HostGraph, HostProgram\n"
+            "from pccl_amd.dsl import CommunicationOp, compile_to_json_string\n"
+            "from helpers import graph_jsons\n"
+            "def rank(me, other, extra):\n"
+            "    with CommunicationOp(name='r%%d' %% me) as op:\n"
+            "        op.tensor(dtype='float32', shape=(64,))\n"
+            "        op.notify(signal_id=1, target_rank=other); op.wait_notify(signal_id=1, source_rank=other)\n"
+            "        op.sm_copy(source_rank=other, src_offset=me * 32, dst_offset=me * 32, size=32)\n"
+            "        if extra: op.notify(signal_id=9, target_rank=other)\n"
+            "        return compile_to_json_string(op.get_graph())\n"
+            "which = sys.argv[1]\n"
+            "if which == 'big': js = graph_jsons('ring', 'build_allreduce', 64, 64 * 4 * 4, 'float32', 'sm', 4)\n"
+            "else: js = [rank(0, 1, which == 'unbalanced'), rank(1, 0, which == 'unbalanced')]\n"
+            "info = HostProgram([HostGraph.from_json(j) for j in js]).info()\n"
+            "print(info['residual_signals'], info['order_checked'], info['race_checked'])\n") % (ROOT, os.path.join(ROOT, "tests"))
+    env = {k: v for k, v in os.environ.items() if k != "PCCL_LOG_LEVEL"}
+
+    def run(which):
+        out = subprocess.run([sys.executable, "-c", code, which], env=env, capture_output=True, text=True, timeout=300)
+        assert out.returncode == 0, out.stderr
+        return out.stdout.split(), out.stderr
+
+    vals, err = run("unbalanced")
+    assert vals == ["2", "1", "1"]
+    assert "[pccl] [warning]" in err and "2 semaphore(s) are left above zero" in err and "reference would carry" in err
+    vals, err = run("balanced")
+    assert vals == ["0", "1", "1"] and "[pccl]" not in err
+    vals, err = run("big")     # 64 ranks x 4 channels: more ops than the quadratic checks take
+    assert vals[1:] == ["0", "0"]
+    assert "[pccl] [warning]" in err and "too many for the notify/wait ambiguity check" in err
 
 
 def test_reference_numbered_pipeline_schedule_is_reported_as_deadlock():
     """The pipelined ring of the reference's bandwidth script (tests/bench_allreduce_tma_bw.py:119-186)
     numbers waits and notifies with one running counter, so every wait after the first step is on
-    an id nobody notifies; the reference gets past it through the spin bail-out of its wait
-    (cuda_executor.cu:946-961).  Linked with exact semaphore semantics this is a deadlock, reported
-    at link time, by the product's linker and by the oracle alike."""
+    an id nobody notifies.  The reference's wait has no bail-out (cuda_executor.cu:946-961 spins
+    until the count is above zero), so it can only pass there on counts left over from earlier
+    executions.  Linked with exact semaphore semantics, every count starting at zero, this is a
+    deadlock, reported at link time, by the product's linker and by the oracle alike."""
     from helpers import pipelined_ring_allreduce, oracle_buffers, seeded_inputs
     from pccl_amd.dsl import compile_to_json_string
     world, n = 4, 4096
