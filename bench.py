@@ -1,25 +1,39 @@
 #!/usr/bin/env python3
-"""Headline benchmark: the 8-virtual-rank, 512 MB-per-rank bf16 ring-allreduce graph on one MI355X.
+"""Benchmark of the executor on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode auto|column|stepwise]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--mode auto|column|stepwise|persistent]
 
-A step is one execution of the compiled graph (448 data ops over 8 rank buffers resident in HBM),
-in place on the rank buffers, one launch of the column runner.  Prints ONE JSON line.
+The default (``--config c2``) is the headline: the 8-virtual-rank, 512 MiB-per-rank bf16 ring-allreduce
+graph (4 channels, 448 data ops), in place on 8 rank buffers resident in HBM.  A step is one
+execution of the compiled graph.  Prints ONE JSON line (``c4`` prints one per message size and
+collective).
 
-* value     algorithmic schedule bytes (reduce 3*n*esize, copy 2*n*esize, summed over the linked
-            program = 5*(R-1)*S) times K, divided by the wall time of the K timed steps
-* roofline  the same bytes divided by the average kernel duration measured with HIP events on the
-            launch stream (torch's current stream, which is the stream the C ABI launches on),
-            against the 8 TB/s HBM peak; `traffic` is the measured HBM bytes per launch from the
-            committed rocprofv3 counter summary when present
-* cpu_baseline  the CPU oracle (oracle/, OpenMP) executing the same graph shape on a bounded sample
-            on this box's host cores; a reported baseline, not the target
+* value      HBM bytes the step actually moves, divided by the wall time per step.  For the column
+             runner these are the bytes its plan loads and stores (every rank buffer read once and
+             written once: 16 S for the headline), which the committed rocprofv3 FETCH_SIZE /
+             WRITE_SIZE figures confirm; for the level and persistent runners every op moves its
+             full bytes, so the figure is the algorithmic byte count (5 (R-1) S).
+* roofline   the same bytes divided by the average kernel duration measured with HIP events on the
+             launch stream (torch's current stream, which is the stream the C ABI launches on),
+             against the 8 TB/s HBM peak.  ``traffic`` is the counter-measured figure of the
+             profile named in ``traffic_source`` (null where no profile covers the run).
+* algorithmic_equiv_GBps   the schedule's algorithmic bytes (reduce 3 n esize, copy 2 n esize over the
+             linked program) per second: what a runner that executes op by op would have to
+             sustain to be as fast.  Not an HBM rate.
+* cpu_baseline   the CPU oracle (oracle/, OpenMP) executing the same graph on this box's host
+             cores; a reported baseline, not the target
 
-Inputs: one CPU generator seeded 0; for rank r = 0..7, for slice s = 0..7, draw
-torch.randn(N/8) and cast to bf16 (rank-major, slice-major) — N(0,1) values as the configuration
+Other configurations: c3 = recursive halving-doubling allreduce, 16 ranks, 64 MiB f32, 2 channels;
+c4 = ring reduce_scatter and allgather, 8 ranks, fp16, 4 KB to 512 MB per rank as staged calls;
+c5 = binary-tree allreduce, 32 ranks, 96 MiB per rank, int32 SUM and f32 MAX (``--c5-dtype``), every
+op cut into 8 ragged pieces off 16-byte alignment.
+
+Headline inputs: one CPU generator seeded 0; for rank r = 0..7, for slice s = 0..7, draw
+torch.randn(N/8) and cast to bf16 (rank-major, slice-major) - N(0,1) values as the configuration
 prescribes, generated in slices to bound host memory.  The first execution is verified at full size
-before anything is timed: all ranks must hold bit-identical results and those must equal the
-ring's per-element reduction order evaluated with plain torch bf16 adds.
+before anything is timed: all ranks must hold bit-identical results, those must equal the ring's
+per-element reduction order evaluated with plain torch bf16 adds, and their sha256 must be the
+one the CPU oracle produced (tests/golden/headline_sha256.json).
 """
 from __future__ import annotations
 
@@ -33,32 +47,30 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-R = 8
-N = 268_435_456          # bf16 elements per rank = 512 MiB
-CHANNELS = 4
-DTYPE = "bfloat16"
 PEAK_GBPS = 8000.0
-WORKLOAD = "ring_allreduce_sum_R8_bf16_512MiB_per_rank_4ch"
+METRIC = "HBM GB/s & % of 8 TB/s peak (bytes read+written per second)"
 
 
 def log(msg: str) -> None:
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
-def build_graphs(n: int, channels: int):
-    from pccl_amd.dsl import RingAllreduce, compile_to_json_string
-    return [compile_to_json_string(RingAllreduce().build_allreduce(r, R, n, dtype=DTYPE, executor="sm",
-                                                                   num_channels=channels))
-            for r in range(R)]
+# ----------------------------------------------------------------------------------------- workloads
+
+def graphs(alg: str, method: str, world: int, n: int, dtype: str, channels: int, **ext):
+    from pccl_amd.dsl import ALGORITHMS, compile_to_json_string
+    a = ALGORITHMS[alg]()
+    return [compile_to_json_string(getattr(a, method)(r, world, n, dtype=dtype, executor="sm",
+                                                      num_channels=channels, **ext)) for r in range(world)]
 
 
-def make_inputs(n: int, device):
+def headline_inputs(n: int, world: int, device):
     import torch
     g = torch.Generator().manual_seed(0)
     slices = 8
     per = n // slices
     bufs = []
-    for r in range(R):
+    for _ in range(world):
         buf = torch.empty(n, dtype=torch.bfloat16, device=device)
         for s in range(slices):
             buf[s * per:(s + 1) * per] = torch.randn(per, generator=g).to(torch.bfloat16).to(device)
@@ -68,17 +80,18 @@ def make_inputs(n: int, device):
 
 def ring_expected(inputs, n: int, channels: int):
     """Ring order (chunk c of channel ch: acc = x_c; acc = x_(c+k) + acc, k = 1..R-1), each add
-    rounded to bf16, evaluated with torch's own bf16 add on the GPU."""
+    rounded to the storage type, evaluated with torch's own adds on the GPU."""
     import torch
+    world = len(inputs)
     per_ch = n // channels
-    per_rank = per_ch // R
+    per_rank = per_ch // world
     out = torch.empty_like(inputs[0])
     for ch in range(channels):
-        for c in range(R):
+        for c in range(world):
             lo = ch * per_ch + c * per_rank
             acc = inputs[c][lo:lo + per_rank].clone()
-            for k in range(1, R):
-                acc = inputs[(c + k) % R][lo:lo + per_rank] + acc
+            for k in range(1, world):
+                acc = inputs[(c + k) % world][lo:lo + per_rank] + acc
             out[lo:lo + per_rank] = acc
     return out
 
@@ -92,6 +105,102 @@ def sha256_of(t) -> str:
         h.update(flat[i:i + step].cpu().numpy().tobytes())
     return h.hexdigest()
 
+
+class Workload:
+    """One configuration: graphs, inputs, how to check a result, which profile measured its traffic."""
+
+    def __init__(self, key, name, world, n, dtype, jsons, make_inputs, check, traffic_stem=None, channels=1):
+        self.key, self.name, self.world, self.n, self.dtype = key, name, world, n, dtype
+        self.jsons, self.make_inputs, self.check, self.traffic_stem, self.channels = jsons, make_inputs, check, traffic_stem, channels
+
+
+def workload_c2(args, dev):
+    import torch
+    world, n, ch = 8, args.elems, args.channels
+    full = n == 268_435_456 and ch == 4
+
+    def make():
+        if args.gpu_inputs:
+            torch.manual_seed(0)
+            return [torch.randn(n, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(world)]
+        return headline_inputs(n, world, dev)
+
+    def check(pristine, bufs):
+        same = all(torch.equal(bufs[0].view(torch.int16), b.view(torch.int16)) for b in bufs[1:])
+        want = ring_expected(pristine, n, ch)
+        exact = torch.equal(want.view(torch.int16), bufs[0].view(torch.int16))
+        ref32 = sum(p[:1 << 20].float() for p in pristine)
+        rel = ((bufs[0][:1 << 20].float() - ref32).abs() / ref32.abs().clamp_min(1.0)).max().item()
+        v = {"ranks_identical": bool(same), "matches_ring_order_bf16": bool(exact),
+             "max_rel_err_vs_fp32_sum_first_1Mi": round(rel, 5), "output_sha256": sha256_of(bufs[0])}
+        ok = same and exact
+        golden_path = os.path.join(ROOT, "tests", "golden", "headline_sha256.json")
+        if full and not args.gpu_inputs and os.path.exists(golden_path):
+            golden = json.load(open(golden_path))
+            v["input_rank0_matches_committed_sha256"] = sha256_of(pristine[0]) == golden["input_sha256_per_rank"][0]
+            v["output_matches_committed_oracle_sha256"] = v["output_sha256"] == golden["output_sha256"]
+            ok = ok and v["input_rank0_matches_committed_sha256"] and v["output_matches_committed_oracle_sha256"]
+        return ok, v
+
+    name = "ring_allreduce_sum_R8_bf16_512MiB_per_rank_4ch" if full else f"ring_allreduce_sum_R8_bf16_{n}elems_per_rank_{ch}ch"
+    return Workload("c2", name, world, n, "bf16", graphs("ring", "build_allreduce", world, n, "bfloat16", ch), make, check,
+                    "ring_allreduce_R8_bf16_512MiB" if full else None, ch)
+
+
+def workload_c3(args, dev):
+    import torch
+    world, n = 16, 16_777_216
+
+    def make():
+        g = torch.Generator().manual_seed(0)
+        return [(torch.rand(n, generator=g) * 2 - 1).to(dev) for _ in range(world)]
+
+    def check(pristine, bufs):
+        same = all(torch.equal(bufs[0].view(torch.int32), b.view(torch.int32)) for b in bufs[1:])
+        # halving-doubling order: a balanced pairwise tree over the rank bits, low bit first
+        vals = [p.clone() for p in pristine]
+        k = 1
+        while k < world:
+            vals = [vals[r ^ k] + vals[r] if (r ^ k) > r else vals[r] + vals[r ^ k] for r in range(world)]
+            k <<= 1
+        exact = torch.equal(vals[0].view(torch.int32), bufs[0].view(torch.int32))
+        ref = torch.stack([p.double() for p in pristine]).sum(0)
+        rel = ((bufs[0].double() - ref).abs() / ref.abs().clamp_min(1.0)).max().item()
+        return same and exact and rel < 1e-6 * world, {"ranks_identical": bool(same), "matches_pairwise_order_f32": bool(exact),
+                                                     "max_rel_err_vs_f64_sum": float(f"{rel:.3g}"), "tolerance": 1e-6 * world}
+
+    return Workload("c3", "rhd_allreduce_sum_R16_f32_64MiB_per_rank_2ch", world, n, "f32",
+                    graphs("rhd", "build_allreduce", world, n, "float32", 2), make, check, "rhd_allreduce_R16_f32_64MiB", 2)
+
+
+def workload_c5(args, dev):
+    import torch
+    from pccl_amd.dsl import ragged_cuts
+    world, n = 32, 25_165_824
+    cuts = ragged_cuts(n, 8, seed=0)
+    is_int = args.c5_dtype == "int32"
+
+    def make():
+        g = torch.Generator().manual_seed(0)
+        if is_int:
+            return [torch.randint(-1000, 1000, (n,), generator=g, dtype=torch.int32).to(dev) for _ in range(world)]
+        return [torch.randn(n, generator=g).to(dev) for _ in range(world)]
+
+    def check(pristine, bufs):
+        want = torch.stack(pristine).sum(0, dtype=torch.int32) if is_int else torch.stack(pristine).amax(0)
+        ok = all(torch.equal(b.view(torch.int32), want.view(torch.int32)) for b in bufs)
+        return ok, {"every_rank_equals_" + ("int32_wrapping_sum" if is_int else "f32_max"): bool(ok)}
+
+    if is_int:
+        return Workload("c5", "tree_allreduce_sum_R32_int32_96MiB_per_rank_ragged8", world, n, "int32",
+                        graphs("tree", "build_allreduce", world, n, "int32", 1, reduce_op="sum", cuts=cuts), make, check,
+                        "tree_allreduce_R32_int32_sum_96MiB")
+    return Workload("c5", "tree_allreduce_max_R32_f32_96MiB_per_rank_ragged8", world, n, "f32",
+                    graphs("tree", "build_allreduce", world, n, "float32", 1, reduce_op="max", cuts=cuts), make, check,
+                    "tree_allreduce_R32_f32_max_96MiB")
+
+
+# ----------------------------------------------------------------------------------------- helpers
 
 def device_info(dev) -> dict:
     """Name, CU count and - best effort, from the driver's sysfs files - the current clocks and the
@@ -127,23 +236,27 @@ def device_info(dev) -> dict:
     return info
 
 
-def cpu_baseline(sample_elems: int, channels: int, reps: int = 3):
-    """Time the CPU oracle on the same graph shape at `sample_elems` elements per rank."""
+def cpu_baseline(jsons, world: int, sample_elems: int, np_dtype: str, label: str, reps: int = 3):
+    """Time the CPU oracle on the given graphs (`sample_elems` elements per rank)."""
     import numpy as np
     from oracle import oracle
-    graphs = [oracle.Graph(json.loads(j)) for j in build_graphs(sample_elems, channels)]
+    gs = [oracle.Graph(json.loads(j)) for j in jsons]
     rng = np.random.default_rng(0)
     threads = os.cpu_count() or 1
     env = os.environ.get("OMP_NUM_THREADS")
     if env and env.isdigit():
         threads = int(env)
-    # first touch by filling; bf16 bit patterns of N(0,1)-like magnitudes
-    bufs = [(rng.integers(0x3C00, 0x4000, sample_elems, dtype=np.uint16)) for _ in range(R)]
-    stats = oracle.run(graphs, bufs, threads=threads)      # warm-up
+    if np_dtype == "uint16":     # bf16 / f16 bit patterns of N(0,1)-like magnitudes; first touch by filling
+        bufs = [rng.integers(0x3C00, 0x4000, sample_elems, dtype=np.uint16) for _ in range(world)]
+    elif np_dtype == "int32":
+        bufs = [rng.integers(-1000, 1000, sample_elems, dtype=np.int32) for _ in range(world)]
+    else:
+        bufs = [rng.standard_normal(sample_elems, dtype=np.float32) for _ in range(world)]
+    stats = oracle.run(gs, bufs, threads=threads)      # warm-up
     times = []
     for _ in range(reps):
         t0 = time.perf_counter()
-        stats = oracle.run(graphs, bufs, threads=threads)
+        stats = oracle.run(gs, bufs, threads=threads)
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
@@ -155,68 +268,79 @@ def cpu_baseline(sample_elems: int, channels: int, reps: int = 3):
         pass
     return {"value": round(stats.bytes / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "cpu_model": model, "host_cpus_visible": os.cpu_count(),
-            "sample": f"same ring graph (R={R}, {channels} channels, bf16) at {sample_elems} elements "
-                      f"per rank ({sample_elems * 2 >> 20} MiB), {stats.bytes} algorithmic bytes, median of "
-                      f"{reps} runs after 1 warm-up, {med * 1e3:.1f} ms"}
+            "sample": f"{label} at {sample_elems} elements per rank, {stats.bytes} algorithmic bytes (every op moves its "
+                      f"full bytes on the CPU), median of {reps} runs after 1 warm-up, {med * 1e3:.1f} ms"}
 
 
-def measured_traffic(mode: str, levels: int):
-    """HBM bytes per execution of the headline graph from the committed rocprofv3 counter summaries
-    (FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy): one launch of the column kernel, or one launch
-    per dependency level of the level kernel."""
-    if mode == "persistent":
-        return None
-    kernel = "level_kernel" if mode == "stepwise" else "column_slot_kernel"
-    path = os.path.join(ROOT, "profiles", f"{kernel}_ring_allreduce_R8_bf16_512MiB.traffic.json")
+def committed_traffic(kernel: str, stem: str | None):
+    """HBM bytes per launch from the committed rocprofv3 counter summary of `kernel` on the workload
+    `stem` (FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy), with the file it comes from."""
+    if not stem:
+        return None, None
+    rel = os.path.join("profiles", f"{kernel}_{stem}.traffic.json")
     try:
-        with open(path) as f:
-            per_launch = json.load(f).get("hbm_bytes_per_launch")
+        with open(os.path.join(ROOT, rel)) as f:
+            return json.load(f).get("hbm_bytes_per_launch"), rel
     except (OSError, ValueError):
-        return None
-    if per_launch is None:
-        return None
-    return per_launch * levels if mode == "stepwise" else per_launch
+        return None, None
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--mode", default="auto")
-    ap.add_argument("--elems", type=int, default=N, help="elements per rank (default: the headline size)")
-    ap.add_argument("--channels", type=int, default=CHANNELS)
-    ap.add_argument("--vecs-per-thread", type=int, default=0)
-    ap.add_argument("--num-blocks", type=int, default=-1)
-    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
-                    help="engine option to set before the run (e.g. lds_slots=0, slot_threads=128); repeatable")
-    ap.add_argument("--rank-skew-bytes", type=int, default=0,
-                    help="carve the rank buffers out of one allocation, each this many bytes further in than its size")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-verify", action="store_true")
-    ap.add_argument("--gpu-inputs", action="store_true",
-                    help="draw the inputs with the GPU generator (tuning sweeps only; not the prescribed inputs)")
-    ap.add_argument("--cpu-sample-elems", type=int, default=N)
-    ap.add_argument("--cpu-reps", type=int, default=60)
-    ap.add_argument("--calibrate-copy-bytes", type=int, default=0,
-                    help="also launch the library's plain copy kernel on this many bytes (3 times): a "
-                         "known-traffic reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU: the R ranks are virtual ranks resident in one "
-              "MI355X's HBM and no multi-GPU path exists; run with --gpus 1", file=sys.stderr)
-        return 2
-
+def timed_inplace(eng, name, bufs, steps, warmup):
+    """K timed executions in place: wall time per step and per-launch HIP-event times."""
     import torch
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the executor has no CPU fallback", file=sys.stderr)
-        return 1
-    from pccl_amd.engine import Engine
+    for _ in range(warmup):
+        eng.execute_inplace(name, bufs)
+    torch.cuda.synchronize()
+    ev0 = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ev1 = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev0[i].record()
+        eng.execute_inplace(name, bufs)
+        ev1[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall * 1e3 / steps, [a.elapsed_time(b) for a, b in zip(ev0, ev1)]
 
-    n, channels = args.elems, args.channels
-    dev = torch.device("cuda", 0)
-    eng = Engine(R, 0)
-    for r, text in enumerate(build_graphs(n, channels)):
+
+def moved_bytes(info: dict, mode: str, staged: bool = False):
+    """HBM bytes one execution moves, by what kind of runner executes it."""
+    if mode in ("stepwise", "persistent") or not info["position_aligned"]:
+        return info["algorithmic_bytes"], "algorithmic bytes: every op moves its full bytes in this mode"
+    if staged and info["staged_load_bytes"] + info["staged_store_bytes"] > 0:
+        return info["staged_load_bytes"] + info["staged_store_bytes"], "bytes the column plan of the staged call loads and stores"
+    return info["column_load_bytes"] + info["column_store_bytes"], "bytes the column plan loads and stores"
+
+
+def side_leg(eng, name, bufs, mode, reps, alg_bytes):
+    import torch
+    eng.set_option("mode", mode)
+    for _ in range(2):
+        eng.execute_inplace(name, bufs)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        eng.execute_inplace(name, bufs)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    if mode == "persistent":
+        eng.sync_operation(name)      # would raise if a bounded wait had expired
+    eng.set_option("mode", "auto")
+    rate = alg_bytes / (ms * 1e-3) / 1e9
+    return {"mode": mode, "ms_per_step": round(ms, 4), "GB/s": round(rate, 1), "frac_of_hbm_peak": round(rate / PEAK_GBPS, 4),
+            "note": "HBM traffic equals the algorithmic bytes in this mode: every op moves its full bytes"}
+
+
+# ----------------------------------------------------------------------------------------- in-place configurations
+
+def run_inplace(args, wl: Workload, dev) -> int:
+    import torch
+    from pccl_amd.engine import Engine
+    eng = Engine(wl.world, 0)
+    for r, text in enumerate(wl.jsons):
         eng.register_operation_json("bench", text, r)
     eng.set_option("mode", args.mode)
     if args.vecs_per_thread:
@@ -231,24 +355,9 @@ def main() -> int:
     log(f"program: {info}")
 
     t0 = time.perf_counter()
-    if args.gpu_inputs:
-        torch.manual_seed(0)
-        pristine = [torch.randn(n, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(R)]
-    else:
-        pristine = make_inputs(n, dev)
+    pristine = wl.make_inputs()
     log(f"inputs generated in {time.perf_counter() - t0:.1f} s")
-    if args.rank_skew_bytes:
-        # rank buffers carved out of one allocation, rank r starting r * (size + skew) bytes in: the
-        # same position of different ranks then falls on different memory channels
-        stride = n + args.rank_skew_bytes // 2
-        arena = torch.empty(R * stride, dtype=torch.bfloat16, device=dev)
-        bufs = [arena[r * stride:r * stride + n] for r in range(R)]
-        for b, p in zip(bufs, pristine):
-            b.copy_(p)
-        log("rank buffer addresses: " + " ".join(hex(b.data_ptr()) for b in bufs))
-    else:
-        bufs = [p.clone() for p in pristine]
-        log("rank buffer addresses: " + " ".join(hex(b.data_ptr()) for b in bufs))
+    bufs = [p.clone() for p in pristine]
 
     # the first execution in the process (tables just uploaded, nothing of the buffers in any cache)
     c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -260,24 +369,9 @@ def main() -> int:
 
     verify = {}
     if not args.no_verify:
-        same = all(torch.equal(bufs[0].view(torch.int16), b.view(torch.int16)) for b in bufs[1:])
-        want = ring_expected(pristine, n, channels)
-        exact = torch.equal(want.view(torch.int16), bufs[0].view(torch.int16))
-        ref32 = sum(p[:1 << 20].float() for p in pristine)
-        rel = ((bufs[0][:1 << 20].float() - ref32).abs() / ref32.abs().clamp_min(1.0)).max().item()
-        verify = {"ranks_identical": bool(same), "matches_ring_order_bf16": bool(exact),
-                  "max_rel_err_vs_fp32_sum_first_1Mi": round(rel, 5), "output_sha256": sha256_of(bufs[0])}
-        # at the headline size with the prescribed inputs: the hashes committed with the tests (the
-        # output hash is what the CPU oracle computes at full size, tests/golden/make_headline_sha256.py)
-        golden_path = os.path.join(ROOT, "tests", "golden", "headline_sha256.json")
-        if n == N and channels == CHANNELS and not args.gpu_inputs and os.path.exists(golden_path):
-            golden = json.load(open(golden_path))
-            verify["input_rank0_matches_committed_sha256"] = sha256_of(pristine[0]) == golden["input_sha256_per_rank"][0]
-            verify["output_matches_committed_oracle_sha256"] = verify["output_sha256"] == golden["output_sha256"]
-            exact = exact and verify["input_rank0_matches_committed_sha256"] and verify["output_matches_committed_oracle_sha256"]
+        ok, verify = wl.check(pristine, bufs)
         log(f"verify: {verify}")
-        del want
-        if not (same and exact):
+        if not ok:
             print(json.dumps({"error": "verification failed", **verify}))
             return 1
         for b, p in zip(bufs, pristine):
@@ -292,117 +386,188 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        eng.execute_inplace("bench", bufs)
-    torch.cuda.synchronize()
-    ev0 = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ev1 = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        ev0[i].record()
-        eng.execute_inplace("bench", bufs)
-        ev1[i].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kern_ms = [a.elapsed_time(b) for a, b in zip(ev0, ev1)]
+    ms_per_step, kern_ms = timed_inplace(eng, "bench", bufs, args.steps, args.warmup)
     avg_ms = sum(kern_ms) / len(kern_ms)
-    ms_per_step = wall * 1e3 / args.steps
-    value = alg_bytes / (ms_per_step * 1e-3) / 1e9
-    achieved = alg_bytes / (avg_ms * 1e-3) / 1e9
+    hbm_bytes, hbm_note = moved_bytes(info, args.mode)
+    value = hbm_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = hbm_bytes / (avg_ms * 1e-3) / 1e9
+    reps = max(3, args.steps // 4)
 
     # end to end the reference's way: input and output staging copies included
-    outs = [torch.empty_like(p) for p in pristine]
-    eng.execute_operation("bench", pristine, outs)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    reps = max(3, args.steps // 4)
-    for _ in range(reps):
-        eng.execute_operation_async("bench", pristine, outs)
-    e1.record()
-    torch.cuda.synchronize()
-    staged_ms = e0.elapsed_time(e1) / reps
-    del outs
-
-    # the same graph op by op (one launch per dependency level, every op moving its full bytes)
-    op_by_op = None
-    if args.mode == "auto":
-        eng.set_option("mode", "stepwise")
-        for _ in range(2):
-            eng.execute_inplace("bench", bufs)
+    staged = None
+    if wl.key == "c2":
+        outs = [torch.empty_like(p) for p in pristine]
+        eng.execute_operation("bench", pristine, outs)
         torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
-            eng.execute_inplace("bench", bufs)
+            eng.execute_operation_async("bench", pristine, outs)
         e1.record()
         torch.cuda.synchronize()
-        sw_ms = e0.elapsed_time(e1) / reps
-        eng.set_option("mode", "auto")
-        op_by_op = {"mode": "stepwise", "ms_per_step": round(sw_ms, 4), "GB/s": round(alg_bytes / (sw_ms * 1e-3) / 1e9, 1),
-                    "frac_of_hbm_peak": round(alg_bytes / (sw_ms * 1e-3) / 1e9 / PEAK_GBPS, 4),
-                    "note": "HBM traffic equals the algorithmic bytes in this mode (profiles/level_kernel_*.md)"}
+        staged_ms = e0.elapsed_time(e1) / reps
+        del outs
+        sb, _ = moved_bytes(info, args.mode, staged=True)
+        staged = {"ms_per_call": round(staged_ms, 4), "hbm_GB/s": round(sb / (staged_ms * 1e-3) / 1e9, 1),
+                  "note": "the reference's call shape (separate input and output tensors per rank, execute_operation_async); "
+                          "in column mode the staging copies are fused into the program, so this is again one launch"}
 
-    # and as one persistent launch whose workgroups order themselves through device-side flags
-    persistent = None
-    if args.mode == "auto":
-        eng.set_option("mode", "persistent")
-        for _ in range(2):
-            eng.execute_inplace("bench", bufs)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            eng.execute_inplace("bench", bufs)
-        e1.record()
-        torch.cuda.synchronize()
-        pm_ms = e0.elapsed_time(e1) / reps
-        eng.sync_operation("bench")      # would raise if a bounded wait had expired
-        eng.set_option("mode", "auto")
-        persistent = {"mode": "persistent", "ms_per_step": round(pm_ms, 4), "GB/s": round(alg_bytes / (pm_ms * 1e-3) / 1e9, 1),
-                      "frac_of_hbm_peak": round(alg_bytes / (pm_ms * 1e-3) / 1e9 / PEAK_GBPS, 4),
-                      "note": "one launch for the whole graph, every op moving its full bytes, ordering by device-side flags (one per work item, one ready word per op)"}
+    # the same graph op by op (one launch per dependency level), and as one persistent launch whose
+    # workgroups order themselves through device-side flags
+    op_by_op = persistent = None
+    if args.mode == "auto" and not args.no_side_legs:
+        op_by_op = side_leg(eng, "bench", bufs, "stepwise", reps, alg_bytes)
+        persistent = side_leg(eng, "bench", bufs, "persistent", reps, alg_bytes)
+        persistent["note"] += "; one launch for the whole graph, ordering by device-side flags (one per work item, one ready word per op)"
 
-    default_runner = not any(kv.split("=")[0] in ("lds_slots", "slot_threads", "slot_direct") for kv in args.option)
-    traffic = measured_traffic(args.mode, info["num_levels"]) if (n == N and channels == CHANNELS and default_runner) else None
+    default_runner = not any(kv.split("=")[0].startswith(("lds_slots", "slot_")) for kv in args.option)
+    column = args.mode in ("auto", "column") and info["position_aligned"]
+    kernel = "column_slot_kernel" if column else "level_kernel" if args.mode == "stepwise" else "persistent_kernel"
+    traffic, traffic_source = committed_traffic(kernel, wl.traffic_stem) if default_runner else (None, None)
+    if traffic is not None and kernel == "level_kernel":
+        traffic *= info["num_levels"]      # the profile gives one launch; an execution is one launch per level
     result = {
-        "metric": "HBM GB/s (algorithmic schedule bytes read+written per second), 8-vrank 512MB bf16 ring allreduce graph",
+        "metric": METRIC + ", " + ("8-vrank 512MB bf16 ring allreduce graph" if wl.key == "c2" else wl.name),
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": WORKLOAD if (n == N and channels == CHANNELS) else
-                   f"ring_allreduce_sum_R8_bf16_{n}elems_per_rank_{channels}ch",
-                   "virtual_ranks": R, "bytes_per_rank": n * 2, "channels": channels, "data_ops": info["num_data_ops"],
-                   "algorithmic_bytes_per_step": alg_bytes, "mode": args.mode, "in_place": True},
+        "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
+        "config": {"workload": wl.name, "virtual_ranks": wl.world, "bytes_per_rank": wl.n * (2 if wl.dtype in ("bf16", "f16") else 4),
+                   "channels": wl.channels, "data_ops": info["num_data_ops"], "algorithmic_bytes_per_step": alg_bytes,
+                   "hbm_bytes_per_step": hbm_bytes, "mode": args.mode, "in_place": True},
         "pct_of_hbm_peak": round(100 * value / PEAK_GBPS, 1),
+        "algorithmic_equiv_GBps": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_GBPS, 4), "traffic": traffic,
+                     "frac": round(achieved / PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                     "bytes_counted": hbm_note, "kernel": kernel,
                      "kernel_ms_avg": round(avg_ms, 4), "kernel_ms_min": round(min(kern_ms), 4),
                      "kernel_ms_median": round(sorted(kern_ms)[len(kern_ms) // 2], 4),
                      "kernel_ms_first_execution": round(cold_ms, 4),
                      "planned_load_bytes": info["column_load_bytes"], "planned_store_bytes": info["column_store_bytes"]},
-        "end_to_end_staged": {"ms_per_call": round(staged_ms, 4), "GB/s": round(alg_bytes / (staged_ms * 1e-3) / 1e9, 1),
-                              "note": "the reference's call shape (separate input and output tensors per rank, execute_operation_async); "
-                                      "the staging copies are fused into the program, so this is again one launch"},
+        "end_to_end_staged": staged,
         "op_by_op": op_by_op,
         "single_launch_flag_ordered": persistent,
         "device": device_info(dev),
         "verify": verify,
     }
-    if result["roofline"]["frac"] > 1:
-        result["roofline"]["note"] = ("achieved counts the schedule's algorithmic bytes (35 S); the column runner executes "
-                                      "the same ops with 16 S of HBM traffic (forwarded values and re-read partial results "
-                                      "stay in registers and LDS), so hbm_frac, not frac, is the memory system's utilisation")
+    if traffic:
+        result["roofline"]["traffic_vs_counted"] = round(traffic / hbm_bytes, 4)
     if args.gpu_inputs:
         result["data"] = "synthetic (GPU generator: tuning run)"
-    if traffic:
-        result["roofline"]["hbm_frac"] = round(traffic / (avg_ms * 1e-3) / 1e9 / PEAK_GBPS, 4)
     if not args.no_cpu_baseline:
         del bufs, pristine
         torch.cuda.empty_cache()
-        result["cpu_baseline"] = cpu_baseline(min(args.cpu_sample_elems, n), channels, args.cpu_reps)
+        np_dtype = "uint16" if wl.dtype in ("bf16", "f16") else "int32" if wl.dtype == "int32" else "float32"
+        result["cpu_baseline"] = cpu_baseline(wl.jsons, wl.world, wl.n, np_dtype, wl.name + ": the same graphs", args.cpu_reps)
     print(json.dumps(result))
     eng.close()
     return 0
+
+
+# ----------------------------------------------------------------------------------------- c4: message-size sweep
+
+def run_c4(args, dev) -> int:
+    """Ring reduce_scatter and allgather, 8 ranks, fp16, N(0, 0.1) inputs, 4 KB to 512 MB per rank,
+    as staged calls (the reference's call shape: separate input and output tensors).  One JSON line
+    per collective and size: latency per call and HBM rate; the knee is the result."""
+    import torch
+    from pccl_amd.engine import Engine
+    world = 8
+    sizes = [4096 * 4 ** k for k in range(9)] + [512 << 20]
+    if args.c4_bytes:
+        sizes = [int(s) for s in args.c4_bytes.split(",")]
+    g = torch.Generator(device="cuda").manual_seed(0)
+    for nbytes in sizes:
+        n = nbytes // 2
+        chunk = n // world
+        for method, in_elems, out_elems in (("build_reduce_scatter", n, chunk), ("build_allgather", chunk, n)):
+            eng = Engine(world, 0)
+            try:
+                jsons = graphs("ring", method, world, n, "float16", 1)
+                for r, j in enumerate(jsons):
+                    eng.register_operation_json("bench", j, r)
+                eng.set_option("mode", args.mode)
+                for kv in args.option:
+                    key, _, val = kv.partition("=")
+                    eng.set_option(key, val)
+                info = eng.op_info("bench")
+                x = [(torch.randn(in_elems, generator=g, device="cuda") * 0.1).half() for _ in range(world)]
+                outs = [torch.empty(out_elems, dtype=torch.float16, device="cuda") for _ in range(world)]
+                call = eng.prepare("bench", x, outs)
+                for _ in range(args.warmup):
+                    call()
+                torch.cuda.synchronize()
+                ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+                t0 = time.perf_counter()
+                for a, b in ev:
+                    a.record()
+                    call()
+                    b.record()
+                torch.cuda.synchronize()
+                wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+                ms = sorted(a.elapsed_time(b) for a, b in ev)
+                avg = sum(ms) / len(ms)
+                hbm, note = moved_bytes(info, args.mode, staged=True)
+                if args.mode in ("stepwise", "persistent"):
+                    hbm += 2 * world * (in_elems + out_elems)      # the two batched staging copies, read + write, 2 bytes per element
+                    note += " plus the input and output staging copies"
+                print(json.dumps({
+                    "metric": METRIC + f", ring {method[6:]} R8 fp16 staged call", "value": round(hbm / (wall_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                    "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True,
+                    "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+                    "config": {"workload": f"ring_{method[6:]}_R8_f16_{nbytes}B_per_rank", "virtual_ranks": world, "bytes_per_rank": nbytes,
+                               "channels": 1, "data_ops": info["num_data_ops"], "algorithmic_bytes_per_step": info["algorithmic_bytes"],
+                               "hbm_bytes_per_step": hbm, "mode": args.mode, "in_place": False},
+                    "latency_us_median": round(ms[len(ms) // 2] * 1e3, 2), "latency_us_min": round(ms[0] * 1e3, 2),
+                    "algorithmic_equiv_GBps": round(info["algorithmic_bytes"] / (wall_ms * 1e-3) / 1e9, 1),
+                    "roofline": {"bound": "hbm", "achieved": round(hbm / (avg * 1e-3) / 1e9, 1), "peak": PEAK_GBPS, "unit": "GB/s",
+                                 "frac": round(hbm / (avg * 1e-3) / 1e9 / PEAK_GBPS, 4), "traffic": None, "traffic_source": None,
+                                 "bytes_counted": note, "kernel_ms_avg": round(avg, 5)}}), flush=True)
+            finally:
+                eng.close()
+    return 0
+
+
+# ----------------------------------------------------------------------------------------- main
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--mode", default="auto")
+    ap.add_argument("--elems", type=int, default=268_435_456, help="c2: elements per rank (default: the headline size)")
+    ap.add_argument("--channels", type=int, default=4, help="c2: channels of the ring")
+    ap.add_argument("--c5-dtype", default="int32", choices=["int32", "float32"], help="c5: int32 SUM or float32 MAX")
+    ap.add_argument("--c4-bytes", default="", help="c4: comma-separated bytes per rank instead of the full sweep")
+    ap.add_argument("--vecs-per-thread", type=int, default=0)
+    ap.add_argument("--num-blocks", type=int, default=-1)
+    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
+                    help="engine option to set before the run (e.g. lds_slots=0, slot_threads=128); repeatable")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--no-side-legs", action="store_true", help="skip the op-by-op and single-launch legs of an auto-mode run")
+    ap.add_argument("--gpu-inputs", action="store_true",
+                    help="c2: draw the inputs with the GPU generator (tuning runs only; not the prescribed inputs)")
+    ap.add_argument("--cpu-reps", type=int, default=20)
+    ap.add_argument("--calibrate-copy-bytes", type=int, default=0,
+                    help="also launch the library's plain copy kernel on this many bytes (3 times): a "
+                         "known-traffic reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU: the R ranks are virtual ranks resident in one "
+              "MI355X's HBM and no multi-GPU path exists; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the executor has no CPU fallback", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda", 0)
+    if args.config == "c4":
+        return run_c4(args, dev)
+    wl = {"c2": workload_c2, "c3": workload_c3, "c5": workload_c5}[args.config](args, dev)
+    return run_inplace(args, wl, dev)
 
 
 if __name__ == "__main__":

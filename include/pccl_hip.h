@@ -231,7 +231,10 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * the output tensors directly instead of staging through the engine's rank buffers);
  * "lds_slots" = "1" | "0" (column runner keeps values it re-reads in per-thread LDS slots, so each
  * rank buffer is read and written at most once per position; "0" re-reads them through memory);
- * "slot_threads" = 0 | 64 | 128 | 256 (workgroup size of that runner, 0 = from the rank count);
+ * "slot_threads" = 0 | 64 | 128 | 256 | 512 | 1024 (workgroup size of that runner, 0 = from the rank count);
+ * "slot_vecs" = 0 | 1 | 2 | 4 (16-byte vectors per thread of that runner: a workgroup's tile is
+ * slot_threads x slot_vecs vectors of every rank; 0 = from the rank count); "slot_lds_kib" = 0..160
+ * (least LDS a workgroup of that runner asks for, which bounds the workgroups per CU; 0 = chosen);
  * "slot_direct" = "1" | "0" (first touches loaded straight into LDS, or through registers);
  * "level_graph" = "0" | "1" (the level runner launches level by level, or replays the launches of an
  * execution as one HIP graph captured per set of rank pointers);
@@ -242,6 +245,10 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * persistent runners; the marker library is loaded at run time and PCCL_ERR_UNSUPPORTED is returned
  * if there is none; the environment variable PCCL_TRACE_RANGES=1 sets it for new contexts). */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
+/* The current value of an option as text (the keys of pccl_hip_set_option, and "num_vranks"): what the
+ * environment switches PCCL_NUM_BLOCKS / PCCL_DISABLE_FUSED / PCCL_TRACE_RANGES left in a new context
+ * can be read back here.  No counterpart in the reference. */
+int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t cap);
 
 /* Engine::exeOp / exeOpAsync (reference csrc/engine_c.cc:269-560): for every virtual rank r copy
  * inputs[r] into rank buffer r (allgather: at r*in_bytes), run the program, copy the result to

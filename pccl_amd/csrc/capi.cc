@@ -320,10 +320,23 @@ struct OpEntry {
     DevBuf gather;                        // gather plan of an alltoall graph (DevGatherCopy records)
     int64_t gather_tiles = 0;
     int gather_copy_tiles = 0;            // > 0: every copy of the gather plan has this many tiles
+    // Linking has a host half (the program and the tables derived from it; no HIP call) and a device
+    // half (the tables uploaded: allocations and copies).  Inspection needs the first only; the
+    // second happens at the first execution, and not on a stream that is being captured.
+    bool host_linked = false;
+    struct HostTables {
+        std::vector<DevColSegment> segs, direct_segs;
+        std::vector<DevGatherCopy> gather;
+        std::vector<DevStepOp> step_ops;
+        std::vector<int32_t> item_op;
+    } host;
     DevBuf segs, direct_segs, instrs, pre, step_ops, step_deps, item_op, state;
     int64_t total_tiles = 0, direct_tiles = 0;
+    int seg_tiles = 0, direct_seg_tiles = 0;   // > 0: every segment of the plan has this many tiles
     int vecs_per_thread = 0;
     int slot_threads = 0;
+    int slot_vecs = 1;                    // slot runner: vectors per thread
+    int slot_lds_bytes = 0;               // slot runner: dynamic LDS per workgroup
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool timed = false;
     bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
@@ -352,10 +365,12 @@ struct OpEntry {
         if (ev1) (void)hipEventDestroy(ev1);
         ev0 = ev1 = nullptr;
         linked = false; timed = false;
+        host_linked = false; host = HostTables{};
     }
 };
 
 enum class Mode { Auto, Column, Stepwise, Persistent };
+constexpr size_t kMaxSlotLdsBytes = 160 * 1024;   // LDS of one gfx950 CU
 
 }  // namespace
 
@@ -374,6 +389,8 @@ struct pccl_hip_ctx {
     bool trace_ranges = false;            // emit profiler ranges around the stages of a call
     bool lds_slots = true;                // column runner keeps re-read values in LDS slots
     int slot_threads = 0;                 // slot runner workgroup size (0: chosen from the rank count)
+    int slot_vecs = 0;                    // slot runner vectors per thread (0: chosen from the rank count)
+    int slot_lds_kib = 0;                 // slot runner: least dynamic LDS a workgroup asks for (0: chosen), which bounds the workgroups per CU
     bool slot_direct = true;              // slot runner fetches first touches straight into LDS
     bool level_graph = false;             // level runner replays its launches as one HIP graph (measured:
                                           // no faster than launching level by level, so off by default)
@@ -415,9 +432,11 @@ void ensure_buffers(pccl_hip_ctx* ctx, size_t bytes, hipStream_t stream) {
     ctx->buf_bytes = rounded;
 }
 
-void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, bool check_stream = false) {
-    if (e.linked) return;
-    if (check_stream) refuse_setup_under_capture(stream, "link the operation and upload its plan tables");
+// Host half of linking: the program, the shape of the slot runner's workgroups, the tables as the
+// kernels read them.  No HIP call.
+void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
+    if (e.host_linked) return;
+    e.host = OpEntry::HostTables{};
     std::vector<const RankGraph*> gs;
     for (int r = 0; r < ctx->R; ++r) gs.push_back(e.graphs[r].get());
     LinkOptions opt;
@@ -441,11 +460,31 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, boo
         bool reads_back = false;
         for (const ColInstr& in : P.col_instrs)
             if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || (in.store & STORE_KIND) == 1) reads_back = true;
-        e.slot_threads = 0;
-        if (ctx->lds_slots && ctx->slot_threads > 0) e.slot_threads = ctx->slot_threads;
-        else if (ctx->lds_slots && (reads_back || ctx->R <= 16)) e.slot_threads = ctx->R <= 8 ? 256 : ctx->R <= 16 ? 128 : 64;
-        const int64_t tile_v = e.slot_threads > 0 ? e.slot_threads : 256 * (int64_t)e.vecs_per_thread;
-        auto device_segments = [&](const std::vector<ColSegment>& segs, int64_t* total) {
+        e.slot_threads = 0; e.slot_vecs = 1; e.slot_lds_bytes = 0;
+        if (ctx->lds_slots && (ctx->slot_threads > 0 || reads_back || ctx->R <= 16)) {
+            // Shape of a workgroup: threads x vectors per thread, and how much LDS it asks for.  One
+            // workgroup per CU (asking for more than half of the CU's 160 KiB) that holds 8 KiB of
+            // every rank is what the memory system likes best where that fits: 8 ranks 512 x 1,
+            // 16 ranks 256 x 2 (128 KiB of slots); 32 ranks 128 x 2 (4 KiB of every rank in 128 KiB),
+            // 64 ranks 128 x 1.  Few ranks keep small workgroups, several per CU.
+            const int R = ctx->R;
+            int threads = R <= 4 ? 256 : R <= 8 ? 512 : R <= 16 ? 256 : 128;
+            int vecs = R <= 4 ? 1 : R <= 8 ? 1 : R <= 32 ? 2 : 1;
+            int lds_kib = R <= 4 ? 0 : 96;
+            if (ctx->slot_threads > 0) { threads = ctx->slot_threads; if (ctx->slot_vecs == 0) vecs = 1; if (ctx->slot_lds_kib == 0) lds_kib = 0; }
+            if (ctx->slot_vecs > 0) vecs = ctx->slot_vecs;
+            if (ctx->slot_lds_kib > 0) lds_kib = ctx->slot_lds_kib;
+            if (!ctx->slot_direct) vecs = 1;
+            if (threads * vecs > 1024) throw Error{PCCL_ERR_INVALID, "slot runner: slot_threads x slot_vecs may not exceed 1024"};
+            const size_t need = (size_t)R * vecs * threads * 16;
+            if (need > kMaxSlotLdsBytes)
+                throw Error{PCCL_ERR_INVALID, "slot runner: " + std::to_string(R) + " ranks x " + std::to_string(vecs) + " vectors x " + std::to_string(threads) +
+                                                  " threads x 16 bytes exceed the " + std::to_string(kMaxSlotLdsBytes >> 10) + " KiB of LDS a workgroup may use"};
+            e.slot_threads = threads; e.slot_vecs = vecs;
+            e.slot_lds_bytes = (int)std::min<size_t>(std::max<size_t>(need, (size_t)lds_kib << 10), kMaxSlotLdsBytes);
+        }
+        const int64_t tile_v = e.slot_threads > 0 ? (int64_t)e.slot_threads * e.slot_vecs : 256 * (int64_t)e.vecs_per_thread;
+        auto device_segments = [&](const std::vector<ColSegment>& segs, int64_t* total, int* uniform) {
             std::vector<DevColSegment> ds(segs.size());
             int64_t tiles = 0;
             for (size_t i = 0; i < segs.size(); ++i) {
@@ -459,22 +498,27 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, boo
                 d.prog_start = s.prog_start; d.prog_len = s.prog_len;
                 d.pre_start = s.pre_start; d.pre_words = s.pre_words;
                 d.streaming = 1; d.pad_ = 0; d.bcast_mask = s.bcast_mask;
+                d.pre_mask = 0;
+                for (int w = 0; w < s.pre_words; ++w)
+                    for (int j = 0; j < 8; ++j) {
+                        const unsigned r = (unsigned)(P.col_pre[s.pre_start + w] >> (8 * j) & 0xFF);
+                        if (r != 0xFF) d.pre_mask |= 1ull << r;
+                    }
                 for (int k = 0; k < s.prog_len; ++k) {
                     const ColInstr& in = P.col_instrs[s.prog_start + k];
                     if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || (in.store & STORE_KIND) == 1) d.streaming = 0;
                 }
             }
             *total = tiles;
+            // all segments the same number of tiles?  (the kernels then compute the segment of a tile)
+            const int64_t per = ds.size() > 1 ? ds[1].first_tile : tiles;
+            bool same = per > 0 && tiles == per * (int64_t)ds.size() && tiles < ((int64_t)1 << 32) && per <= INT32_MAX;
+            for (size_t i = 0; i < ds.size() && same; ++i) same = ds[i].first_tile == (int64_t)i * per;
+            *uniform = same ? (int)per : 0;
             return ds;
         };
-        auto ds = device_segments(P.segs, &e.total_tiles);
-        e.segs.upload(ds.data(), ds.size() * sizeof(DevColSegment));
-        if (!P.direct_segs.empty()) {
-            auto dd = device_segments(P.direct_segs, &e.direct_tiles);
-            e.direct_segs.upload(dd.data(), dd.size() * sizeof(DevColSegment));
-        }
-        e.instrs.upload(P.col_instrs.data(), P.col_instrs.size() * sizeof(ColInstr));
-        e.pre.upload(P.col_pre.data(), P.col_pre.size() * sizeof(uint64_t));
+        e.host.segs = device_segments(P.segs, &e.total_tiles, &e.seg_tiles);
+        if (!P.direct_segs.empty()) e.host.direct_segs = device_segments(P.direct_segs, &e.direct_tiles, &e.direct_seg_tiles);
     }
     if (!P.gather.empty()) {
         std::vector<DevGatherCopy> gc(P.gather.size());
@@ -493,7 +537,7 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, boo
         bool same = per > 0 && tiles == per * (int64_t)gc.size() && tiles <= INT32_MAX;
         for (size_t i = 0; i < gc.size() && same; ++i) same = gc[i].first_tile == (int64_t)i * per;
         if (same) e.gather_copy_tiles = (int)per;
-        e.gather.upload(gc.data(), gc.size() * sizeof(DevGatherCopy));
+        e.host.gather = std::move(gc);
     }
     // stepwise plan
     {
@@ -514,16 +558,10 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, boo
         for (size_t k = 0; k < P.ops.size(); ++k)
             if (k == 0 || P.ops[k].level != P.ops[k - 1].level) e.level_item_begin.push_back(P.step_ops[k].first_item);
         e.level_item_begin.push_back((int)P.num_items);
-        e.step_ops.upload(so.data(), so.size() * sizeof(DevStepOp));
-        e.step_deps.upload(P.step_deps.data(), P.step_deps.size() * sizeof(int32_t));
-        e.item_op.upload(item_op.data(), item_op.size() * sizeof(int32_t));
-        std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * ((size_t)P.num_items + P.ops.size() + 1), 0);
-        e.state.upload(zeros.data(), zeros.size());
-        e.epoch = 0;
+        e.host.step_ops = std::move(so);
+        e.host.item_op = std::move(item_op);
     }
-    HIP_TRY(hipEventCreate(&e.ev0));
-    HIP_TRY(hipEventCreate(&e.ev1));
-    e.linked = true;
+    e.host_linked = true;
     warn_about(P, "operation linked over " + std::to_string(ctx->R) + " virtual ranks", ctx->check_races);
     if (log_threshold() <= LOG_INFO)   // the reference's "Fused step executor enabled" line (engine_c.cc:357)
         log_line(LOG_INFO, "linked " + std::to_string(ctx->R) + " rank graphs: " + std::to_string(P.ops.size()) + " data ops on " +
@@ -534,6 +572,31 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, boo
                                                                              : std::string("register runner"))
                                                    : std::string("not position aligned: level / persistent runner")) +
                                (P.gather.empty() ? "" : "; alltoall gather plan of " + std::to_string(P.gather.size()) + " copies"));
+}
+
+// Device half: upload the tables (allocations and copies, hence never on a capturing stream).
+void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, bool check_stream = false) {
+    if (e.linked) return;
+    if (check_stream) refuse_setup_under_capture(stream, "upload the operation's plan tables");
+    link_host(ctx, e);
+    const Program& P = e.prog;
+    const OpEntry::HostTables& h = e.host;
+    e.segs.upload(h.segs.data(), h.segs.size() * sizeof(DevColSegment));
+    e.direct_segs.upload(h.direct_segs.data(), h.direct_segs.size() * sizeof(DevColSegment));
+    if (P.position_aligned) {
+        e.instrs.upload(P.col_instrs.data(), P.col_instrs.size() * sizeof(ColInstr));
+        e.pre.upload(P.col_pre.data(), P.col_pre.size() * sizeof(uint64_t));
+    }
+    e.gather.upload(h.gather.data(), h.gather.size() * sizeof(DevGatherCopy));
+    e.step_ops.upload(h.step_ops.data(), h.step_ops.size() * sizeof(DevStepOp));
+    e.step_deps.upload(P.step_deps.data(), P.step_deps.size() * sizeof(int32_t));
+    e.item_op.upload(h.item_op.data(), h.item_op.size() * sizeof(int32_t));
+    std::vector<char> zeros(sizeof(StepState) + sizeof(int32_t) * ((size_t)P.num_items + P.ops.size() + 1), 0);
+    e.state.upload(zeros.data(), zeros.size());
+    e.epoch = 0;
+    HIP_TRY(hipEventCreate(&e.ev0));
+    HIP_TRY(hipEventCreate(&e.ev1));
+    e.linked = true;
 }
 
 OpEntry& find_entry(pccl_hip_ctx* ctx, const char* name) {
@@ -620,8 +683,8 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
         ColumnLaunch L{};
         L.segs = (const DevColSegment*)e.segs.p; L.num_segs = (int)P.segs.size();
         L.instrs = (const uint64_t*)e.instrs.p; L.pre = (const uint64_t*)e.pre.p;
-        L.slot_threads = e.slot_threads; L.num_ranks = ctx->R; L.slot_direct = ctx->slot_direct;
-        L.total_tiles = e.total_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
+        L.slot_threads = e.slot_threads; L.slot_vecs = e.slot_vecs; L.slot_lds_bytes = e.slot_lds_bytes; L.num_ranks = ctx->R; L.slot_direct = ctx->slot_direct;
+        L.total_tiles = e.total_tiles; L.seg_tiles = e.seg_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
         L.num_blocks = ctx->num_blocks;
         rc = launch_column(L, ptrs, stream);
     } else {
@@ -681,8 +744,8 @@ bool run_direct(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
     ColumnLaunch L{};
     L.segs = (const DevColSegment*)e.direct_segs.p; L.num_segs = (int)P.direct_segs.size();
     L.instrs = (const uint64_t*)e.instrs.p; L.pre = (const uint64_t*)e.pre.p;
-    L.slot_threads = e.slot_threads; L.num_ranks = ctx->R; L.slot_direct = ctx->slot_direct;
-    L.total_tiles = e.direct_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
+    L.slot_threads = e.slot_threads; L.slot_vecs = e.slot_vecs; L.slot_lds_bytes = e.slot_lds_bytes; L.num_ranks = ctx->R; L.slot_direct = ctx->slot_direct;
+    L.total_tiles = e.direct_tiles; L.seg_tiles = e.direct_seg_tiles; L.dtype = P.dtype; L.vecs_per_thread = e.vecs_per_thread;
     L.num_blocks = ctx->num_blocks;
     TraceRange exe(ctx->trace_ranges, "execute"), range(ctx->trace_ranges, "fused_kernel");
     int rc = launch_column(L, ptrs, stream);
@@ -805,7 +868,8 @@ int register_graph(pccl_hip_ctx* ctx, const char* name, int vrank, RankGraph&& g
     HIP_TRY(hipSetDevice(ctx->device));
     OpEntry& e = ctx->ops[name];
     if (e.graphs.empty()) e.graphs.resize(ctx->R);
-    if (e.linked) { HIP_TRY(hipDeviceSynchronize()); e.release(); }  // re-registration replaces the op
+    if (e.linked) HIP_TRY(hipDeviceSynchronize());
+    if (e.linked || e.host_linked) e.release();  // re-registration replaces the op
     e.graphs[vrank] = std::make_unique<RankGraph>(std::move(g));
     if (log_threshold() <= LOG_INFO)   // reference engine_c.cc:168,199
         log_line(LOG_INFO, std::string("operation '") + name + "' registered for virtual rank " + std::to_string(vrank) + ": " +
@@ -896,14 +960,25 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             int u = std::atoi(value);
             if (u != 1 && u != 2 && u != 4) return fail(PCCL_ERR_INVALID, "vecs_per_thread must be 1, 2 or 4");
             ctx->vecs_per_thread = u; relink = true;
-        } else if (k == "slot_direct") ctx->slot_direct = std::atoi(value) != 0;
+        } else if (k == "slot_direct") { ctx->slot_direct = std::atoi(value) != 0; relink = true; }
         else if (k == "level_graph") ctx->level_graph = std::atoi(value) != 0;
         else if (k == "lds_slots") { ctx->lds_slots = std::atoi(value) != 0; relink = true; }
         else if (k == "slot_threads") {
             int t = std::atoi(value);
-            if (t != 0 && t != 64 && t != 128 && t != 256) return fail(PCCL_ERR_INVALID, "slot_threads must be 0 (automatic), 64, 128 or 256");
-            if ((size_t)t * ctx->R * 16 > 64 * 1024) return fail(PCCL_ERR_INVALID, "slot_threads x ranks x 16 bytes exceeds the 64 KiB of LDS a workgroup may use");
+            if (t != 0 && t != 64 && t != 128 && t != 256 && t != 512 && t != 1024) return fail(PCCL_ERR_INVALID, "slot_threads must be 0 (automatic), 64, 128, 256, 512 or 1024");
+            if ((size_t)t * ctx->R * 16 * std::max(1, ctx->slot_vecs) > kMaxSlotLdsBytes) return fail(PCCL_ERR_INVALID, "slot_threads x slot_vecs x ranks x 16 bytes exceeds the 160 KiB of LDS a workgroup may use");
             ctx->slot_threads = t; relink = true;
+        }
+        else if (k == "slot_vecs") {
+            int v = std::atoi(value);
+            if (v != 0 && v != 1 && v != 2 && v != 4) return fail(PCCL_ERR_INVALID, "slot_vecs must be 0 (automatic), 1, 2 or 4");
+            if ((size_t)v * ctx->R * 16 * std::max(64, ctx->slot_threads) > kMaxSlotLdsBytes) return fail(PCCL_ERR_INVALID, "slot_threads x slot_vecs x ranks x 16 bytes exceeds the 160 KiB of LDS a workgroup may use");
+            ctx->slot_vecs = v; relink = true;
+        }
+        else if (k == "slot_lds_kib") {
+            int b = std::atoi(value);
+            if (b < 0 || b > 160) return fail(PCCL_ERR_INVALID, "slot_lds_kib must be 0 (automatic) to 160");
+            ctx->slot_lds_kib = b; relink = true;
         }
         else if (k == "step_tile_bytes") {
             int64_t b = std::atoll(value);
@@ -915,6 +990,35 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             HIP_TRY(hipDeviceSynchronize());
             for (auto& kv : ctx->ops) kv.second.release();
         }
+        return 0;
+    });
+}
+
+int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t cap) {
+    return guarded([&] {
+        if (!ctx || !key || !value || cap == 0) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        const std::string k = key;
+        std::string v;
+        if (k == "mode") v = ctx->mode == Mode::Auto ? "auto" : ctx->mode == Mode::Column ? "column" : ctx->mode == Mode::Stepwise ? "stepwise" : "persistent";
+        else if (k == "num_blocks") v = std::to_string(ctx->num_blocks);
+        else if (k == "timing") v = std::to_string((int)ctx->timing);
+        else if (k == "trace_ranges") v = std::to_string((int)ctx->trace_ranges);
+        else if (k == "fuse_staging") v = std::to_string((int)ctx->fuse_staging);
+        else if (k == "wait_timeout_ms") v = std::to_string(ctx->wait_timeout_ms);
+        else if (k == "check_races") v = std::to_string((int)ctx->check_races);
+        else if (k == "vecs_per_thread") v = std::to_string(ctx->vecs_per_thread);
+        else if (k == "slot_direct") v = std::to_string((int)ctx->slot_direct);
+        else if (k == "level_graph") v = std::to_string((int)ctx->level_graph);
+        else if (k == "lds_slots") v = std::to_string((int)ctx->lds_slots);
+        else if (k == "slot_threads") v = std::to_string(ctx->slot_threads);
+        else if (k == "slot_vecs") v = std::to_string(ctx->slot_vecs);
+        else if (k == "slot_lds_kib") v = std::to_string(ctx->slot_lds_kib);
+        else if (k == "step_tile_bytes") v = std::to_string(ctx->step_tile_bytes);
+        else if (k == "num_vranks") v = std::to_string(ctx->R);
+        else return fail(PCCL_ERR_INVALID, "unknown option '" + k + "'");
+        if (v.size() + 1 > cap) return fail(PCCL_ERR_INVALID, "value buffer too small");
+        std::memcpy(value, v.c_str(), v.size() + 1);
         return 0;
     });
 }
@@ -999,7 +1103,7 @@ int pccl_hip_op_info(pccl_hip_ctx* ctx, const char* name, pccl_program_info* out
         std::lock_guard<std::mutex> lock(ctx->mu);
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
-        link_entry(ctx, e);
+        link_host(ctx, e);      // inspection needs no device memory
         fill_info(e.prog, out);
         if (e.slot_threads > 0) {   // the traffic of the runner this context would launch
             out->column_load_bytes = e.prog.slot_load_bytes;

@@ -30,6 +30,7 @@ struct DevColSegment {
     int32_t streaming;       // 1: every load is a first touch and every live store is final
     int32_t pad_;
     uint64_t bcast_mask;     // ranks that receive the accumulator after the last instruction
+    uint64_t pre_mask;       // ranks the program reads by first touch (the pre list as a set)
 };
 
 struct DevStepOp {    // 64 bytes: one 16-dword scalar load
@@ -67,10 +68,13 @@ struct ColumnLaunch {
     int32_t vecs_per_thread;  // 1, 2 or 4 (register runner)
     int32_t num_blocks;       // 0: one workgroup per tile
     int32_t slot_threads;     // 0: register runner (re-read values go through memory);
-                              // 64, 128 or 256: workgroup size of the slot runner (re-read values in LDS)
+                              // 64 ... 1024: workgroup size of the slot runner (re-read values in LDS)
+    int32_t slot_vecs;        // slot runner: 16-byte vectors per thread (1, 2 or 4); a tile is slot_threads x slot_vecs vectors
+    int32_t slot_lds_bytes;   // slot runner: dynamic LDS of a workgroup (>= num_ranks x slot_vecs x slot_threads x 16)
     int32_t num_ranks;        // slot runner: LDS slots per thread
     int32_t slot_direct;      // slot runner: 1 = first touches are loaded straight into LDS
     int32_t xcd_run;          // run length of the tile-to-XCD mapping; filled in by the launcher
+    int32_t seg_tiles;        // > 0: every segment has this many tiles (segment = tile / seg_tiles, fewer than 2^32 tiles); 0: search
 };
 
 struct StepwiseLaunch {

@@ -154,11 +154,77 @@ __device__ __forceinline__ u32x4 vec_op_words(u32x4 a, u32x4 b, int redop) {
     return r;
 }
 
+// Sums of whole vectors take a shorter road than word_op: the arithmetic runs as if no NaN could
+// come out, one unordered compare per pair of results notes whether one did, and only lanes that
+// saw one go back and canonicalise (rare: the branch is skipped by the whole wave otherwise).
+// The results are those of word_op bit for bit.  bf16 rounds with v_cvt_pk_bf16_f32, which was
+// checked on this GPU against the integer form of bf16_round_hi for every non-NaN float.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+template <int DT>
+__device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
+    if constexpr (DT == PCCL_F32) {
+        const float r0 = as_f32(a.x) + as_f32(b.x), r1 = as_f32(a.y) + as_f32(b.y);
+        const float r2 = as_f32(a.z) + as_f32(b.z), r3 = as_f32(a.w) + as_f32(b.w);
+        u32x4 r = {as_u32(r0), as_u32(r1), as_u32(r2), as_u32(r3)};
+        if (__builtin_expect(__builtin_isunordered(r0, r1) | __builtin_isunordered(r2, r3), 0)) {
+            if (r0 != r0) r.x = 0x7FFFFFFFu;
+            if (r1 != r1) r.y = 0x7FFFFFFFu;
+            if (r2 != r2) r.z = 0x7FFFFFFFu;
+            if (r3 != r3) r.w = 0x7FFFFFFFu;
+        }
+        return r;
+    } else if constexpr (DT == PCCL_BF16) {
+        u32x4 r;
+        bool nan = false;
+        const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+        uint32_t rw[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = as_f32(aw[i] << 16) + as_f32(bw[i] << 16);
+            const float hi = as_f32(aw[i] & 0xFFFF0000u) + as_f32(bw[i] & 0xFFFF0000u);
+            nan |= __builtin_isunordered(lo, hi);
+            const f32x2 pair = {lo, hi};
+            rw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
+        }
+        if (__builtin_expect(nan, 0)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if ((rw[i] & 0x7FFFu) > 0x7F80u) rw[i] = (rw[i] & 0xFFFF0000u) | 0x7FFFu;
+                if ((rw[i] & 0x7FFF0000u) > 0x7F800000u) rw[i] = (rw[i] & 0x0000FFFFu) | 0x7FFF0000u;
+            }
+        }
+        r.x = rw[0]; r.y = rw[1]; r.z = rw[2]; r.w = rw[3];
+        return r;
+    } else if constexpr (DT == PCCL_F16) {
+        const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+        uint32_t rw[4];
+        bool nan = false;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const h2 s = __builtin_bit_cast(h2, aw[i]) + __builtin_bit_cast(h2, bw[i]);
+            nan |= __builtin_isunordered(s[0], s[1]);
+            rw[i] = __builtin_bit_cast(uint32_t, s);
+        }
+        if (__builtin_expect(nan, 0)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if ((rw[i] & 0x7FFFu) > 0x7C00u) rw[i] = (rw[i] & 0xFFFF0000u) | 0x7FFFu;
+                if ((rw[i] & 0x7FFF0000u) > 0x7C000000u) rw[i] = (rw[i] & 0x0000FFFFu) | 0x7FFF0000u;
+            }
+        }
+        u32x4 r = {rw[0], rw[1], rw[2], rw[3]};
+        return r;
+    } else {
+        return vec_op_words<DT>(a, b, PCCL_SUM);
+    }
+}
+
 // One decision on the operator per vector: each branch below inlines the word code with a
 // constant operator, so the four words run back to back without tests in between.
 template <int DT>
 __device__ __forceinline__ u32x4 vec_op(u32x4 a, u32x4 b, int redop) {
-    if (redop == PCCL_SUM) return vec_op_words<DT>(a, b, PCCL_SUM);
+    if (redop == PCCL_SUM) return vec_sum<DT>(a, b);
     if (redop == PCCL_MAX) return vec_op_words<DT>(a, b, PCCL_MAX);
     return vec_op_words<DT>(a, b, PCCL_MIN);
 }
@@ -743,6 +809,23 @@ __device__ __forceinline__ void column_edge_tile(const DevColSegment& seg, const
     }
 }
 
+// Which segment a tile belongs to (uniform).  When all segments have the same number of tiles - the
+// chunks of a ring, the halves of a halving-doubling schedule - that is a shift or a division;
+// otherwise a binary search over the segments' first tiles, log2 dependent table reads in front of
+// the workgroup's first load.
+__device__ __forceinline__ int find_segment(const ColumnLaunch& L, int64_t tile) {
+    if (L.seg_tiles > 0) {
+        const uint32_t per = (uint32_t)L.seg_tiles;
+        return (per & (per - 1)) == 0 ? (int)((uint32_t)tile >> __builtin_ctz(per)) : (int)((uint32_t)tile / per);
+    }
+    int lo = 0, hi = L.num_segs;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (as_const(L.segs)[mid].first_tile <= tile) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 template <int DT, int U>
 __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPtrs ptrs) {
     constexpr int ES = ElemBytes<DT>::value;
@@ -754,12 +837,7 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
     for (int64_t w = blockIdx.x; w < span_tiles(L.total_tiles, L.xcd_run); w += gridDim.x) {
         const int64_t tile = xcd_tile(w, L.xcd_run);
         if (tile >= L.total_tiles) continue;
-        // segment lookup (uniform)
-        int lo = 0, hi = L.num_segs;
-        while (hi - lo > 1) {
-            int mid = (lo + hi) >> 1;
-            if (as_const(L.segs)[mid].first_tile <= tile) lo = mid; else hi = mid;
-        }
+        const int lo = find_segment(L, tile);
         const DevColSegment seg = load_const(L.segs + lo);
         const int64_t vfirst = seg.first_vec + (tile - seg.first_tile) * TILE_V;
         const PCCL_CONST uint64_t* prog = as_const(L.instrs) + seg.prog_start;
@@ -788,87 +866,207 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
 // halving-doubling butterflies, trees).  A thread only ever touches its own slots, so no barrier
 // is needed.  Results are bit-identical to the op-by-op execution for the same reason as above.
 
+// Rank pointers without a memory access per use: lane l of every wave keeps the pointers of rank l
+// (the wave has 64 lanes and a context at most 64 ranks), and a uniform rank picks its pointer
+// with v_readlane.  Reading a pointer from the kernel arguments instead is a scalar load of its
+// own - a hundred cycles and more each time, in front of every first-touch load, every store and
+// every broadcast of a program, which a workgroup that has the CU to itself cannot hide.
+struct LanePtr {
+    uint32_t lo, hi;
+    __device__ __forceinline__ explicit LanePtr(const char* p) : lo((uint32_t)(uintptr_t)p), hi((uint32_t)((uintptr_t)p >> 32)) {
+        // The pointer arrives by a vector load.  Passing it through an empty asm makes the compiler
+        // wait for that load here, once; otherwise every use inside a loop that also issues memory
+        // operations is preceded by a wait for all of them (vmcnt(0)), which serialises the loop.
+        asm volatile("" : "+v"(lo), "+v"(hi));
+    }
+    __device__ __forceinline__ char* of(int rank) const {
+        const uint32_t l = __builtin_amdgcn_readlane(lo, rank), h = __builtin_amdgcn_readlane(hi, rank);
+        return reinterpret_cast<char*>((uintptr_t)l | (uintptr_t)h << 32);
+    }
+};
+static_assert(kMaxR == 64, "one lane per rank");
+
+// Slot (rank r, vector v) of thread t in a workgroup of T threads with V vectors per thread sits at
+// index (r * V + v) * T + t: consecutive lanes 16 bytes apart (conflict-free 128-bit accesses), and a
+// wave's 64 lanes form the contiguous 1 KiB block that one direct-to-LDS load fills.
 template <int N>
-__device__ __forceinline__ void slot_fetch(uint64_t word, const RankPtrs& ptrs, u32x4* slots, int T, int tid, int64_t off) {
-    u32x4 v[N];
+__device__ __forceinline__ void slot_fetch(uint64_t word, const RankPtrs& ptrs, u32x4* slots, int V, int v, int T, int tid, int64_t off) {
+    u32x4 x[N];
 #pragma unroll
-    for (int i = 0; i < N; ++i) v[i] = ldv_nt(ptrs.p[kMaxR + (int)((word >> (8 * i)) & 0xFF)] + off);
+    for (int i = 0; i < N; ++i) x[i] = ldv_nt(ptrs.p[kMaxR + (int)((word >> (8 * i)) & 0xFF)] + off);
 #pragma unroll
-    for (int i = 0; i < N; ++i) slots[(int)((word >> (8 * i)) & 0xFF) * T + tid] = v[i];
+    for (int i = 0; i < N; ++i) slots[((int)((word >> (8 * i)) & 0xFF) * V + v) * T + tid] = x[i];
 }
 
 // The same fetch without staging registers: a 128-bit load that the memory pipeline writes
 // straight into LDS (lane l of the wave lands at the wave-uniform LDS base + 16 l), so a thread
 // can have every first-touch load of its program in flight at once.
-__device__ __forceinline__ void slot_fetch_direct(int rank, const RankPtrs& ptrs, u32x4* slots, int T, int tid, int64_t off) {
-    const char* g = ptrs.p[kMaxR + rank] + off;
-    u32x4* wave_base = slots + rank * T + (tid & ~63);
+__device__ __forceinline__ void slot_fetch_direct(const char* rank_base, u32x4* slots, int slot, int T, int tid, int64_t off) {
+    const char* g = rank_base + off;
+    u32x4* wave_base = slots + slot * T + (tid & ~63);
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
                                      (__attribute__((address_space(3))) void*)wave_base, 16, 0, 2 /* nt */);
 }
 
-template <int DT, bool DIRECT>
-__global__ __launch_bounds__(kThreads) void column_slot_kernel(ColumnLaunch L, RankPtrs ptrs) {
+// A tile is T x V vectors of every rank: thread t owns vectors t, t + T, ..., t + (V - 1) T of it,
+// so that every wave access is 1 KiB contiguous and the workgroup covers 16 T V contiguous bytes
+// of each rank buffer.  What the memory system rewards (measured on MI355X with a bare kernel of
+// this shape, 8 buffers of 512 MiB read and written in place): the same 32 KiB of slots as five
+// workgroups of 256 threads per CU 5.97 TB/s; one workgroup per CU holding 64 KiB of slots, 8 KiB
+// of every rank, 6.40 (256 threads x 2 vectors) to 6.55 TB/s (512 threads x 1); 128 KiB of slots
+// 6.1 to 6.3.  Fewer, larger workgroups keep the requests of a CU in a narrow range of addresses.
+// Elements [lo, hi) of a vector (0 <= lo <= hi <= elements per vector) to memory: the whole vector
+// as one streaming store, a part of it element by element.
+template <int DT>
+__device__ __forceinline__ void store_vector_part(char* p, u32x4 x, int lo, int hi) {
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int VE = 16 / ES;
+    if (lo == 0 && hi == VE) { stv_nt(p, x); return; }
+    for (int e = lo; e < hi; ++e) {
+        const int wi = (e * ES) >> 2;
+        const uint32_t word = wi == 0 ? x.x : wi == 1 ? x.y : wi == 2 ? x.z : x.w;
+        store_elem<DT>(p + e * ES, word >> (((e * ES) & 3) * 8));
+    }
+}
+
+// One tile of the slot runner.  MASKED: the tile is cut by the segment's ends.  Such a tile runs
+// the same way with three differences: a vector that lies outside the segment is neither loaded nor
+// stored; a vector that the boundary cuts is loaded whole - a 16-byte vector at a 16-byte boundary
+// that holds one valid element lies in that element's page, so the load cannot fault, and what it
+// brings in from beyond the boundary is computed on and thrown away - and stored element by
+// element, only the elements inside.
+template <int DT, bool DIRECT, int V, bool MASKED>
+__device__ __forceinline__ void slot_tile(const ColumnLaunch& L, const DevColSegment& seg, const RankPtrs& ptrs, const LanePtr& in_ptr,
+                                          const LanePtr& out_ptr, u32x4* slots, int64_t vfirst, int T, int tid) {
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int VE = 16 / ES;
+    const PCCL_CONST uint64_t* prog = as_const(L.instrs) + seg.prog_start;
+    int64_t off[V];
+    int elo[V], ehi[V];   // MASKED: the elements of vector v inside the segment
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const int64_t vec = vfirst + (int64_t)v * T + tid;
+        off[v] = vec * 16;
+        elo[v] = 0; ehi[v] = VE;
+        if constexpr (MASKED) {
+            const int64_t e0 = vec * VE;
+            const int64_t a = seg.start > e0 ? seg.start - e0 : 0, b = seg.end - e0 < VE ? seg.end - e0 : VE;
+            elo[v] = (int)(a < VE ? a : VE);
+            ehi[v] = (int)(b > elo[v] ? b : elo[v]);
+        }
+    }
+    const PCCL_CONST uint64_t* pre = as_const(L.pre) + seg.pre_start;
+    uint64_t w4[4] = {prog[0], prog[1], prog[2], prog[3]};
+    if constexpr (DIRECT) {
+        // the ranks this program reads by first touch, as a mask in the segment record: nothing
+        // else has to be read before the first load can go out
+        for (uint64_t m = seg.pre_mask; m; m &= m - 1) {
+            const int rank = __builtin_ctzll(m);
+            const char* base = in_ptr.of(rank);
+#pragma unroll
+            for (int v = 0; v < V; ++v)
+                if (!MASKED || ehi[v] > elo[v]) slot_fetch_direct(base, slots, rank * V + v, T, tid, off[v]);
+        }
+        // the loads above write LDS behind the compiler's back: wait for all of them before
+        // any slot is read, and keep the slot reads below this point
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+        for (int i = 0; i < seg.pre_words; ++i) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                if (MASKED && ehi[v] <= elo[v]) continue;
+                uint64_t word = pre[i];
+                if ((word >> 56) != 0xFF) { slot_fetch<8>(word, ptrs, slots, V, v, T, tid, off[v]); continue; }
+                if (((word >> 24) & 0xFF) != 0xFF) { slot_fetch<4>(word, ptrs, slots, V, v, T, tid, off[v]); word >>= 32; }
+                if (((word >> 8) & 0xFF) != 0xFF) { slot_fetch<2>(word, ptrs, slots, V, v, T, tid, off[v]); word >>= 16; }
+                if ((word & 0xFF) != 0xFF) slot_fetch<1>(word, ptrs, slots, V, v, T, tid, off[v]);
+            }
+        }
+    }
+    u32x4 acc[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = u32x4{0, 0, 0, 0};
+    // The interpreter loop.  Programs are padded to a multiple of 4 instructions (one scalar load
+    // brings in four; the first four were asked for before the wait above), and the loop is
+    // software-pipelined: both slot operands of the NEXT instruction are read - always, whether it
+    // uses them or not, so that no branch stands between the reads - while the current instruction
+    // computes.  An instruction never reads from a slot what its predecessor wrote there (it takes
+    // such a value from the accumulator; that is how the planner builds the programs), so reading
+    // ahead of the predecessor's slot write is safe.
+    ColInstrDev in = unpack_instr(w4[0]);
+    u32x4 xa[V], xb[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) { xa[v] = slots[(in.peer * V + v) * T + tid]; xb[v] = slots[(in.self * V + v) * T + tid]; }
+    for (int k = 0; k < seg.prog_len; k += 4) {
+        const int kn = k + 4 < seg.prog_len ? k + 4 : k;   // the last group re-reads itself (unused)
+        const uint64_t n4[4] = {prog[kn], prog[kn + 1], prog[kn + 2], prog[kn + 3]};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const ColInstrDev nin = unpack_instr(j < 3 ? w4[j + 1] : n4[0]);
+            u32x4 na[V], nb[V];
+#pragma unroll
+            for (int v = 0; v < V; ++v) { na[v] = slots[(nin.peer * V + v) * T + tid]; nb[v] = slots[(nin.self * V + v) * T + tid]; }
+            const int kind = in.store & 3;
+            const bool to_mem = kind == 2 || (kind == 1 && (in.store & 4));
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const u32x4 a = in.a_src == 2 ? acc[v] : xa[v];
+                const u32x4 b = in.b_src == 2 ? acc[v] : xb[v];
+                acc[v] = in.b_src != 0 ? vec_op<DT>(a, b, in.redop) : a;
+            }
+            if (kind == 1) {
+#pragma unroll
+                for (int v = 0; v < V; ++v) slots[(in.self * V + v) * T + tid] = acc[v];
+            }
+            if (to_mem) {
+                char* const dst = out_ptr.of(in.self);
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    if constexpr (MASKED) store_vector_part<DT>(dst + off[v], acc[v], elo[v], ehi[v]);
+                    else stv_nt(dst + off[v], acc[v]);
+                }
+            }
+            in = nin;
+#pragma unroll
+            for (int v = 0; v < V; ++v) { xa[v] = na[v]; xb[v] = nb[v]; }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w4[j] = n4[j];
+    }
+    for (uint64_t m = seg.bcast_mask; m; m &= m - 1) {
+        char* const dst = out_ptr.of(__builtin_ctzll(m));
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            if constexpr (MASKED) store_vector_part<DT>(dst + off[v], acc[v], elo[v], ehi[v]);
+            else stv_nt(dst + off[v], acc[v]);
+        }
+    }
+}
+
+// (A workgroup has at most 1024 / V threads, so that the V-fold register need of the pipelined loop fits.)
+template <int DT, bool DIRECT, int V>
+__global__ __launch_bounds__(1024 / V) void column_slot_kernel(ColumnLaunch L, RankPtrs ptrs) {
     extern __shared__ u32x4 slots[];
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
     const int T = blockDim.x;
     const int tid = threadIdx.x;
-    const int64_t tile_v = T;
+    const int64_t tile_v = (int64_t)T * V;
+    const LanePtr out_ptr(ptrs.p[tid & 63]), in_ptr(ptrs.p[kMaxR + (tid & 63)]);   // stores / first-touch loads
+    // A workgroup that walks several tiles (a grid capped at the number of workgroups resident at
+    // once) keeps the segment record while its tiles stay in one segment: from the second tile on
+    // nothing has to be read before the first load goes out.
+    int have = -1;
+    DevColSegment seg{};
     for (int64_t w = blockIdx.x; w < span_tiles(L.total_tiles, L.xcd_run); w += gridDim.x) {
         const int64_t tile = xcd_tile(w, L.xcd_run);
         if (tile >= L.total_tiles) continue;
-        int lo = 0, hi = L.num_segs;
-        while (hi - lo > 1) {
-            int mid = (lo + hi) >> 1;
-            if (as_const(L.segs)[mid].first_tile <= tile) lo = mid; else hi = mid;
-        }
-        const DevColSegment seg = load_const(L.segs + lo);
+        const int lo = find_segment(L, tile);
+        if (lo != have) { seg = load_const(L.segs + lo); have = lo; }
         const int64_t vfirst = seg.first_vec + (tile - seg.first_tile) * tile_v;
-        const PCCL_CONST uint64_t* prog = as_const(L.instrs) + seg.prog_start;
         const bool interior = vfirst * VE >= seg.start && (vfirst + tile_v) * VE <= seg.end;
-        if (!interior) {
-            column_edge_tile<DT>(seg, prog, ptrs, vfirst, tile_v, tid, T);
-            continue;
-        }
-        const int64_t off = (vfirst + tid) * 16;
-        const PCCL_CONST uint64_t* pre = as_const(L.pre) + seg.pre_start;
-        if constexpr (DIRECT) {
-            for (int i = 0; i < seg.pre_words; ++i) {
-                uint64_t word = pre[i];
-                for (int j = 0; j < 8 && (word & 0xFF) != 0xFF; ++j, word >>= 8)
-                    slot_fetch_direct((int)(word & 0xFF), ptrs, slots, T, tid, off);
-            }
-            // the loads above write LDS behind the compiler's back: wait for all of them before
-            // any slot is read, and keep the slot reads below this point
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        } else {
-            for (int i = 0; i < seg.pre_words; ++i) {
-                uint64_t word = pre[i];
-                if ((word >> 56) != 0xFF) { slot_fetch<8>(word, ptrs, slots, T, tid, off); continue; }
-                if (((word >> 24) & 0xFF) != 0xFF) { slot_fetch<4>(word, ptrs, slots, T, tid, off); word >>= 32; }
-                if (((word >> 8) & 0xFF) != 0xFF) { slot_fetch<2>(word, ptrs, slots, T, tid, off); word >>= 16; }
-                if ((word & 0xFF) != 0xFF) slot_fetch<1>(word, ptrs, slots, T, tid, off);
-            }
-        }
-        u32x4 acc = u32x4{0, 0, 0, 0};
-        // programs are padded to a multiple of 4 instructions: one scalar load brings in four
-        for (int k = 0; k < seg.prog_len; k += 4) {
-            const uint64_t w[4] = {prog[k], prog[k + 1], prog[k + 2], prog[k + 3]};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const ColInstrDev in = unpack_instr(w[j]);
-                const u32x4 a = in.a_src == 2 ? acc : slots[in.peer * T + tid];
-                if (in.b_src != 0) {
-                    const u32x4 b = in.b_src == 2 ? acc : slots[in.self * T + tid];
-                    acc = vec_op<DT>(a, b, in.redop);
-                } else acc = a;
-                const int kind = in.store & 3;
-                if (kind == 1) slots[in.self * T + tid] = acc;
-                if (kind == 2 || (kind == 1 && (in.store & 4))) stv_nt(ptrs.p[in.self] + off, acc);
-            }
-        }
-        if (seg.bcast_mask) broadcast_store<true>(seg.bcast_mask, ptrs, off, acc);
+        if (interior) slot_tile<DT, DIRECT, V, false>(L, seg, ptrs, in_ptr, out_ptr, slots, vfirst, T, tid);
+        else slot_tile<DT, DIRECT, V, true>(L, seg, ptrs, in_ptr, out_ptr, slots, vfirst, T, tid);
     }
 }
 
@@ -911,6 +1109,38 @@ static int grid_for_tiles(int64_t ntiles, int run) {
     return (int)(ntiles < cap ? ntiles : cap);
 }
 
+// The slot runner's launch: L.slot_vecs vectors per thread, L.slot_lds_bytes of dynamic LDS (at
+// least the slots; more to limit the workgroups per CU).  More than 64 KiB of dynamic LDS has to be
+// allowed per kernel and device once.
+template <class K>
+static int launch_slot_kernel(K kernel, std::atomic<int>* allowed, const ColumnLaunch& L, const RankPtrs& ptrs, unsigned grid, hipStream_t s) {
+    const int dev = current_device();
+    const int lds = L.slot_lds_bytes;
+    if (L.slot_threads * L.slot_vecs > 1024) return (int)hipErrorInvalidValue;   // the kernels' launch bounds
+    if (lds > 64 * 1024 && allowed[dev].load(std::memory_order_relaxed) < lds) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (rc != hipSuccess) return (int)rc;
+        allowed[dev].store(lds, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(L.slot_threads), (size_t)lds, s, L, ptrs);
+    return (int)hipGetLastError();
+}
+
+template <int DT>
+static int launch_slot_dt(const ColumnLaunch& L, const RankPtrs& ptrs, unsigned grid, hipStream_t s) {
+    static std::atomic<int> allowed[5][kMaxDevices];   // per kernel of this element type
+    if (L.slot_direct) {
+        switch (L.slot_vecs) {
+            case 1: return launch_slot_kernel(column_slot_kernel<DT, true, 1>, allowed[0], L, ptrs, grid, s);
+            case 2: return launch_slot_kernel(column_slot_kernel<DT, true, 2>, allowed[1], L, ptrs, grid, s);
+            case 4: return launch_slot_kernel(column_slot_kernel<DT, true, 4>, allowed[2], L, ptrs, grid, s);
+            default: return (int)hipErrorInvalidValue;
+        }
+    }
+    if (L.slot_vecs != 1) return (int)hipErrorInvalidValue;   // fetching through registers: one vector per thread
+    return launch_slot_kernel(column_slot_kernel<DT, false, 1>, allowed[3], L, ptrs, grid, s);
+}
+
 template <int DT>
 static int launch_column_dt(const ColumnLaunch& L0, const RankPtrs& ptrs, hipStream_t s) {
     ColumnLaunch L = L0;
@@ -919,12 +1149,7 @@ static int launch_column_dt(const ColumnLaunch& L0, const RankPtrs& ptrs, hipStr
     if (L.num_blocks > 0 && grid > L.num_blocks) grid = L.num_blocks;
     if (grid > (1 << 30)) grid = 1 << 30;
     if (grid <= 0) return 0;
-    if (L.slot_threads > 0) {
-        const size_t lds = (size_t)L.num_ranks * L.slot_threads * 16;
-        if (L.slot_direct) hipLaunchKernelGGL((column_slot_kernel<DT, true>), dim3((unsigned)grid), dim3(L.slot_threads), lds, s, L, ptrs);
-        else hipLaunchKernelGGL((column_slot_kernel<DT, false>), dim3((unsigned)grid), dim3(L.slot_threads), lds, s, L, ptrs);
-        return (int)hipGetLastError();
-    }
+    if (L.slot_threads > 0) return launch_slot_dt<DT>(L, ptrs, (unsigned)grid, s);
     switch (L.vecs_per_thread) {
         case 1: hipLaunchKernelGGL((column_kernel<DT, 1>), dim3((unsigned)grid), dim3(kThreads), 0, s, L, ptrs); break;
         case 2: hipLaunchKernelGGL((column_kernel<DT, 2>), dim3((unsigned)grid), dim3(kThreads), 0, s, L, ptrs); break;

@@ -78,19 +78,33 @@ class Engine:
             if rc in (_lib.ERR_NOT_FOUND, _lib.ERR_NOT_A_GRAPH):   # where the reference's loader returns false
                 return False
             _lib.check(rc)
+            if name not in self._elem_bytes:
+                self._note_dtype(name, _lib.HostGraph.from_file(path))
         return True
 
     def register_operation_json(self, name: str, text: str, rank: int) -> bool:
         self._elem_bytes.pop(name, None)
         data = text.encode()
         _lib.check(self._L.pccl_hip_register_json(self._h, name.encode(), rank, data, len(data)))
+        self._note_dtype(name, _lib.HostGraph.from_json(text))
         return True
+
+    def _note_dtype(self, name: str, graph) -> None:
+        """Remember the element size of the operation's graphs at registration (a host-side parse), so
+        that checking the tensors of a call never has to link the operation: linking allocates, which
+        a caller that is capturing its stream cannot have."""
+        self._elem_bytes[name] = self._DTYPE_BYTES[graph.dtype]
 
     def last_error(self) -> str:
         return self._L.pccl_hip_last_error().decode(errors="replace")
 
     def set_option(self, key: str, value) -> None:
         _lib.check(self._L.pccl_hip_set_option(self._h, key.encode(), str(value).encode()))
+
+    def get_option(self, key: str) -> str:
+        buf = ctypes.create_string_buffer(64)
+        _lib.check(self._L.pccl_hip_get_option(self._h, key.encode(), buf, len(buf)))
+        return buf.value.decode()
 
     # -- execution ----------------------------------------------------------------------------
     def _as_list(self, t: TensorList, what: str) -> List[torch.Tensor]:

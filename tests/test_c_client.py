@@ -1,5 +1,6 @@
-"""The C ABI used from plain C (tests/c_abi/ring_client.c): compiled with gcc against
-include/pccl_hip.h, linked to libpccl_hip.so and libamdhip64 only."""
+"""The C ABI used from plain C (tests/c_abi/ring_client.c, compiled with gcc) and from a stand-alone
+C++ translation unit that lays its trigger arrays out with the reference's own struct declarations
+(tests/c_abi/adapter_check.cc); both link libpccl_hip.so and libamdhip64 only."""
 import os
 import subprocess
 
@@ -8,11 +9,12 @@ import pytest
 from helpers import ROOT
 
 CLIENT = os.path.join(ROOT, "tests", "c_abi", "build", "ring_client")
+ADAPTER = os.path.join(ROOT, "tests", "c_abi", "build", "adapter_check")
 GRAPHS = os.path.join(ROOT, "tests", "golden", "graphs")
 
 
 def client():
-    if not os.path.exists(CLIENT):
+    if not os.path.exists(CLIENT) or not os.path.exists(ADAPTER):
         from tests.c_abi import build          # not built yet (build() of the entry module does it)
         build.build()
     return CLIENT
@@ -35,3 +37,15 @@ def test_ring_allreduce_from_plain_c(stem, world, n):
     p = subprocess.run([client(), str(n)] + files, capture_output=True, text=True, timeout=120)
     assert p.returncode == 0, p.stdout + p.stderr
     assert f"ok ranks={world} elements={n}" in p.stdout
+
+
+@pytest.mark.gpu
+def test_trigger_arrays_laid_out_by_the_reference_headers():
+    """The row of the drop-in boundary that no loader of this repository touches: arrays built from
+    struct declarations with the reference's field order (proxy_trigger.h:8-30, primitive.h:8-17)
+    go through pccl_hip_register_triggers and pccl_hip_execute in all three modes and give the closed
+    form R (R + 1) / 2."""
+    client()
+    p = subprocess.run([ADAPTER], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "ok triggers laid out by the reference's headers: ranks=2 elements=2048 result=3" in p.stdout

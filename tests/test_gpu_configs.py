@@ -103,18 +103,27 @@ def test_config5_tree_32_ranks_96mb_ragged(engine_factory, dtype, redop, kind, m
     assert info["num_data_ops"] == 62 * 8                # every tree op cut into 8 ragged pieces
 
 
-@pytest.mark.parametrize("mode", ["column", "stepwise"])
-@pytest.mark.parametrize("nbytes", [4096, 65536, 1 << 20, 16 << 20, 256 << 20, 512 << 20])
+C4_SIZES = [4096 * 4 ** k for k in range(9)] + [512 << 20]      # 4 KB .. 256 MB in powers of 4, and 512 MB
+
+
+@pytest.mark.parametrize("mode", ["column", "stepwise", "persistent"])
+@pytest.mark.parametrize("nbytes", C4_SIZES)
 def test_config4_reduce_scatter_allgather_fp16(engine_factory, nbytes, mode):
+    """Configuration 4: every size of the sweep in every mode, as staged calls.  The results must
+    equal the ring's reduction order written with torch fp16 adds and the definitions of the two
+    collectives; up to 16 MB per rank they are also compared with the CPU oracle."""
+    from helpers import bits_equal, oracle_buffers
     world = 8
     n = nbytes // 2
     chunk = n // world
     print(f"config 4: RS/AG R={world} {nbytes} B per rank fp16, mode={mode}", flush=True)
     engine = engine_factory(world)
     x = dev_inputs("randn0.1", world, n, "float16")
+    with_oracle = nbytes <= (16 << 20)
     # reduce_scatter: chunk r of the ring-ordered sum lands on rank r
     name = f"rs_{nbytes}_{mode}"
-    register(engine, name, graph_jsons("ring", "build_reduce_scatter", world, n, "float16", "sm", 1), mode)
+    jsons = graph_jsons("ring", "build_reduce_scatter", world, n, "float16", "sm", 1)
+    register(engine, name, jsons, mode)
     outs = engine.execute_operation(name, x, [torch.zeros(chunk, dtype=torch.float16, device="cuda") for _ in range(world)])
     for c in range(world):
         lo = c * chunk
@@ -123,15 +132,101 @@ def test_config4_reduce_scatter_allgather_fp16(engine_factory, nbytes, mode):
         for k in range(1, world):
             acc = x[(c + 1 + k) % world][lo:lo + chunk] + acc
         assert same_bits(outs[c], acc), f"reduce_scatter chunk {c}"
+    if with_oracle:
+        want = oracle_buffers(jsons, [t.cpu() for t in x], "float16")
+        for c in range(world):
+            assert bits_equal(outs[c], want[c][c * chunk:(c + 1) * chunk]), f"reduce_scatter chunk {c} against the oracle"
     del outs
     # allgather: rank r contributes chunk r
     name = f"ag_{nbytes}_{mode}"
-    register(engine, name, graph_jsons("ring", "build_allgather", world, n, "float16", "sm", 1), mode)
+    jsons = graph_jsons("ring", "build_allgather", world, n, "float16", "sm", 1)
+    register(engine, name, jsons, mode)
     parts = [t[:chunk].contiguous() for t in x]
     outs = engine.execute_operation(name, parts, [torch.zeros(n, dtype=torch.float16, device="cuda") for _ in range(world)])
     whole = torch.cat(parts)
     for r in range(world):
         assert same_bits(outs[r], whole), f"allgather rank {r}"
+    if with_oracle:
+        want = oracle_buffers(jsons, [p.cpu() for p in parts], "float16", buffer_elems=n, place=lambda r: r * chunk)
+        for r in range(world):
+            assert bits_equal(outs[r], want[r]), f"allgather rank {r} against the oracle"
+    engine.set_option("mode", "auto")
+
+
+@pytest.mark.parametrize("dtype,redop,kind", [("int32", "sum", "randint"), ("float32", "max", "randn")])
+def test_config5_through_the_superoptimising_compiler(engine_factory, dtype, redop, kind):
+    """Configuration 5's graphs as `Compiler(enable_superopt=True)` emits them: the data ops arrive as
+    tma.reduce / tma.copy under the executor cuda_tma (the upgrade the reference's pass makes,
+    pccl/dsl/superopt/pass_.py:76-87) and run as the SM ops, at the full size, ragged pieces and all."""
+    import json
+    from pccl_amd.dsl import ALGORITHMS, Compiler
+    world, n = 32, 25_165_824
+    print(f"config 5 through Compiler(enable_superopt=True): tree R={world} n={n} {dtype} {redop}", flush=True)
+    cuts = ragged_cuts(n, 8, seed=0)
+    tree = ALGORITHMS["tree"]()
+    comp = Compiler(enable_superopt=True, topology=None)
+    docs = [comp.compile_to_dict(tree.build_allreduce(r, world, n, dtype=dtype, executor="sm", num_channels=1,
+                                                      reduce_op=redop, cuts=cuts)) for r in range(world)]
+    prims = {op["primitive"] for d in docs for op in d["operations"]}
+    execs = {op["executor"] for d in docs for op in d["operations"] if op["primitive"].startswith(("tma.", "sm."))}
+    assert {"tma.reduce", "tma.copy"} <= prims and "sm.reduce" not in prims and "sm.copy" not in prims
+    assert execs == {"cuda_tma"}
+    x = dev_inputs(kind, world, n, dtype)
+    engine = engine_factory(world)
+    want = torch.stack(x).sum(0, dtype=torch.int32) if redop == "sum" else torch.stack(x).amax(0)
+    for mode in ("auto", "persistent"):
+        name = f"c5_superopt_{dtype}_{mode}"
+        register(engine, name, [json.dumps(d) for d in docs], mode)
+        bufs = [t.clone() for t in x]
+        engine.execute_inplace(name, bufs, sync=True)
+        for r in range(world):
+            assert same_bits(bufs[r], want), f"mode {mode}, rank {r}"
+        del bufs
+    engine.set_option("mode", "auto")
+
+
+def test_config2_prescribed_inputs_match_the_committed_oracle_hash_in_every_mode(engine_factory):
+    """The headline configuration on its prescribed inputs (CPU generator, seed 0, drawn rank by rank
+    in eight slices and cast to bf16): the result of the column, level and persistent runners must
+    hash to what the CPU oracle produced for the full graph (tests/golden/headline_sha256.json,
+    written by tests/golden/make_headline_sha256.py)."""
+    import hashlib
+    import json
+    import os
+    from helpers import GOLDEN
+    golden = json.load(open(os.path.join(GOLDEN, "headline_sha256.json")))
+    world, n, slices = 8, 268_435_456, 8
+    print("config 2 on the prescribed inputs against the committed sha256, three modes", flush=True)
+
+    def sha(t):
+        h = hashlib.sha256()
+        flat = t.view(torch.int16)
+        for i in range(0, flat.numel(), 1 << 26):
+            h.update(flat[i:i + (1 << 26)].cpu().numpy().tobytes())
+        return h.hexdigest()
+
+    g = torch.Generator().manual_seed(0)
+    per = n // slices
+    x = []
+    for r in range(world):
+        buf = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+        for s in range(slices):
+            buf[s * per:(s + 1) * per] = torch.randn(per, generator=g).to(torch.bfloat16).cuda()
+        x.append(buf)
+        print(f"  rank {r} drawn", flush=True)
+    assert sha(x[0]) == golden["input_sha256_per_rank"][0] and sha(x[7]) == golden["input_sha256_per_rank"][7]
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 4)
+    engine = engine_factory(world)
+    for mode in ("column", "stepwise", "persistent"):
+        print(f"  mode={mode}", flush=True)
+        register(engine, f"c2_golden_{mode}", jsons, mode)
+        bufs = [t.clone() for t in x]
+        engine.execute_inplace(f"c2_golden_{mode}", bufs, sync=True)
+        assert sha(bufs[0]) == golden["output_sha256"], f"mode {mode}"
+        for r in range(1, world):
+            assert same_bits(bufs[r], bufs[0]), f"mode {mode}: rank {r} differs from rank 0"
+        del bufs
+    engine.set_option("mode", "auto")
 
 
 def test_config2_headline_shape_in_all_modes_agree(engine_factory):
