@@ -462,15 +462,18 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
             if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || (in.store & STORE_KIND) == 1) reads_back = true;
         e.slot_threads = 0; e.slot_vecs = 1; e.slot_lds_bytes = 0;
         if (ctx->lds_slots && (ctx->slot_threads > 0 || reads_back || ctx->R <= 16)) {
-            // Shape of a workgroup: threads x vectors per thread, and how much LDS it asks for.  One
-            // workgroup per CU (asking for more than half of the CU's 160 KiB) that holds 8 KiB of
-            // every rank is what the memory system likes best where that fits: 8 ranks 512 x 1,
-            // 16 ranks 256 x 2 (128 KiB of slots); 32 ranks 128 x 2 (4 KiB of every rank in 128 KiB),
-            // 64 ranks 128 x 1.  Few ranks keep small workgroups, several per CU.
+            // Shape of a workgroup: threads x vectors per thread (a tile is that many 16-byte vectors of
+            // every rank), chosen so that the slots of a workgroup are 64 KiB at most and at least two
+            // workgroups share a CU - one computes while the other waits for memory.  Measured on
+            // MI355X, same box and call: 8 ranks x 512 MiB bf16 ring 256 x 1 (five per CU) 1.43 ms,
+            // 256 x 2 (two per CU, 8 KiB of every rank per tile) 1.39; 32-rank tree 64 x 1 1.19 ms,
+            // 128 x 1 1.12; 16 ranks the same from 128 to 512 threads.  One workgroup per CU with
+            // larger tiles, which a bare kernel of this traffic shape likes best (1.31 ms for the
+            // ring), loses here: the program's arithmetic is then not overlapped with anything.
             const int R = ctx->R;
-            int threads = R <= 4 ? 256 : R <= 8 ? 512 : R <= 16 ? 256 : 128;
-            int vecs = R <= 4 ? 1 : R <= 8 ? 1 : R <= 32 ? 2 : 1;
-            int lds_kib = R <= 4 ? 0 : 96;
+            int threads = R <= 16 ? 256 : R <= 32 ? 128 : 64;
+            int vecs = R > 4 && R <= 8 ? 2 : 1;
+            int lds_kib = 0;
             if (ctx->slot_threads > 0) { threads = ctx->slot_threads; if (ctx->slot_vecs == 0) vecs = 1; if (ctx->slot_lds_kib == 0) lds_kib = 0; }
             if (ctx->slot_vecs > 0) vecs = ctx->slot_vecs;
             if (ctx->slot_lds_kib > 0) lds_kib = ctx->slot_lds_kib;

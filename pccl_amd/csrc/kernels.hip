@@ -167,7 +167,9 @@ __device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
         const float r0 = as_f32(a.x) + as_f32(b.x), r1 = as_f32(a.y) + as_f32(b.y);
         const float r2 = as_f32(a.z) + as_f32(b.z), r3 = as_f32(a.w) + as_f32(b.w);
         u32x4 r = {as_u32(r0), as_u32(r1), as_u32(r2), as_u32(r3)};
-        if (__builtin_expect(__builtin_isunordered(r0, r1) | __builtin_isunordered(r2, r3), 0)) {
+        // one compare per pair of results, combined on the scalar side: the whole wave takes the
+        // repair branch if any lane saw a NaN (the repairs themselves are per element)
+        if (__builtin_expect((__builtin_amdgcn_ballot_w64(__builtin_isunordered(r0, r1)) | __builtin_amdgcn_ballot_w64(__builtin_isunordered(r2, r3))) != 0, 0)) {
             if (r0 != r0) r.x = 0x7FFFFFFFu;
             if (r1 != r1) r.y = 0x7FFFFFFFu;
             if (r2 != r2) r.z = 0x7FFFFFFFu;
@@ -176,18 +178,18 @@ __device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
         return r;
     } else if constexpr (DT == PCCL_BF16) {
         u32x4 r;
-        bool nan = false;
+        uint64_t nan = 0;
         const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
         uint32_t rw[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float lo = as_f32(aw[i] << 16) + as_f32(bw[i] << 16);
             const float hi = as_f32(aw[i] & 0xFFFF0000u) + as_f32(bw[i] & 0xFFFF0000u);
-            nan |= __builtin_isunordered(lo, hi);
+            nan |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(lo, hi));
             const f32x2 pair = {lo, hi};
             rw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
         }
-        if (__builtin_expect(nan, 0)) {
+        if (__builtin_expect(nan != 0, 0)) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 if ((rw[i] & 0x7FFFu) > 0x7F80u) rw[i] = (rw[i] & 0xFFFF0000u) | 0x7FFFu;
@@ -199,14 +201,14 @@ __device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
     } else if constexpr (DT == PCCL_F16) {
         const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
         uint32_t rw[4];
-        bool nan = false;
+        uint64_t nan = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const h2 s = __builtin_bit_cast(h2, aw[i]) + __builtin_bit_cast(h2, bw[i]);
-            nan |= __builtin_isunordered(s[0], s[1]);
+            nan |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(s[0], s[1]));
             rw[i] = __builtin_bit_cast(uint32_t, s);
         }
-        if (__builtin_expect(nan, 0)) {
+        if (__builtin_expect(nan != 0, 0)) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 if ((rw[i] & 0x7FFFu) > 0x7C00u) rw[i] = (rw[i] & 0xFFFF0000u) | 0x7FFFu;
@@ -866,26 +868,6 @@ __global__ __launch_bounds__(kThreads) void column_kernel(ColumnLaunch L, RankPt
 // halving-doubling butterflies, trees).  A thread only ever touches its own slots, so no barrier
 // is needed.  Results are bit-identical to the op-by-op execution for the same reason as above.
 
-// Rank pointers without a memory access per use: lane l of every wave keeps the pointers of rank l
-// (the wave has 64 lanes and a context at most 64 ranks), and a uniform rank picks its pointer
-// with v_readlane.  Reading a pointer from the kernel arguments instead is a scalar load of its
-// own - a hundred cycles and more each time, in front of every first-touch load, every store and
-// every broadcast of a program, which a workgroup that has the CU to itself cannot hide.
-struct LanePtr {
-    uint32_t lo, hi;
-    __device__ __forceinline__ explicit LanePtr(const char* p) : lo((uint32_t)(uintptr_t)p), hi((uint32_t)((uintptr_t)p >> 32)) {
-        // The pointer arrives by a vector load.  Passing it through an empty asm makes the compiler
-        // wait for that load here, once; otherwise every use inside a loop that also issues memory
-        // operations is preceded by a wait for all of them (vmcnt(0)), which serialises the loop.
-        asm volatile("" : "+v"(lo), "+v"(hi));
-    }
-    __device__ __forceinline__ char* of(int rank) const {
-        const uint32_t l = __builtin_amdgcn_readlane(lo, rank), h = __builtin_amdgcn_readlane(hi, rank);
-        return reinterpret_cast<char*>((uintptr_t)l | (uintptr_t)h << 32);
-    }
-};
-static_assert(kMaxR == 64, "one lane per rank");
-
 // Slot (rank r, vector v) of thread t in a workgroup of T threads with V vectors per thread sits at
 // index (r * V + v) * T + t: consecutive lanes 16 bytes apart (conflict-free 128-bit accesses), and a
 // wave's 64 lanes form the contiguous 1 KiB block that one direct-to-LDS load fills.
@@ -936,8 +918,8 @@ __device__ __forceinline__ void store_vector_part(char* p, u32x4 x, int lo, int 
 // brings in from beyond the boundary is computed on and thrown away - and stored element by
 // element, only the elements inside.
 template <int DT, bool DIRECT, int V, bool MASKED>
-__device__ __forceinline__ void slot_tile(const ColumnLaunch& L, const DevColSegment& seg, const RankPtrs& ptrs, const LanePtr& in_ptr,
-                                          const LanePtr& out_ptr, u32x4* slots, int64_t vfirst, int T, int tid) {
+__device__ __forceinline__ void slot_tile(const ColumnLaunch& L, const DevColSegment& seg, const RankPtrs& ptrs,
+                                          u32x4* slots, int64_t vfirst, int T, int tid) {
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
     const PCCL_CONST uint64_t* prog = as_const(L.instrs) + seg.prog_start;
@@ -962,7 +944,7 @@ __device__ __forceinline__ void slot_tile(const ColumnLaunch& L, const DevColSeg
         // else has to be read before the first load can go out
         for (uint64_t m = seg.pre_mask; m; m &= m - 1) {
             const int rank = __builtin_ctzll(m);
-            const char* base = in_ptr.of(rank);
+            const char* base = ptrs.p[kMaxR + rank];
 #pragma unroll
             for (int v = 0; v < V; ++v)
                 if (!MASKED || ehi[v] > elo[v]) slot_fetch_direct(base, slots, rank * V + v, T, tid, off[v]);
@@ -986,64 +968,61 @@ __device__ __forceinline__ void slot_tile(const ColumnLaunch& L, const DevColSeg
     u32x4 acc[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) acc[v] = u32x4{0, 0, 0, 0};
-    // The interpreter loop.  Programs are padded to a multiple of 4 instructions (one scalar load
-    // brings in four; the first four were asked for before the wait above), and the loop is
-    // software-pipelined: both slot operands of the NEXT instruction are read - always, whether it
-    // uses them or not, so that no branch stands between the reads - while the current instruction
-    // computes.  An instruction never reads from a slot what its predecessor wrote there (it takes
-    // such a value from the accumulator; that is how the planner builds the programs), so reading
-    // ahead of the predecessor's slot write is safe.
-    ColInstrDev in = unpack_instr(w4[0]);
-    u32x4 xa[V], xb[V];
-#pragma unroll
-    for (int v = 0; v < V; ++v) { xa[v] = slots[(in.peer * V + v) * T + tid]; xb[v] = slots[(in.self * V + v) * T + tid]; }
+    // The interpreter loop.  Programs are padded to a multiple of 4 instructions: one scalar load
+    // brings in four (the first four were asked for before the wait above).  Forms of this loop
+    // that read the next instruction's slot operands ahead, that read both operands
+    // unconditionally to avoid branches, or that kept the rank pointers in lanes (v_readlane
+    // instead of a scalar load per use) were measured and were no faster where several workgroups
+    // share a CU, and slower for MAX programs; this plain form stays.
     for (int k = 0; k < seg.prog_len; k += 4) {
-        const int kn = k + 4 < seg.prog_len ? k + 4 : k;   // the last group re-reads itself (unused)
-        const uint64_t n4[4] = {prog[kn], prog[kn + 1], prog[kn + 2], prog[kn + 3]};
+        if (k > 0) { w4[0] = prog[k]; w4[1] = prog[k + 1]; w4[2] = prog[k + 2]; w4[3] = prog[k + 3]; }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const ColInstrDev nin = unpack_instr(j < 3 ? w4[j + 1] : n4[0]);
-            u32x4 na[V], nb[V];
-#pragma unroll
-            for (int v = 0; v < V; ++v) { na[v] = slots[(nin.peer * V + v) * T + tid]; nb[v] = slots[(nin.self * V + v) * T + tid]; }
+            const ColInstrDev in = unpack_instr(w4[j]);
+            const u32x4* const pa = slots + (in.peer * V) * T + tid;
+            u32x4* const ps = slots + (in.self * V) * T + tid;
             const int kind = in.store & 3;
             const bool to_mem = kind == 2 || (kind == 1 && (in.store & 4));
+            char* const dst = ptrs.p[in.self];
 #pragma unroll
             for (int v = 0; v < V; ++v) {
-                const u32x4 a = in.a_src == 2 ? acc[v] : xa[v];
-                const u32x4 b = in.b_src == 2 ? acc[v] : xb[v];
-                acc[v] = in.b_src != 0 ? vec_op<DT>(a, b, in.redop) : a;
-            }
-            if (kind == 1) {
-#pragma unroll
-                for (int v = 0; v < V; ++v) slots[(in.self * V + v) * T + tid] = acc[v];
-            }
-            if (to_mem) {
-                char* const dst = out_ptr.of(in.self);
-#pragma unroll
-                for (int v = 0; v < V; ++v) {
+                const u32x4 a = in.a_src == 2 ? acc[v] : pa[v * T];
+                if (in.b_src != 0) {
+                    const u32x4 b = in.b_src == 2 ? acc[v] : ps[v * T];
+                    acc[v] = vec_op<DT>(a, b, in.redop);
+                } else acc[v] = a;
+                if (kind == 1) ps[v * T] = acc[v];
+                if (to_mem) {
                     if constexpr (MASKED) store_vector_part<DT>(dst + off[v], acc[v], elo[v], ehi[v]);
                     else stv_nt(dst + off[v], acc[v]);
                 }
             }
-            in = nin;
+        }
+    }
+    // the broadcast tail, four rank pointers fetched per round so that their scalar loads overlap
+    for (uint64_t m = seg.bcast_mask; m;) {
+        char* dsts[4];
+        int n = 0;
 #pragma unroll
-            for (int v = 0; v < V; ++v) { xa[v] = na[v]; xb[v] = nb[v]; }
+        for (int i = 0; i < 4; ++i) {
+            const int r = m ? __builtin_ctzll(m) : 0;
+            if (m) { m &= m - 1; n = i + 1; }
+            dsts[i] = ptrs.p[r];
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) w4[j] = n4[j];
-    }
-    for (uint64_t m = seg.bcast_mask; m; m &= m - 1) {
-        char* const dst = out_ptr.of(__builtin_ctzll(m));
+        for (int i = 0; i < 4; ++i) {
+            if (i >= n) break;
+            char* const dst = dsts[i];
 #pragma unroll
-        for (int v = 0; v < V; ++v) {
-            if constexpr (MASKED) store_vector_part<DT>(dst + off[v], acc[v], elo[v], ehi[v]);
-            else stv_nt(dst + off[v], acc[v]);
+            for (int v = 0; v < V; ++v) {
+                if constexpr (MASKED) store_vector_part<DT>(dst + off[v], acc[v], elo[v], ehi[v]);
+                else stv_nt(dst + off[v], acc[v]);
+            }
         }
     }
 }
 
-// (A workgroup has at most 1024 / V threads, so that the V-fold register need of the pipelined loop fits.)
+// (A workgroup has at most 1024 / V threads, so that the V-fold register need fits.)
 template <int DT, bool DIRECT, int V>
 __global__ __launch_bounds__(1024 / V) void column_slot_kernel(ColumnLaunch L, RankPtrs ptrs) {
     extern __shared__ u32x4 slots[];
@@ -1052,7 +1031,6 @@ __global__ __launch_bounds__(1024 / V) void column_slot_kernel(ColumnLaunch L, R
     const int T = blockDim.x;
     const int tid = threadIdx.x;
     const int64_t tile_v = (int64_t)T * V;
-    const LanePtr out_ptr(ptrs.p[tid & 63]), in_ptr(ptrs.p[kMaxR + (tid & 63)]);   // stores / first-touch loads
     // A workgroup that walks several tiles (a grid capped at the number of workgroups resident at
     // once) keeps the segment record while its tiles stay in one segment: from the second tile on
     // nothing has to be read before the first load goes out.
@@ -1065,8 +1043,8 @@ __global__ __launch_bounds__(1024 / V) void column_slot_kernel(ColumnLaunch L, R
         if (lo != have) { seg = load_const(L.segs + lo); have = lo; }
         const int64_t vfirst = seg.first_vec + (tile - seg.first_tile) * tile_v;
         const bool interior = vfirst * VE >= seg.start && (vfirst + tile_v) * VE <= seg.end;
-        if (interior) slot_tile<DT, DIRECT, V, false>(L, seg, ptrs, in_ptr, out_ptr, slots, vfirst, T, tid);
-        else slot_tile<DT, DIRECT, V, true>(L, seg, ptrs, in_ptr, out_ptr, slots, vfirst, T, tid);
+        if (interior) slot_tile<DT, DIRECT, V, false>(L, seg, ptrs, slots, vfirst, T, tid);
+        else slot_tile<DT, DIRECT, V, true>(L, seg, ptrs, slots, vfirst, T, tid);
     }
 }
 
