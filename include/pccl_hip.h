@@ -21,6 +21,7 @@ extern "C" {
 #define PCCL_HIP_MAX_CHANNELS 8     /* reference include/common/config.h:27 */
 #define PCCL_HIP_NUM_SIGNALS 4096   /* reference include/common/config.h:24 (ints per rank) */
 #define PCCL_HIP_MAX_FUSED_STEPS 128 /* reference include/common/config.h:28 */
+#define PCCL_HIP_STATIC_WORKSPACE_BYTES (4u << 20) /* device memory pccl_hip_execute_inplace_static works in, per GPU */
 
 typedef enum {
     PCCL_OK = 0,
@@ -262,6 +263,22 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
  * No counterpart in the reference, whose rank buffers belong to the engine. */
 int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
                              void* stream, int sync);
+/* pccl_hip_execute_inplace for callers that cannot allocate: code whose stream is being captured into a
+ * graph, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * The call allocates no device memory and copies nothing: it runs the operation as ONE launch of the
+ * persistent (flag-ordered) runner whose tables and progress block (error words, one flag per work
+ * item, one ready word per data op, the op and dependency tables, the item-to-op map) live in a
+ * workspace of PCCL_HIP_STATIC_WORKSPACE_BYTES that is part of the library's device image; what has to
+ * reach the device travels in kernel arguments.  An operation that needs more (the error says how much;
+ * larger work items - option "step_tile_bytes" - need less) is refused with PCCL_ERR_INVALID, and so are
+ * rank buffers smaller than the graph addresses.  The first call for an operation links it on the host
+ * (host memory only; pccl_hip_op_info does the same ahead of time).  Every GPU has one such workspace,
+ * shared by all contexts and operations and keeping the last call's contents: when another operation
+ * used it last, this call first clears the progress block and rewrites the tables (by kernels on
+ * `stream`), which it refuses to do on a capturing stream (execute once outside the capture first).
+ * Calls that overlap in time on one GPU - two streams, two threads - race on the workspace. */
+int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
+                                    void* stream, int sync);
 /* Engine::syncOp / Engine::resetSignals (reference csrc/engine_c.cc:562-593). */
 int pccl_hip_sync(pccl_hip_ctx* ctx, const char* name);
 int pccl_hip_reset_signals(pccl_hip_ctx* ctx, const char* name);

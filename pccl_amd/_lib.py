@@ -85,7 +85,7 @@ EXPORTS = [
     "pccl_program_free", "pccl_program_get_info", "pccl_program_get_ops", "pccl_program_get_column",
     "pccl_hip_create",
     "pccl_hip_destroy", "pccl_hip_register_file", "pccl_hip_register_json", "pccl_hip_register_triggers",
-    "pccl_hip_set_option", "pccl_hip_get_option", "pccl_hip_execute", "pccl_hip_execute_inplace", "pccl_hip_sync",
+    "pccl_hip_set_option", "pccl_hip_get_option", "pccl_hip_execute", "pccl_hip_execute_inplace", "pccl_hip_execute_inplace_static", "pccl_hip_sync",
     "pccl_hip_reset_signals", "pccl_hip_op_info", "pccl_hip_last_kernel_ms", "pccl_hip_reduce",
     "pccl_hip_copy", "pccl_hip_last_error", "pccl_hip_version",
 ]
@@ -134,6 +134,7 @@ def lib() -> ctypes.CDLL:
         "pccl_hip_get_option": (i32, [vp, cp, ctypes.c_char_p, ctypes.c_size_t]),
         "pccl_hip_execute": (i32, [vp, cp, P(vp), P(vp), sz, sz, vp, i32]),
         "pccl_hip_execute_inplace": (i32, [vp, cp, P(vp), sz, vp, i32]),
+        "pccl_hip_execute_inplace_static": (i32, [vp, cp, P(vp), sz, vp, i32]),
         "pccl_hip_sync": (i32, [vp, cp]),
         "pccl_hip_reset_signals": (i32, [vp, cp]),
         "pccl_hip_op_info": (i32, [vp, cp, P(ProgramInfo)]),

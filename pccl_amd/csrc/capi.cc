@@ -4,6 +4,7 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <atomic>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -329,6 +330,7 @@ struct OpEntry {
         std::vector<DevGatherCopy> gather;
         std::vector<DevStepOp> step_ops;
         std::vector<int32_t> item_op;
+        std::vector<int32_t> step_deps_padded;   // the dependency lists padded to whole 8-byte words
     } host;
     DevBuf segs, direct_segs, instrs, pre, step_ops, step_deps, item_op, state;
     int64_t total_tiles = 0, direct_tiles = 0;
@@ -340,6 +342,8 @@ struct OpEntry {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool timed = false;
     bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
+    bool ran_static = false;              // the same for a launch in the static workspace
+    uint64_t generation = 0;              // which host link these tables come from (never reused in the process)
     int epoch = 0;                        // persistent runner: launches so far
     std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
     // Level runner: the launches of one execution captured as a HIP graph, per set of rank
@@ -563,7 +567,11 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
         e.level_item_begin.push_back((int)P.num_items);
         e.host.step_ops = std::move(so);
         e.host.item_op = std::move(item_op);
+        e.host.step_deps_padded = P.step_deps;
+        if (e.host.step_deps_padded.size() % 2) e.host.step_deps_padded.push_back(0);
     }
+    static std::atomic<uint64_t> link_counter{0};
+    e.generation = ++link_counter;
     e.host_linked = true;
     warn_about(P, "operation linked over " + std::to_string(ctx->R) + " virtual ranks", ctx->check_races);
     if (log_threshold() <= LOG_INFO)   // the reference's "Fused step executor enabled" line (engine_c.cc:357)
@@ -864,6 +872,56 @@ void check_stall(OpEntry& e, const std::string& name) {
                                   ") complete; rank buffers are partially updated"};
 }
 
+// ---- execution in the static workspace (no allocation anywhere in the call) -------------------
+//
+// What the persistent runner needs on the device besides the rank buffers - its progress block (error
+// words, one flag per work item, one ready word per op) and its tables (ops, dependency lists,
+// item -> op map) - laid out in the GPU's static workspace.  One such workspace exists per GPU and
+// every call on that GPU uses it, whichever context or operation it comes from: the host remembers
+// whose tables it holds and rewrites them when another operation takes it over.
+struct StaticWorkspace {
+    std::mutex mu;
+    char* ptr = nullptr;          // device address on this GPU (asked for at pccl_hip_create, with the device current)
+    size_t bytes = 0;
+    uint64_t owner = 0;           // OpEntry::generation whose tables the workspace holds (0: none)
+    int32_t epoch = 0;            // launches since the flags were last cleared
+};
+
+StaticWorkspace& static_ws(int device) {
+    static StaticWorkspace ws[16];
+    return ws[device >= 0 && device < 16 ? device : 0];
+}
+
+struct StaticLayout { size_t state, flags, ready, ops, deps, item_op, total; };
+
+StaticLayout static_layout(const Program& P) {
+    auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    StaticLayout l{};
+    l.state = 0;
+    l.flags = sizeof(StepState);                                   // flags and ready words follow the block directly,
+    l.ready = l.flags + sizeof(int32_t) * (size_t)P.num_items;      // as the kernel expects
+    l.ops = up(l.ready + sizeof(int32_t) * (P.ops.size() + 1));
+    l.deps = up(l.ops + sizeof(DevStepOp) * P.ops.size());
+    l.item_op = up(l.deps + sizeof(int32_t) * (P.step_deps.size() + 2));
+    l.total = up(l.item_op + sizeof(int32_t) * (size_t)P.num_items);
+    return l;
+}
+
+void check_stall_static(pccl_hip_ctx* ctx, OpEntry& e, const std::string& name) {
+    if (!e.ran_static) return;
+    e.ran_static = false;
+    StaticWorkspace& ws = static_ws(ctx->device);
+    std::lock_guard<std::mutex> lock(ws.mu);
+    if (!ws.ptr || ws.owner != e.generation) return;   // another operation has taken the workspace over since
+    StepState st;
+    HIP_TRY(hipMemcpy(&st, ws.ptr, sizeof(st), hipMemcpyDeviceToHost));
+    if (st.error_op == 0) return;
+    ws.owner = 0;                                      // the next call clears and rewrites everything
+    throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting in the static workspace (data op " +
+                                  std::to_string(st.error_op - 1) + " never saw its predecessor " + std::to_string(st.error_dep - 1) +
+                                  " complete); rank buffers are partially updated"};
+}
+
 int register_graph(pccl_hip_ctx* ctx, const char* name, int vrank, RankGraph&& g) {
     if (!ctx || !name) return fail(PCCL_ERR_INVALID, "null argument");
     if (vrank < 0 || vrank >= ctx->R) return fail(PCCL_ERR_INVALID, "virtual rank " + std::to_string(vrank) + " outside 0.." + std::to_string(ctx->R - 1));
@@ -898,6 +956,17 @@ int pccl_hip_create(pccl_hip_ctx** out, int device, int num_vranks) {
         ctx->device = device;
         ctx->R = num_vranks;
         ctx->bufs.assign(num_vranks, nullptr);
+        {   // the static workspace of this GPU: its address is asked for here, once per device, with the device current
+            StaticWorkspace& ws = static_ws(device);
+            std::lock_guard<std::mutex> lock(ws.mu);
+            if (!ws.ptr) {
+                void* p = nullptr;
+                size_t n = 0;
+                const int rc = static_workspace(device, &p, &n);
+                if (rc != 0) return fail(PCCL_ERR_HIP, std::string("static workspace: ") + hipGetErrorString((hipError_t)rc));
+                ws.ptr = (char*)p; ws.bytes = n;
+            }
+        }
         if (const char* nb = std::getenv("PCCL_NUM_BLOCKS")) ctx->num_blocks = std::atoi(nb);
         if (std::getenv("PCCL_DISABLE_FUSED")) ctx->mode = Mode::Stepwise;
         if (const char* tr = std::getenv("PCCL_TRACE_RANGES")) ctx->trace_ranges = std::atoi(tr) != 0;
@@ -1066,6 +1135,81 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
     });
 }
 
+int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
+                                    void* stream, int sync) {
+    return guarded([&] {
+        if (!ctx || !bufs) return fail(PCCL_ERR_INVALID, "null argument");
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        HIP_TRY(hipSetDevice(ctx->device));
+        OpEntry& e = find_entry(ctx, name);
+        link_host(ctx, e);                               // host memory only
+        const Program& P = e.prog;
+        hipStream_t s = (hipStream_t)stream;
+        StaticWorkspace& ws = static_ws(ctx->device);
+        std::lock_guard<std::mutex> wlock(ws.mu);
+        if (!ws.ptr) return fail(PCCL_ERR_HIP, "the static workspace of this GPU has no address");
+        const StaticLayout lay = static_layout(P);
+        if (lay.total > ws.bytes)
+            return fail(PCCL_ERR_INVALID, "operation '" + std::string(name) + "' needs " + std::to_string(lay.total) + " bytes of runner tables (" +
+                                              std::to_string(P.num_items) + " work items, " + std::to_string(P.ops.size()) + " data ops); the static workspace holds " +
+                                              std::to_string(ws.bytes) + ": use pccl_hip_execute_inplace, or larger work items (option step_tile_bytes)");
+        const size_t es = elem_size(P.dtype);
+        if ((size_t)P.buffer_elems * es > buf_bytes)
+            return fail(PCCL_ERR_INVALID, "rank buffers of " + std::to_string(buf_bytes) + " bytes are smaller than the " + std::to_string((size_t)P.buffer_elems * es) + " bytes the graph addresses");
+        RankPtrs ptrs;
+        std::memset(&ptrs, 0, sizeof(ptrs));
+        for (int r = 0; r < ctx->R; ++r) {
+            if (!bufs[r]) return fail(PCCL_ERR_INVALID, "null rank buffer " + std::to_string(r));
+            if ((uintptr_t)bufs[r] % es) return fail(PCCL_ERR_INVALID, "rank buffer " + std::to_string(r) + " is not aligned to the element size");
+            ptrs.p[r] = (char*)bufs[r];
+            ptrs.p[PCCL_HIP_MAX_VRANKS + r] = (char*)bufs[r];
+        }
+        if (P.ops.empty()) return 0;
+        const bool capturing = is_capturing(s);
+        int rc = 0;
+        if (ws.owner != e.generation || ws.epoch >= 0x3FFFFFF0) {
+            // the workspace holds another operation's tables (or nothing, or the launch numbers have run
+            // out): clear the progress block and write this operation's tables, all by kernels on `s`
+            if (capturing)
+                return fail(PCCL_ERR_INVALID, "the stream is capturing and the static workspace does not hold this operation's tables: "
+                                              "execute it once outside the capture first");
+            rc = launch_fill_zero(ws.ptr, lay.ops, s);   // a fill kernel, not a memset node (the block, the flags, the ready words)
+            if (!rc) rc = launch_table_write(e.host.step_ops.data(), e.host.step_ops.size() * sizeof(DevStepOp), ws.ptr + lay.ops, s);
+            if (!rc) rc = launch_table_write(e.host.step_deps_padded.data(), e.host.step_deps_padded.size() * sizeof(int32_t), ws.ptr + lay.deps, s);
+            if (!rc) rc = launch_item_op_fill((const DevStepOp*)(ws.ptr + lay.ops), (int)P.ops.size(), (int32_t*)(ws.ptr + lay.item_op), s);
+            if (rc) { ws.owner = 0; return fail(PCCL_ERR_HIP, std::string("writing the runner tables: ") + hipGetErrorString((hipError_t)rc)); }
+            ws.owner = e.generation;
+            ws.epoch = 0;
+        }
+        StepwiseLaunch L{};
+        L.ops = (const DevStepOp*)(ws.ptr + lay.ops); L.num_ops = (int)P.ops.size();
+        L.deps = (const int32_t*)(ws.ptr + lay.deps); L.item_op = (const int32_t*)(ws.ptr + lay.item_op);
+        L.num_items = (int)P.num_items; L.tile_elems = P.tile_elems; L.state = (StepState*)ws.ptr;
+        L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
+        L.epoch = capturing ? 0 : ++ws.epoch;            // recorded launches take their number from the device-side counter
+        L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
+        {
+            TraceRange exe(ctx->trace_ranges, "execute"), range(ctx->trace_ranges, "executor_kernel");
+            rc = launch_persistent(L, ptrs, s);
+        }
+        if (rc) { ws.owner = 0; return fail(PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)); }
+        e.ran_static = true;
+        ctx->last_stream = s;
+        if (sync) {
+            HIP_TRY(hipStreamSynchronize(s));
+            StepState st;
+            HIP_TRY(hipMemcpy(&st, ws.ptr, sizeof(st), hipMemcpyDeviceToHost));
+            e.ran_static = false;
+            if (st.error_op != 0) {
+                ws.owner = 0;
+                return fail(PCCL_ERR_HIP, "operation '" + std::string(name) + "': the persistent runner gave up waiting in the static workspace (data op " +
+                                              std::to_string(st.error_op - 1) + " never saw its predecessor " + std::to_string(st.error_dep - 1) + " complete)");
+            }
+        }
+        return 0;
+    });
+}
+
 int pccl_hip_sync(pccl_hip_ctx* ctx, const char* name) {
     return guarded([&] {
         if (!ctx) return fail(PCCL_ERR_INVALID, "null argument");
@@ -1075,6 +1219,7 @@ int pccl_hip_sync(pccl_hip_ctx* ctx, const char* name) {
         HIP_TRY(hipSetDevice(ctx->device));
         HIP_TRY(hipStreamSynchronize(ctx->last_stream));
         check_stall(it->second, it->first);
+        check_stall_static(ctx, it->second, it->first);
         return 0;
     });
 }

@@ -111,6 +111,14 @@ struct StageOffsets { int64_t src[PCCL_HIP_MAX_VRANKS]; int64_t dst[PCCL_HIP_MAX
 int launch_stage(const RankPtrs& src, const RankPtrs& dst, const StageOffsets& off, int R, size_t bytes, void* stream);
 int launch_fill_zero(void* dst, size_t nbytes, void* stream);
 
+// The static workspace of `device` (which must be the current device the first time): its device
+// address and size.  Returns a hipError_t value.
+int static_workspace(int device, void** ptr, size_t* bytes);
+// `nbytes` (a multiple of 8) of host memory to device memory at `dst` through kernel arguments.
+struct TablePayload { uint64_t w[448]; };   // 3.5 KiB: a kernel's arguments may take 4 KiB
+int launch_table_write(const void* src, size_t nbytes, void* dst, void* stream);
+int launch_item_op_fill(const DevStepOp* ops, int num_ops, int32_t* item_op, void* stream);
+
 int device_cu_count(int device);
 
 }  // namespace pccl_hip

@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstring>
 
 #include "kernels.h"
 
@@ -1270,6 +1271,73 @@ int launch_gather(const DevGatherCopy* copies, int n, int64_t total_tiles, int c
     if (n <= 0 || total_tiles <= 0) return 0;
     const int run = run_for_tiles(total_tiles);
     hipLaunchKernelGGL(gather_kernel, dim3(grid_for_tiles(total_tiles, run)), dim3(kThreads), 0, (hipStream_t)stream, copies, n, total_tiles, copy_tiles, src, dst, run);
+    return (int)hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------- static workspace
+//
+// Device memory of a stated, fixed size that exists from the moment the library is loaded: the
+// persistent runner's tables and progress block of a call that may not allocate live here.  Every
+// GPU the library runs on holds its own copy of the array at its own address; the array's name is
+// a host-side stand-in, not a device address, so host code asks the runtime for the address once
+// per device and from then on only ever uses that pointer.  Every call on a GPU shares that GPU's
+// array, which keeps the last call's contents.
+static __device__ __align__(256) unsigned char scratch[PCCL_HIP_STATIC_WORKSPACE_BYTES];
+
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int static_workspace(int device, void** ptr, size_t* bytes) {
+    if (device < 0 || device >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    void* p = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!p) {
+        int cur = -1;
+        hipError_t rc = hipGetDevice(&cur);
+        if (rc != hipSuccess) return (int)rc;
+        if (cur != device) return (int)hipErrorInvalidDevice;   // the address is asked for with its device current
+        rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (rc != hipSuccess) return (int)rc;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[device].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    *bytes = sizeof(scratch);
+    return 0;
+}
+
+// Table bytes carried to the device by the kernel arguments themselves: no copy engine, no staging
+// buffer, nothing allocated anywhere.
+__global__ __launch_bounds__(kThreads) void table_write_kernel(TablePayload payload, uint64_t* dst, int nwords) {
+    for (int i = threadIdx.x; i < nwords; i += kThreads) dst[i] = payload.w[i];
+}
+
+int launch_table_write(const void* src, size_t nbytes, void* dst, void* stream) {
+    if (nbytes % 8 || (uintptr_t)dst % 8) return (int)hipErrorInvalidValue;
+    const char* s = (const char*)src;
+    char* d = (char*)dst;
+    while (nbytes > 0) {
+        TablePayload payload;
+        const size_t n = nbytes < sizeof(payload.w) ? nbytes : sizeof(payload.w);
+        std::memcpy(payload.w, s, n);
+        hipLaunchKernelGGL(table_write_kernel, dim3(1), dim3(kThreads), 0, (hipStream_t)stream, payload, (uint64_t*)d, (int)(n / 8));
+        hipError_t rc = hipGetLastError();
+        if (rc != hipSuccess) return (int)rc;
+        s += n; d += n; nbytes -= n;
+    }
+    return 0;
+}
+
+// item -> op map of the stepwise plan, rebuilt on the device from the op table (op k owns items
+// [first_item, first_item + ntiles)).
+__global__ __launch_bounds__(kThreads) void item_op_fill_kernel(const DevStepOp* ops, int num_ops, int32_t* item_op) {
+    for (int k = blockIdx.x; k < num_ops; k += gridDim.x) {
+        const int first = ops[k].first_item, n = ops[k].ntiles;
+        for (int t = threadIdx.x; t < n; t += kThreads) item_op[first + t] = k;
+    }
+}
+
+int launch_item_op_fill(const DevStepOp* ops, int num_ops, int32_t* item_op, void* stream) {
+    if (num_ops <= 0) return 0;
+    hipLaunchKernelGGL(item_op_fill_kernel, dim3(num_ops < 1024 ? num_ops : 1024), dim3(kThreads), 0, (hipStream_t)stream, ops, num_ops, item_op);
     return (int)hipGetLastError();
 }
 

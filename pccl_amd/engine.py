@@ -166,6 +166,16 @@ class Engine:
                                                     _current_stream_ptr(self.device), int(sync)))
         return bs
 
+    def execute_inplace_static(self, name: str, bufs: TensorList, sync: bool = False):
+        """``execute_inplace`` for callers that cannot allocate: one launch of the persistent runner in
+        the GPU's static workspace (see ``pccl_hip_execute_inplace_static``).  No counterpart in the
+        reference."""
+        bs = self._as_list(bufs, "bufs")
+        self._check_dtype(name, bs, "bufs")
+        _lib.check(self._L.pccl_hip_execute_inplace_static(self._h, name.encode(), self._ptrs(bs), min(b.nbytes for b in bs),
+                                                           _current_stream_ptr(self.device), int(sync)))
+        return bs
+
     def prepare(self, name: str, inputs: TensorList, outputs: Optional[TensorList] = None) -> "PreparedCall":
         """Check the tensors and build the argument arrays once; the returned object launches the
         operation on those tensors with nothing but the C call per invocation (for loops that issue

@@ -1,0 +1,104 @@
+"""pccl_hip_execute_inplace_static: the in-place execution for callers that cannot allocate.  Called
+through the C ABI and compared bit for bit with pccl_hip_execute_inplace on the same inputs, on
+calls in a row that share the GPU's static workspace: a larger operation, then a smaller one (whose
+tables replace the first one's and whose flags must not be confused with what the first left
+behind), then the first again, then repeated launches of one operation."""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import bits_equal, graph_jsons, mismatch_report, seeded_inputs
+from pccl_amd import _lib
+from pccl_amd._lib import ERR_INVALID
+
+pytestmark = pytest.mark.gpu
+
+
+def _ptrs(ts):
+    return (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _register(L, h, name, jsons):
+    for r, j in enumerate(jsons):
+        data = j.encode()
+        _lib.check(L.pccl_hip_register_json(h, name.encode(), r, data, len(data)))
+
+
+def test_static_workspace_execution_matches_the_allocating_entry_point():
+    L = _lib.lib()
+    world = 8
+    h = ctypes.c_void_p()
+    _lib.check(L.pccl_hip_create(ctypes.byref(h), 0, world))
+    try:
+        cases = {   # name -> (graphs, elements per rank, dtype, input kind)
+            "large": (graph_jsons("ring", "build_allreduce", world, 1 << 20, "bfloat16", "sm", 2), 1 << 20, "bfloat16", "randn"),
+            "small": (graph_jsons("rhd", "build_allreduce", world, 3 * 4096, "float32", "sm", 1), 3 * 4096, "float32", "randn"),
+            "tree": (graph_jsons("tree", "build_allreduce", world, 40000, "int32", "sm", 1, reduce_op="max"), 40000, "int32", "randint"),
+        }
+        inputs, want = {}, {}
+        for name, (jsons, n, dtype, kind) in cases.items():
+            _register(L, h, name, jsons)
+            inputs[name] = [t.cuda() for t in seeded_inputs(kind, world, n, dtype, seed=len(name))]
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+
+        def run_static(name):
+            bufs = [t.clone() for t in inputs[name]]
+            _lib.check(L.pccl_hip_execute_inplace_static(h, name.encode(), _ptrs(bufs), bufs[0].nbytes, _stream(), 1))
+            return bufs
+
+        # the static entry point first, on operations that have never been linked on the device
+        print("static: large, then small, then large again", flush=True)
+        got = {"large": run_static("large")}
+        got["small"] = run_static("small")            # the second call, on a smaller input
+        got["large2"] = run_static("large")
+        got["tree"] = run_static("tree")
+        torch.cuda.synchronize()
+        # nothing of the device's memory was taken by those calls beyond the clones made here
+        clones = sum(t.nbytes for bufs in got.values() for t in bufs)
+        assert free_before - torch.cuda.mem_get_info()[0] <= clones + (64 << 20), "the static entry point seems to have allocated"
+
+        # the existing entry point on the same inputs (persistent runner and the default runner)
+        for mode in ("persistent", "auto"):
+            _lib.check(L.pccl_hip_set_option(h, b"mode", mode.encode()))
+            for name in cases:
+                bufs = [t.clone() for t in inputs[name]]
+                _lib.check(L.pccl_hip_execute_inplace(h, name.encode(), _ptrs(bufs), bufs[0].nbytes, _stream(), 1))
+                want[name] = bufs
+                keys = [name, "large2"] if name == "large" else [name]
+                for key in keys:
+                    for r in range(world):
+                        assert bits_equal(got[key][r], bufs[r]), f"{key} vs execute_inplace ({mode}), rank {r}: {mismatch_report(got[key][r], bufs[r])}"
+
+        # many launches in a row of one operation, alternating with another: flags of earlier launches
+        # must never satisfy a later one
+        print("static: 40 launches alternating between two operations", flush=True)
+        for i in range(40):
+            name = "small" if i % 3 else "tree"
+            bufs = run_static(name)
+            for r in range(world):
+                assert bits_equal(bufs[r], want[name][r]), f"launch {i} ({name}), rank {r}"
+
+        # asynchronous launches followed by pccl_hip_sync
+        bufs = [t.clone() for t in inputs["small"]]
+        _lib.check(L.pccl_hip_execute_inplace_static(h, b"small", _ptrs(bufs), bufs[0].nbytes, _stream(), 0))
+        _lib.check(L.pccl_hip_sync(h, b"small"))
+        for r in range(world):
+            assert bits_equal(bufs[r], want["small"][r])
+
+        # limits: rank buffers too small, and an operation whose tables exceed the workspace
+        small_bufs = [t[:100].clone() for t in inputs["large"]]
+        assert L.pccl_hip_execute_inplace_static(h, b"large", _ptrs(small_bufs), small_bufs[0].nbytes, _stream(), 1) == ERR_INVALID
+        assert b"smaller than" in L.pccl_hip_last_error()
+        _lib.check(L.pccl_hip_set_option(h, b"step_tile_bytes", b"4096"))
+        _register(L, h, "huge", graph_jsons("ring", "build_allreduce", world, 1 << 27, "bfloat16", "sm", 4))
+        rc = L.pccl_hip_execute_inplace_static(h, b"huge", _ptrs(small_bufs), small_bufs[0].nbytes, _stream(), 1)
+        assert rc == ERR_INVALID and b"static workspace holds" in L.pccl_hip_last_error(), L.pccl_hip_last_error()
+        assert L.pccl_hip_execute_inplace_static(h, b"nope", _ptrs(small_bufs), 200, _stream(), 1) == _lib.ERR_NOT_FOUND
+    finally:
+        L.pccl_hip_destroy(h)
