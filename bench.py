@@ -357,7 +357,18 @@ def run_inplace(args, wl: Workload, dev) -> int:
     t0 = time.perf_counter()
     pristine = wl.make_inputs()
     log(f"inputs generated in {time.perf_counter() - t0:.1f} s")
-    bufs = [p.clone() for p in pristine]
+    if args.rank_skew_bytes:
+        # rank buffers carved out of one allocation, rank r starting r * (size + skew) bytes in: the same
+        # position of different ranks then falls on different memory channels
+        es = pristine[0].element_size()
+        stride = wl.n + args.rank_skew_bytes // es
+        arena = torch.empty(wl.world * stride, dtype=pristine[0].dtype, device=dev)
+        bufs = [arena[r * stride:r * stride + wl.n] for r in range(wl.world)]
+        for b, p in zip(bufs, pristine):
+            b.copy_(p)
+    else:
+        bufs = [p.clone() for p in pristine]
+    log("rank buffer addresses: " + " ".join(hex(b.data_ptr()) for b in bufs[:4]) + " ...")
 
     # the first execution in the process (tables just uploaded, nothing of the buffers in any cache)
     c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -476,6 +487,14 @@ def run_c4(args, dev) -> int:
     if args.c4_bytes:
         sizes = [int(s) for s in args.c4_bytes.split(",")]
     g = torch.Generator(device="cuda").manual_seed(0)
+    if args.calibrate_copy_bytes:
+        from pccl_amd import _lib
+        src = torch.empty(args.calibrate_copy_bytes, dtype=torch.uint8, device=dev).random_(0, 256)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(_lib.lib().pccl_hip_copy(3, src.data_ptr(), dst.data_ptr(), src.numel(), None))
+        torch.cuda.synchronize()
+        del src, dst
     for nbytes in sizes:
         n = nbytes // 2
         chunk = n // world
@@ -508,7 +527,7 @@ def run_c4(args, dev) -> int:
                 avg = sum(ms) / len(ms)
                 hbm, note = moved_bytes(info, args.mode, staged=True)
                 if args.mode in ("stepwise", "persistent"):
-                    hbm += 2 * world * (in_elems + out_elems)      # the two batched staging copies, read + write, 2 bytes per element
+                    hbm += 2 * 2 * world * (in_elems + out_elems)  # the two batched staging copies: read + write, 2 bytes per element
                     note += " plus the input and output staging copies"
                 print(json.dumps({
                     "metric": METRIC + f", ring {method[6:]} R8 fp16 staged call", "value": round(hbm / (wall_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
@@ -544,6 +563,8 @@ def main() -> int:
     ap.add_argument("--num-blocks", type=int, default=-1)
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
                     help="engine option to set before the run (e.g. lds_slots=0, slot_threads=128); repeatable")
+    ap.add_argument("--rank-skew-bytes", type=int, default=0,
+                    help="carve the rank buffers out of one allocation, each this many bytes further in than its size")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--no-side-legs", action="store_true", help="skip the op-by-op and single-launch legs of an auto-mode run")
