@@ -45,8 +45,9 @@
  *                      and offsets that are not multiples of 16 bytes have no defined reference
  *                      result.  This oracle processes all n elements at any alignment.  EXTENSION,
  *                      parity unpinned by the reference; pinned by closed forms.
- *   MAX / MIN, int32   the reference runtime ignores reduce_op and rejects int32.  EXTENSION, pinned
- *                      by torch amax/amin/sum over the stacked inputs.
+ *   MAX / MIN, int32   the reference runtime ignores reduce_op and rejects int32.  EXTENSION: MAX and
+ *                      MIN are IEEE 754-2019 maximum / minimum (NaN propagates, -0 < +0), pinned by
+ *                      torch maximum / minimum / amax / amin and by known answers for the zeros.
  *
  * Build: gcc -O2 -fopenmp -shared -fPIC (see oracle/build.py).  No dependency on ROCm or torch.
  */
@@ -164,13 +165,18 @@ static inline uint16_t oracle_add_f16(uint16_t a, uint16_t b) {
     return f32_to_f16_rne(f16_to_f32(a) + f16_to_f32(b));
 }
 
-/* MAX / MIN (extension): NaN-propagating, result NaN is canonical. */
+/* MAX / MIN (extension): IEEE 754-2019 maximum / minimum.  A NaN operand gives NaN (canonical);
+ * -0 orders below +0, so the result does not depend on the order of the operands.  Operands that
+ * compare equal are either bit-identical or the two zeros: AND of the bit patterns keeps +0 for the
+ * maximum, OR keeps -0 for the minimum, and both leave identical patterns alone. */
 static inline float sel_max_f32(float a, float b) {
     if (a != a || b != b) return u2f(0x7FFFFFFFu);
+    if (a == b) return u2f(f2u(a) & f2u(b));
     return a > b ? a : b;
 }
 static inline float sel_min_f32(float a, float b) {
     if (a != a || b != b) return u2f(0x7FFFFFFFu);
+    if (a == b) return u2f(f2u(a) | f2u(b));
     return a < b ? a : b;
 }
 

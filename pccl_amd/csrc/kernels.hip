@@ -44,12 +44,28 @@ template <int DT> struct ElemBytes { static constexpr int value = (DT == PCCL_F3
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
 
+// MAX / MIN are IEEE 754-2019 maximum / minimum: a NaN operand gives NaN (written canonically, like
+// every NaN result here) and -0 orders below +0.  gfx950 has both as one instruction
+// (v_maximum3_f32 / v_minimum3_f32 and their packed f16 forms).
+template <int OP>
+__device__ __forceinline__ float f32_comb(float a, float b) {
+    if constexpr (OP == PCCL_SUM) return a + b;
+    else if constexpr (OP == PCCL_MAX) return __builtin_elementwise_maximum(a, b);
+    else return __builtin_elementwise_minimum(a, b);
+}
+template <int OP>
+__device__ __forceinline__ h2 f16x2_comb(h2 a, h2 b) {
+    if constexpr (OP == PCCL_SUM) return a + b;
+    else if constexpr (OP == PCCL_MAX) return __builtin_elementwise_maximum(a, b);
+    else return __builtin_elementwise_minimum(a, b);
+}
+__device__ __forceinline__ float f32_comb(float a, float b, int redop) {
+    return redop == PCCL_SUM ? f32_comb<PCCL_SUM>(a, b) : redop == PCCL_MAX ? f32_comb<PCCL_MAX>(a, b) : f32_comb<PCCL_MIN>(a, b);
+}
+
 __device__ __forceinline__ uint32_t f32_op(uint32_t ua, uint32_t ub, int redop) {
-    const float a = as_f32(ua), b = as_f32(ub);
-    if (redop == PCCL_SUM) { const float r = a + b; return (r != r) ? 0x7FFFFFFFu : as_u32(r); }
-    // one unordered compare, one ordered compare, two selects on the bit patterns
-    const uint32_t pick = redop == PCCL_MAX ? (a > b ? ua : ub) : (a < b ? ua : ub);
-    return __builtin_isunordered(a, b) ? 0x7FFFFFFFu : pick;
+    const float r = f32_comb(as_f32(ua), as_f32(ub), redop);
+    return (r != r) ? 0x7FFFFFFFu : as_u32(r);
 }
 
 // float -> bf16 bits in the HIGH half of the result, round to nearest even, canonical NaN
@@ -59,29 +75,16 @@ __device__ __forceinline__ uint32_t bf16_round_hi(float f) {
     return (f != f) ? 0x7FFF0000u : (r & 0xFFFF0000u);
 }
 
-__device__ __forceinline__ float bf16_sel(float a, float b, int redop) {
-    if (redop == PCCL_SUM) return a + b;
-    if (a != a || b != b) return as_f32(0x7FFFFFFFu);
-    return redop == PCCL_MAX ? (a > b ? a : b) : (a < b ? a : b);
-}
-
 __device__ __forceinline__ uint32_t bf16x2_op(uint32_t a, uint32_t b, int redop) {
-    float lo = bf16_sel(as_f32(a << 16), as_f32(b << 16), redop);
-    float hi = bf16_sel(as_f32(a & 0xFFFF0000u), as_f32(b & 0xFFFF0000u), redop);
+    // a selected value is a bf16 already, so the rounding below only acts on sums
+    float lo = f32_comb(as_f32(a << 16), as_f32(b << 16), redop);
+    float hi = f32_comb(as_f32(a & 0xFFFF0000u), as_f32(b & 0xFFFF0000u), redop);
     return bf16_round_hi(hi) | (bf16_round_hi(lo) >> 16);
 }
 
 __device__ __forceinline__ uint32_t f16x2_op(uint32_t ua, uint32_t ub, int redop) {
-    h2 a = __builtin_bit_cast(h2, ua), b = __builtin_bit_cast(h2, ub), r;
-    if (redop == PCCL_SUM) r = a + b;
-    else {
-        for (int k = 0; k < 2; ++k) {
-            _Float16 x = a[k], y = b[k];
-            bool nan = (x != x) || (y != y);
-            _Float16 m = redop == PCCL_MAX ? (x > y ? x : y) : (x < y ? x : y);
-            r[k] = nan ? __builtin_bit_cast(_Float16, (uint16_t)0x7FFF) : m;
-        }
-    }
+    const h2 a = __builtin_bit_cast(h2, ua), b = __builtin_bit_cast(h2, ub);
+    const h2 r = redop == PCCL_SUM ? f16x2_comb<PCCL_SUM>(a, b) : redop == PCCL_MAX ? f16x2_comb<PCCL_MAX>(a, b) : f16x2_comb<PCCL_MIN>(a, b);
     uint32_t u = __builtin_bit_cast(uint32_t, r);
     if (r[0] != r[0]) u = (u & 0xFFFF0000u) | 0x7FFFu;
     if (r[1] != r[1]) u = (u & 0x0000FFFFu) | 0x7FFF0000u;
@@ -105,12 +108,10 @@ __device__ __forceinline__ uint32_t fp8_pair_op(uint32_t x, uint32_t y, uint32_t
         // the float sum of two f16-representable values rounds to f16 exactly as their f16 sum
         r0 = (float)(_Float16)(a.x + b.x);
         r1 = (float)(_Float16)(a.y + b.y);
-    } else if (redop == PCCL_MAX) {
-        r0 = a.x > b.x ? a.x : b.x; r1 = a.y > b.y ? a.y : b.y;
     } else {
-        r0 = a.x < b.x ? a.x : b.x; r1 = a.y < b.y ? a.y : b.y;
+        r0 = f32_comb(a.x, b.x, redop); r1 = f32_comb(a.y, b.y, redop);
     }
-    const bool n0 = (r0 != r0) || __builtin_isunordered(a.x, b.x), n1 = (r1 != r1) || __builtin_isunordered(a.y, b.y);
+    const bool n0 = r0 != r0, n1 = r1 != r1;
     r0 = n0 ? 0.0f : __builtin_fminf(__builtin_fmaxf(r0, -kMax), kMax);
     r1 = n1 ? 0.0f : __builtin_fminf(__builtin_fmaxf(r1, -kMax), kMax);
     if constexpr (E5M2) out = __builtin_amdgcn_cvt_pk_bf8_f32(r0, r1, out, HI);
@@ -155,18 +156,18 @@ __device__ __forceinline__ u32x4 vec_op_words(u32x4 a, u32x4 b, int redop) {
     return r;
 }
 
-// Sums of whole vectors take a shorter road than word_op: the arithmetic runs as if no NaN could
+// Whole vectors take a shorter road than word_op: the arithmetic runs as if no NaN could
 // come out, one unordered compare per pair of results notes whether one did, and only lanes that
 // saw one go back and canonicalise (rare: the branch is skipped by the whole wave otherwise).
 // The results are those of word_op bit for bit.  bf16 rounds with v_cvt_pk_bf16_f32, which was
 // checked on this GPU against the integer form of bf16_round_hi for every non-NaN float.
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
-template <int DT>
-__device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
+template <int DT, int OP>
+__device__ __forceinline__ u32x4 vec_fast(u32x4 a, u32x4 b) {
     if constexpr (DT == PCCL_F32) {
-        const float r0 = as_f32(a.x) + as_f32(b.x), r1 = as_f32(a.y) + as_f32(b.y);
-        const float r2 = as_f32(a.z) + as_f32(b.z), r3 = as_f32(a.w) + as_f32(b.w);
+        const float r0 = f32_comb<OP>(as_f32(a.x), as_f32(b.x)), r1 = f32_comb<OP>(as_f32(a.y), as_f32(b.y));
+        const float r2 = f32_comb<OP>(as_f32(a.z), as_f32(b.z)), r3 = f32_comb<OP>(as_f32(a.w), as_f32(b.w));
         u32x4 r = {as_u32(r0), as_u32(r1), as_u32(r2), as_u32(r3)};
         // one compare per pair of results, combined on the scalar side: the whole wave takes the
         // repair branch if any lane saw a NaN (the repairs themselves are per element)
@@ -184,8 +185,8 @@ __device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
         uint32_t rw[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float lo = as_f32(aw[i] << 16) + as_f32(bw[i] << 16);
-            const float hi = as_f32(aw[i] & 0xFFFF0000u) + as_f32(bw[i] & 0xFFFF0000u);
+            const float lo = f32_comb<OP>(as_f32(aw[i] << 16), as_f32(bw[i] << 16));
+            const float hi = f32_comb<OP>(as_f32(aw[i] & 0xFFFF0000u), as_f32(bw[i] & 0xFFFF0000u));
             nan |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(lo, hi));
             const f32x2 pair = {lo, hi};
             rw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
@@ -205,7 +206,7 @@ __device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
         uint64_t nan = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const h2 s = __builtin_bit_cast(h2, aw[i]) + __builtin_bit_cast(h2, bw[i]);
+            const h2 s = f16x2_comb<OP>(__builtin_bit_cast(h2, aw[i]), __builtin_bit_cast(h2, bw[i]));
             nan |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(s[0], s[1]));
             rw[i] = __builtin_bit_cast(uint32_t, s);
         }
@@ -219,7 +220,7 @@ __device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
         u32x4 r = {rw[0], rw[1], rw[2], rw[3]};
         return r;
     } else {
-        return vec_op_words<DT>(a, b, PCCL_SUM);
+        return vec_op_words<DT>(a, b, OP);
     }
 }
 
@@ -227,9 +228,9 @@ __device__ __forceinline__ u32x4 vec_sum(u32x4 a, u32x4 b) {
 // constant operator, so the four words run back to back without tests in between.
 template <int DT>
 __device__ __forceinline__ u32x4 vec_op(u32x4 a, u32x4 b, int redop) {
-    if (redop == PCCL_SUM) return vec_sum<DT>(a, b);
-    if (redop == PCCL_MAX) return vec_op_words<DT>(a, b, PCCL_MAX);
-    return vec_op_words<DT>(a, b, PCCL_MIN);
+    if (redop == PCCL_SUM) return vec_fast<DT, PCCL_SUM>(a, b);
+    if (redop == PCCL_MAX) return vec_fast<DT, PCCL_MAX>(a, b);
+    return vec_fast<DT, PCCL_MIN>(a, b);
 }
 
 // one element at byte address granularity (heads, tails, partial vectors, misaligned ranges)

@@ -52,6 +52,40 @@ def test_reduce_matches_oracle(dtype, redop, n):
     assert bits_equal(dc, want), mismatch_report(dc, want)
 
 
+EDGE_F32 = [0x00000000, 0x80000000, 0x00000001, 0x80000001, 0x007FFFFF, 0x807FFFFF, 0x00800000, 0x80800000,
+            0x3F800000, 0xBF800000, 0x3F800001, 0x3F7FFFFF, 0x7F7FFFFF, 0xFF7FFFFF, 0x7F800000, 0xFF800000,
+            0x7F800001, 0x7FC00000, 0xFFC00000, 0x7FFFFFFF, 0xFFFFFFFF, 0x7FA00000, 0x4B800000, 0x4B7FFFFF,
+            0x33800000, 0x33FFFFFF, 0x7F000000, 0xFF000000, 0x00400000, 0x80400000, 0x40490FDB, 0xC0490FDB]
+EDGE_F16 = [0x0000, 0x8000, 0x0001, 0x8001, 0x03FF, 0x83FF, 0x0400, 0x8400, 0x3C00, 0xBC00, 0x3C01, 0x3BFF,
+            0x7BFF, 0xFBFF, 0x7C00, 0xFC00, 0x7C01, 0x7E00, 0xFE00, 0x7FFF, 0xFFFF, 0x7D00, 0x6400, 0x63FF,
+            0x1400, 0x17FF, 0x7800, 0xF800, 0x0200, 0x8200, 0x4248, 0xC248]
+EDGE_BF16 = [0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x807F, 0x0080, 0x8080, 0x3F80, 0xBF80, 0x3F81, 0x3F7F,
+             0x7F7F, 0xFF7F, 0x7F80, 0xFF80, 0x7F81, 0x7FC0, 0xFFC0, 0x7FFF, 0xFFFF, 0x7FA0, 0x4380, 0x437F,
+             0x3B80, 0x3BFF, 0x7F00, 0xFF00, 0x0040, 0x8040, 0x4049, 0xC049]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("redop", ["sum", "max", "min"])
+@pytest.mark.parametrize("lead", [0, 1])
+def test_reduce_every_pair_of_edge_values(dtype, redop, lead):
+    """Both zeros, the smallest and largest denormals and normals, neighbours of 1, infinities, quiet
+    and signalling NaNs with several payloads, values whose sum rounds at the last place: all 1,024
+    ordered pairs, bit for bit against the oracle.  `lead` = 1 shifts the operands one element off
+    16-byte alignment so that the element-wise edge code runs the same pairs as the vector body."""
+    codes = {"float32": EDGE_F32, "float16": EDGE_F16, "bfloat16": EDGE_BF16}[dtype]
+    raw = np.uint32 if dtype == "float32" else np.uint16
+    c = np.array(codes, dtype=raw)
+    a = np.concatenate([np.zeros(lead, raw), np.repeat(c, len(c))])
+    b = np.concatenate([np.zeros(lead, raw), np.tile(c, len(c))])
+    want = oracle.reduce(dtype, redop, a[lead:].copy(), b[lead:].copy())
+    ta, tb = from_raw(a, dtype).cuda(), from_raw(b, dtype).cuda()
+    tc = torch.empty_like(ta)
+    gpu_reduce(dtype, redop, ta[lead:], tb[lead:], tc[lead:])
+    got = to_raw(tc[lead:].cpu())
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, [(hex(int(a[lead + i])), hex(int(b[lead + i])), hex(int(got[i])), hex(int(want[i]))) for i in bad[:8]]
+
+
 @pytest.mark.parametrize("dtype", ["float8_e4m3", "float8_e5m2"])
 @pytest.mark.parametrize("redop", ["sum", "max", "min"])
 def test_fp8_reduce_all_operand_pairs(dtype, redop):

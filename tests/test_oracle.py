@@ -112,6 +112,20 @@ def test_max_min_match_torch(dtype, redop):
         assert torch.equal(got[~nan], want[~nan])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16"])
+def test_max_min_order_the_two_zeros(dtype):
+    """IEEE 754-2019 maximum / minimum: -0 orders below +0 whatever the operand order (torch and numpy
+    leave the sign of such a tie to the operand order, so this is pinned by its known answers), and
+    equal operands come back unchanged."""
+    neg = {"float32": 0x80000000, "float16": 0x8000, "bfloat16": 0x8000}[dtype]
+    one = {"float32": 0x3F800000, "float16": 0x3C00, "bfloat16": 0x3F80}[dtype]
+    raw = np.uint32 if dtype == "float32" else np.uint16
+    a = np.array([0, neg, 0, neg, one, one | neg], dtype=raw)
+    b = np.array([neg, 0, 0, neg, one, one | neg], dtype=raw)
+    assert oracle.reduce(dtype, "max", a, b).tolist() == [0, 0, 0, neg, one, one | neg]
+    assert oracle.reduce(dtype, "min", a, b).tolist() == [neg, neg, 0, neg, one, one | neg]
+
+
 @pytest.mark.parametrize("dtype", ["float8_e4m3", "float8_e5m2"])
 def test_fp8_sum_all_pairs_match_torch(dtype):
     """Reference vec.h:272-426: widen to f16, one f16 add, narrow with round-to-nearest-even and
