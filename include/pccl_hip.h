@@ -276,7 +276,12 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
  * shared by all contexts and operations and keeping the last call's contents: when another operation
  * used it last, this call first clears the progress block and rewrites the tables (by kernels on
  * `stream`), which it refuses to do on a capturing stream (execute once outside the capture first).
- * Calls that overlap in time on one GPU - two streams, two threads - race on the workspace. */
+ * Calls that overlap in time on one GPU - two streams, two threads - race on the workspace.
+ * A recorded launch stays valid while the workspace holds its operation's tables.  Replayed after
+ * another operation has taken the workspace over it executes nothing (the kernel compares a tag in
+ * its arguments with the one in the workspace before it reads any table) and the next synchronous
+ * call or pccl_hip_sync on that GPU's workspace returns PCCL_ERR_INVALID saying so; execute the
+ * operation once more through this entry point and the recorded launch works again. */
 int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
                                     void* stream, int sync);
 /* Engine::syncOp / Engine::resetSignals (reference csrc/engine_c.cc:562-593). */

@@ -892,6 +892,9 @@ StaticWorkspace& static_ws(int device) {
     return ws[device >= 0 && device < 16 ? device : 0];
 }
 
+// What StepState::owner holds while the workspace carries the tables of `e`: never 0.
+uint32_t static_tag(const OpEntry& e) { return (uint32_t)(e.generation & 0x7FFFFFFFu) | 0x80000000u; }
+
 struct StaticLayout { size_t state, flags, ready, ops, deps, item_op, total; };
 
 StaticLayout static_layout(const Program& P) {
@@ -907,6 +910,15 @@ StaticLayout static_layout(const Program& P) {
     return l;
 }
 
+// A recorded launch that was replayed after the workspace had gone to another operation has left
+// its tag behind (it executed nothing).  Say so once, at the next look at the block.
+void report_stale_launch(StaticWorkspace& ws, const StepState& st) {
+    if (st.stale_owner == 0) return;
+    ws.owner = 0;                                      // the next call clears the block, this word included
+    throw Error{PCCL_ERR_INVALID, "a recorded launch of pccl_hip_execute_inplace_static was replayed after the static workspace had been taken over "
+                                  "by another operation; it executed nothing.  Execute the operation once through this entry point and record it again"};
+}
+
 void check_stall_static(pccl_hip_ctx* ctx, OpEntry& e, const std::string& name) {
     if (!e.ran_static) return;
     e.ran_static = false;
@@ -915,6 +927,7 @@ void check_stall_static(pccl_hip_ctx* ctx, OpEntry& e, const std::string& name) 
     if (!ws.ptr || ws.owner != e.generation) return;   // another operation has taken the workspace over since
     StepState st;
     HIP_TRY(hipMemcpy(&st, ws.ptr, sizeof(st), hipMemcpyDeviceToHost));
+    report_stale_launch(ws, st);
     if (st.error_op == 0) return;
     ws.owner = 0;                                      // the next call clears and rewrites everything
     throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting in the static workspace (data op " +
@@ -1177,6 +1190,9 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
             if (!rc) rc = launch_table_write(e.host.step_ops.data(), e.host.step_ops.size() * sizeof(DevStepOp), ws.ptr + lay.ops, s);
             if (!rc) rc = launch_table_write(e.host.step_deps_padded.data(), e.host.step_deps_padded.size() * sizeof(int32_t), ws.ptr + lay.deps, s);
             if (!rc) rc = launch_item_op_fill((const DevStepOp*)(ws.ptr + lay.ops), (int)P.ops.size(), (int32_t*)(ws.ptr + lay.item_op), s);
+            // last: the block now belongs to this operation (StepState::owner, and a zero launch counter beside it)
+            const uint64_t head = static_tag(e);
+            if (!rc) rc = launch_table_write(&head, sizeof(head), ws.ptr, s);
             if (rc) { ws.owner = 0; return fail(PCCL_ERR_HIP, std::string("writing the runner tables: ") + hipGetErrorString((hipError_t)rc)); }
             ws.owner = e.generation;
             ws.epoch = 0;
@@ -1187,6 +1203,7 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
         L.num_items = (int)P.num_items; L.tile_elems = P.tile_elems; L.state = (StepState*)ws.ptr;
         L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
         L.epoch = capturing ? 0 : ++ws.epoch;            // recorded launches take their number from the device-side counter
+        L.owner_tag = static_tag(e);                     // a replay that finds another operation's tables does nothing
         L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
         {
             TraceRange exe(ctx->trace_ranges, "execute"), range(ctx->trace_ranges, "executor_kernel");
@@ -1200,6 +1217,7 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
             StepState st;
             HIP_TRY(hipMemcpy(&st, ws.ptr, sizeof(st), hipMemcpyDeviceToHost));
             e.ran_static = false;
+            report_stale_launch(ws, st);
             if (st.error_op != 0) {
                 ws.owner = 0;
                 return fail(PCCL_ERR_HIP, "operation '" + std::string(name) + "': the persistent runner gave up waiting in the static workspace (data op " +

@@ -49,11 +49,12 @@ struct DevStepOp {    // 64 bytes: one 16-dword scalar load
 static_assert(sizeof(DevStepOp) == 64, "DevStepOp is read with one scalar load");
 
 struct StepState {      // device memory of the persistent runner
-    uint32_t reserved0;
+    uint32_t owner;        // shared (static) block: tag of the operation whose tables follow; 0 for an operation's own block
     int32_t graph_epoch;   // launch number of the last launch recorded into a graph (see StepwiseLaunch::epoch)
     int32_t error_op;   // 1 + index of the op whose bounded wait expired (0 = none); host clears it
     int32_t error_dep;  // 1 + index of the predecessor it was waiting for
-    int32_t pad[28];
+    uint32_t stale_owner;  // tag of a launch that found another operation's tables in a shared block and did nothing
+    int32_t pad[27];
     // followed by int32 flag[num_items] (the epoch of the launch that last completed the item) and
     // int32 ready[num_ops] (the epoch of the launch in which the op's first tile last saw all predecessors done)
 };
@@ -89,7 +90,7 @@ struct StepwiseLaunch {
     int32_t num_blocks;
     int32_t epoch;            // persistent runner: value a completed item's flag takes in this launch;
                               // 0: take it from StepState::graph_epoch, which the launcher advances first
-    uint32_t reserved1;
+    uint32_t owner_tag;       // persistent runner in a shared block: run only if StepState::owner equals this (0: no check)
     uint64_t timeout_ticks;   // persistent runner: 100 MHz ticks a workgroup may run before a wait gives up
 };
 

@@ -600,6 +600,14 @@ void persistent_kernel(StepwiseLaunch L, RankPtrs ptrs) {
     // the one-thread kernel recorded in front of this one has just advanced.
     const int32_t epoch = L.epoch != 0 ? L.epoch
                                        : __hip_atomic_load(&L.state->graph_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // A launch that works in a block shared between operations - a recorded launch may be replayed
+    // long after it was recorded - first makes sure that the tables behind the block are still its
+    // own: its item count, kernel arguments, would otherwise index another operation's tables.
+    // Wave-uniform, before any barrier: every thread of every workgroup leaves.
+    if (L.owner_tag != 0 && __hip_atomic_load(&L.state->owner, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != L.owner_tag) {
+        if (blockIdx.x == 0 && tid == 0) __hip_atomic_store(&L.state->stale_owner, L.owner_tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
     if (tid == 0) s_stalled = 0;
     __syncthreads();
     // The loop is software-pipelined over the workgroup's items: the descriptor of the next item and

@@ -102,3 +102,69 @@ def test_static_workspace_execution_matches_the_allocating_entry_point():
         assert L.pccl_hip_execute_inplace_static(h, b"nope", _ptrs(small_bufs), 200, _stream(), 1) == _lib.ERR_NOT_FOUND
     finally:
         L.pccl_hip_destroy(h)
+
+
+def test_recorded_launches_and_a_workspace_that_changes_hands():
+    """The entry point under graph capture, the case it exists for.  After one eager call the
+    operation's tables sit in the workspace and a call is kernel launches only: it is recorded into
+    a graph of the caller and every replay is compared with pccl_hip_execute_inplace, with eager
+    work and synchronisations between the replays.  Then another operation takes the workspace over.
+    A replay of the old graph now finds foreign tables behind its kernel arguments: it must execute
+    nothing (the buffers keep what they held), and the next synchronous call reports it.  After an
+    eager call of the first operation the same graph works again."""
+    L = _lib.lib()
+    world, n = 8, 1 << 16
+    h = ctypes.c_void_p()
+    _lib.check(L.pccl_hip_create(ctypes.byref(h), 0, world))
+    try:
+        _register(L, h, "a", graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2))
+        _register(L, h, "b", graph_jsons("rhd", "build_allreduce", world, 4096, "float32", "sm", 1))
+        src = [t.cuda() for t in seeded_inputs("randn", world, n, "bfloat16", seed=21)]
+        want = [t.clone() for t in src]
+        _lib.check(L.pccl_hip_execute_inplace(h, b"a", _ptrs(want), want[0].nbytes, _stream(), 1))
+        bufs = [t.clone() for t in src]
+        _lib.check(L.pccl_hip_execute_inplace_static(h, b"a", _ptrs(bufs), bufs[0].nbytes, _stream(), 1))
+        for r in range(world):
+            assert bits_equal(bufs[r], want[r]), mismatch_report(bufs[r], want[r])
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for b, t in zip(bufs, src):
+                    b.copy_(t)
+                _lib.check(L.pccl_hip_execute_inplace_static(h, b"a", _ptrs(bufs), bufs[0].nbytes, side.cuda_stream, 0))
+        torch.cuda.current_stream().wait_stream(side)
+        for rep in range(3):
+            print(f"replay {rep}", flush=True)
+            for b in bufs:
+                b.fill_(float(rep))                       # eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for r in range(world):
+                assert bits_equal(bufs[r], want[r]), f"replay {rep}, rank {r}"
+
+        print("another operation takes the workspace, then the old graph is replayed", flush=True)
+        other = [t.cuda() for t in seeded_inputs("randn", world, 4096, "float32", seed=22)]
+        _lib.check(L.pccl_hip_execute_inplace_static(h, b"b", _ptrs(other), other[0].nbytes, _stream(), 1))
+        graph.replay()                                    # copies the inputs in, then a launch that must do nothing
+        torch.cuda.synchronize()
+        for r in range(world):
+            assert bits_equal(bufs[r], src[r]), f"a stale replay touched rank {r}"
+        rc = L.pccl_hip_execute_inplace_static(h, b"b", _ptrs(other), other[0].nbytes, _stream(), 1)
+        assert rc == ERR_INVALID and b"replayed after the static workspace" in L.pccl_hip_last_error()
+
+        print("the first operation again, eagerly and from the graph", flush=True)
+        again = [t.clone() for t in src]
+        _lib.check(L.pccl_hip_execute_inplace_static(h, b"a", _ptrs(again), again[0].nbytes, _stream(), 1))
+        for r in range(world):
+            assert bits_equal(again[r], want[r])
+        graph.replay()
+        torch.cuda.synchronize()
+        for r in range(world):
+            assert bits_equal(bufs[r], want[r]), f"replay after the workspace came back, rank {r}"
+        _lib.check(L.pccl_hip_sync(h, b"a"))
+    finally:
+        _lib.check(L.pccl_hip_destroy(h))
