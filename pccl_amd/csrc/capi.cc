@@ -454,9 +454,7 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
 
     // column plans (in place, and direct = staging fused into the program)
     if (P.position_aligned) {
-        // slot runner: one vector per thread and R 16-byte slots per thread; keep a workgroup's
-        // slots within 32 KiB so that several workgroups share a CU
-        // Exception: a program that never reads a value back (every memory operand a first touch,
+        // The slot runner is the default.  Exception: a program that never reads a value back (every memory operand a first touch,
         // every live store final - the ring's chains) moves the same bytes under the register
         // runner, which needs no LDS; beyond 16 ranks the slots leave room for so few waves that it
         // wins (32-rank bf16 ring 0.99 -> 0.80 ms, 64-rank f32 ring 2.57 -> 1.62 ms; at 16 ranks

@@ -472,3 +472,24 @@ def test_damaged_documents_are_errors_not_crashes():
                 L.pccl_program_free(p)
             L.pccl_graph_free(g)
     assert failed > 50 and loaded > 10
+
+
+def test_bench_finds_the_committed_counter_figures():
+    """bench.py copies the counter-measured HBM bytes per launch of its kernel from the committed
+    rocprofv3 summary of the same workload and names that file (`roofline.traffic_source`): the files
+    it looks for exist, hold a positive byte count and sit beside a summary that names their kernel."""
+    import importlib.util
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_under_test", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    wanted = [("column_slot_kernel", "ring_allreduce_R8_bf16_512MiB"), ("level_kernel", "ring_allreduce_R8_bf16_512MiB"),
+              ("persistent_kernel", "ring_allreduce_R8_bf16_512MiB"), ("column_slot_kernel", "rhd_allreduce_R16_f32_64MiB"),
+              ("column_slot_kernel", "tree_allreduce_R32_int32_sum_96MiB"), ("column_slot_kernel", "tree_allreduce_R32_f32_max_96MiB")]
+    for kernel, stem in wanted:
+        nbytes, rel = bench.committed_traffic(kernel, stem)
+        assert rel == f"profiles/{kernel}_{stem}.traffic.json" and nbytes and nbytes > 0, (kernel, stem)
+        summary = os.path.join(root, "profiles", f"{kernel}_{stem}.md")
+        assert os.path.exists(summary) and kernel in open(summary).read()
+    assert bench.committed_traffic("column_slot_kernel", None) == (None, None)
+    assert bench.committed_traffic("column_slot_kernel", "no_such_workload") == (None, None)
