@@ -237,6 +237,9 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * slot_threads x slot_vecs vectors of every rank; 0 = from the rank count); "slot_lds_kib" = 0..160
  * (least LDS a workgroup of that runner asks for, which bounds the workgroups per CU; 0 = chosen);
  * "slot_direct" = "1" | "0" (first touches loaded straight into LDS, or through registers);
+ * "slot_store_waves" = "-1" | "0" | "1" (1: the final broadcast of a program goes through LDS and each
+ * wave stores whole tiles of some ranks; 0: every wave stores a slice of every rank; -1, the default:
+ * 1 for plans that write at least four times what they read, such as an allgather);
  * "level_graph" = "0" | "1" (the level runner launches level by level, or replays the launches of an
  * execution as one HIP graph captured per set of rank pointers);
  * "trace_ranges" = "0" | "1" (host-side roctx ranges around the stages of a call, under the names of

@@ -74,6 +74,7 @@ struct ColumnLaunch {
     int32_t slot_lds_bytes;   // slot runner: dynamic LDS of a workgroup (>= num_ranks x slot_vecs x slot_threads x 16)
     int32_t num_ranks;        // slot runner: LDS slots per thread
     int32_t slot_direct;      // slot runner: 1 = first touches are loaded straight into LDS
+    int32_t slot_store_waves; // slot runner: 1 = the broadcast tail goes through LDS and each wave stores whole tiles of some ranks
     int32_t xcd_run;          // run length of the tile-to-XCD mapping; filled in by the launcher
     int32_t seg_tiles;        // > 0: every segment has this many tiles (segment = tile / seg_tiles, fewer than 2^32 tiles); 0: search
 };

@@ -1009,6 +1009,28 @@ __device__ __forceinline__ void slot_tile(const ColumnLaunch& L, const DevColSeg
             }
         }
     }
+    if constexpr (!MASKED) {
+        if (L.slot_store_waves && seg.bcast_mask) {
+            // The broadcast tail with the stores dealt to the waves: every thread parks its results in
+            // its own rank-0 slots - slot (0, v) of thread t sits at index v T + t, so the parked
+            // values lie in the order of the tile - and after a barrier wave w stores the whole tile
+            // to the ranks of the mask that fall to it: 16 T V contiguous bytes of one rank from one
+            // wave, instead of 1 KiB of every rank.  (Measured no faster; kept as an option so that the
+            // comparison can be repeated.)
+#pragma unroll
+            for (int v = 0; v < V; ++v) slots[v * T + tid] = acc[v];
+            __syncthreads();
+            const int W = T >> 6, w = tid >> 6, lane = tid & 63;
+            int k = 0;
+            for (uint64_t m = seg.bcast_mask; m; m &= m - 1, ++k) {
+                if (k % W != w) continue;
+                char* const dst = ptrs.p[__builtin_ctzll(m)] + vfirst * 16;
+                for (int j = 0; j < T * V; j += 64) stv_nt(dst + (int64_t)(j + lane) * 16, slots[j + lane]);
+            }
+            __syncthreads();   // a workgroup that walks on to another tile fetches into these slots
+            return;
+        }
+    }
     // the broadcast tail, four rank pointers fetched per round so that their scalar loads overlap
     for (uint64_t m = seg.bcast_mask; m;) {
         char* dsts[4];

@@ -202,17 +202,22 @@ def test_slot_runner_workgroup_shapes(engine_factory, seed):
         for threads, vecs, kib in SLOT_SHAPES:
             if threads * vecs > 1024 or world * threads * vecs * 16 > 160 * 1024:
                 continue
-            print(f"seed {seed} {dtype} R={world}: threads={threads} vecs={vecs} lds_kib={kib}", flush=True)
             eng.set_option("slot_vecs", vecs); eng.set_option("slot_threads", threads); eng.set_option("slot_lds_kib", kib)
-            bufs = [t.cuda() for t in x]
-            eng.execute_inplace("rnd", bufs, sync=True)
-            for r in range(world):
-                assert bits_equal(bufs[r], want[r]), f"{threads}x{vecs}, rank {r}: {mismatch_report(bufs[r], want[r])}"
-            outs = eng.execute_operation("ring", [t.cuda() for t in rx])
-            for r in range(world):
-                assert bits_equal(outs[r], ring_want[r]), f"staged ring {threads}x{vecs}, rank {r}: {mismatch_report(outs[r], ring_want[r])}"
+            # store_waves: the broadcast tail through LDS, whole tiles of a rank stored by one wave;
+            # blocks: a grid smaller than the number of tiles, so that workgroups walk several tiles
+            for store_waves, blocks in ((0, 0), (1, 0), (1, 5)):
+                print(f"seed {seed} {dtype} R={world}: threads={threads} vecs={vecs} lds_kib={kib} store_waves={store_waves} blocks={blocks}", flush=True)
+                eng.set_option("slot_store_waves", store_waves); eng.set_option("num_blocks", blocks)
+                what = f"{threads}x{vecs} store_waves={store_waves} blocks={blocks}"
+                bufs = [t.cuda() for t in x]
+                eng.execute_inplace("rnd", bufs, sync=True)
+                for r in range(world):
+                    assert bits_equal(bufs[r], want[r]), f"{what}, rank {r}: {mismatch_report(bufs[r], want[r])}"
+                outs = eng.execute_operation("ring", [t.cuda() for t in rx])
+                for r in range(world):
+                    assert bits_equal(outs[r], ring_want[r]), f"staged ring {what}, rank {r}: {mismatch_report(outs[r], ring_want[r])}"
         with pytest.raises(PcclError, match="LDS"):
             eng.set_option("slot_threads", 1024); eng.set_option("slot_vecs", 4)
     finally:
-        for key, val in (("slot_vecs", 0), ("slot_threads", 0), ("slot_lds_kib", 0), ("mode", "auto")):
+        for key, val in (("slot_vecs", 0), ("slot_threads", 0), ("slot_lds_kib", 0), ("slot_store_waves", -1), ("num_blocks", 0), ("mode", "auto")):
             eng.set_option(key, val)
