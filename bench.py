@@ -22,6 +22,10 @@ collective).
              sustain to be as fast.  Not an HBM rate.
 * cpu_baseline   the CPU oracle (oracle/, OpenMP) executing the same graph on this box's host
              cores; a reported baseline, not the target
+* other_configs  (plain default run only, after the headline has been measured) configurations 3, 5
+             with both element types and the 512 MB pair of 4, each verified at full size and timed
+             the same way: ms per step, HBM bytes and rate, fraction of peak, and the per-rank
+             alg_bw / bus_bw of the reference's own bandwidth script
 
 Other configurations: c3 = recursive halving-doubling allreduce, 16 ranks, 64 MiB f32, 2 channels;
 c4 = ring reduce_scatter and allgather, 8 ranks, fp16, 4 KB to 512 MB per rank as staged calls;
@@ -313,6 +317,16 @@ def moved_bytes(info: dict, mode: str, staged: bool = False):
     return info["column_load_bytes"] + info["column_store_bytes"], "bytes the column plan loads and stores"
 
 
+def reference_bandwidths(collective: str, data_bytes: int, world: int, ms_per_call: float) -> dict:
+    """Per-rank bandwidths the reference's way (tests/bench_algo_comparison.py:141-156): alg_bw is the
+    rank's full tensor (the allreduce tensor, the reduce_scatter input, the allgather output) over the
+    time of one call, bus_bw scales it by 2 (N - 1) / N for an allreduce and (N - 1) / N otherwise."""
+    alg = data_bytes / (ms_per_call * 1e-3) / 1e9
+    factor = 2 * (world - 1) / world if collective == "allreduce" else (world - 1) / world
+    return {"alg_bw_GBps": round(alg, 1), "bus_bw_GBps": round(alg * factor, 1),
+            "bw_definition": "per virtual rank, reference tests/bench_algo_comparison.py:141-156"}
+
+
 def side_leg(eng, name, bufs, mode, reps, alg_bytes):
     import torch
     eng.set_option("mode", mode)
@@ -420,6 +434,7 @@ def run_inplace(args, wl: Workload, dev) -> int:
         del outs
         sb, _ = moved_bytes(info, args.mode, staged=True)
         staged = {"ms_per_call": round(staged_ms, 4), "hbm_GB/s": round(sb / (staged_ms * 1e-3) / 1e9, 1),
+                  **reference_bandwidths("allreduce", wl.n * 2, wl.world, staged_ms),
                   "note": "the reference's call shape (separate input and output tensors per rank, execute_operation_async); "
                           "in column mode the staging copies are fused into the program, so this is again one launch"}
 
@@ -464,14 +479,138 @@ def run_inplace(args, wl: Workload, dev) -> int:
         result["roofline"]["traffic_vs_counted"] = round(traffic / hbm_bytes, 4)
     if args.gpu_inputs:
         result["data"] = "synthetic (GPU generator: tuning run)"
+    del bufs, pristine
+    eng.close()
+    torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
-        del bufs, pristine
-        torch.cuda.empty_cache()
         np_dtype = "uint16" if wl.dtype in ("bf16", "f16") else "int32" if wl.dtype == "int32" else "float32"
         result["cpu_baseline"] = cpu_baseline(wl.jsons, wl.world, wl.n, np_dtype, wl.name + ": the same graphs", args.cpu_reps)
+    # the other configurations, after everything of the headline has been measured
+    full_default = (wl.key == "c2" and args.mode == "auto" and default_runner and not args.gpu_inputs
+                    and args.elems == 268_435_456 and args.channels == 4 and args.num_blocks < 0 and not args.rank_skew_bytes)
+    if args.other_configs == "on" or (args.other_configs == "auto" and full_default and not args.no_side_legs):
+        result["other_configs"] = other_configs(args, dev)
+        if not all(row["verified"] for row in result["other_configs"]):
+            print(json.dumps({"error": "verification of another configuration failed",
+                              "other_configs": result["other_configs"]}))
+            return 1
     print(json.dumps(result))
-    eng.close()
     return 0
+
+
+# ----------------------------------------------------------------------------------------- the other configurations, briefly
+
+def brief_inplace(args, wl: Workload, dev) -> dict:
+    """One of the other in-place configurations inside the default run: first execution verified at
+    full size as in its own run, then `steps` timed executions with HIP events."""
+    import torch
+    from pccl_amd.engine import Engine
+    eng = Engine(wl.world, 0)
+    try:
+        for r, text in enumerate(wl.jsons):
+            eng.register_operation_json("bench", text, r)
+        info = eng.op_info("bench")
+        pristine = wl.make_inputs()
+        bufs = [p.clone() for p in pristine]
+        eng.execute_inplace("bench", bufs)
+        torch.cuda.synchronize()
+        ok, verify = wl.check(pristine, bufs)
+        for b, p in zip(bufs, pristine):
+            b.copy_(p)
+        ms_per_step, kern_ms = timed_inplace(eng, "bench", bufs, args.steps, args.warmup)
+        avg_ms = sum(kern_ms) / len(kern_ms)
+        hbm_bytes, note = moved_bytes(info, "auto")
+        rate = hbm_bytes / (avg_ms * 1e-3) / 1e9
+        traffic, source = committed_traffic("column_slot_kernel", wl.traffic_stem)
+        out = {"workload": wl.name, "verified": bool(ok), "verify": verify, "ms_per_step": round(ms_per_step, 4),
+               "kernel_ms_avg": round(avg_ms, 4), "kernel_ms_min": round(min(kern_ms), 4),
+               "hbm_bytes_per_step": hbm_bytes, "algorithmic_bytes_per_step": info["algorithmic_bytes"],
+               "GB/s": round(rate, 1), "frac": round(rate / PEAK_GBPS, 4), "bytes_counted": note,
+               "traffic": traffic, "traffic_source": source}
+        out.update(reference_bandwidths("allreduce", wl.n * (2 if wl.dtype in ("bf16", "f16") else 4), wl.world, ms_per_step))
+        return out
+    finally:
+        eng.close()
+        torch.cuda.empty_cache()
+
+
+def brief_c4(args, dev, nbytes: int) -> list:
+    """The 512 MB end point of configuration 4 inside the default run: ring reduce_scatter and
+    allgather, 8 ranks, fp16, as staged calls on separate input and output tensors; the first call is
+    verified against the ring's reduction order evaluated with torch's fp16 adds."""
+    import torch
+    from pccl_amd.engine import Engine
+    world, n = 8, nbytes // 2
+    chunk = n // world
+    g = torch.Generator(device="cuda").manual_seed(0)
+    out = []
+    for method, in_elems, out_elems in (("build_reduce_scatter", n, chunk), ("build_allgather", chunk, n)):
+        eng = Engine(world, 0)
+        try:
+            for r, j in enumerate(graphs("ring", method, world, n, "float16", 1)):
+                eng.register_operation_json("bench", j, r)
+            info = eng.op_info("bench")
+            x = [(torch.randn(in_elems, generator=g, device="cuda") * 0.1).half() for _ in range(world)]
+            outs = [torch.empty(out_elems, dtype=torch.float16, device="cuda") for _ in range(world)]
+            call = eng.prepare("bench", x, outs)
+            call()
+            torch.cuda.synchronize()
+            ok = True
+            if method == "build_reduce_scatter":
+                for c in range(world):          # chunk c: x_(c+1), then + x_(c+2) ... + x_c, each sum rounded to fp16
+                    acc = x[(c + 1) % world][c * chunk:(c + 1) * chunk].clone()
+                    for k in range(2, world + 1):
+                        acc = acc + x[(c + k) % world][c * chunk:(c + 1) * chunk]
+                    ok = ok and torch.equal(acc.view(torch.int16), outs[c].view(torch.int16))
+            else:
+                whole = torch.cat(x)
+                ok = all(torch.equal(o.view(torch.int16), whole.view(torch.int16)) for o in outs)
+                del whole
+            for _ in range(args.warmup):
+                call()
+            torch.cuda.synchronize()
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+            t0 = time.perf_counter()
+            for a, b in ev:
+                a.record()
+                call()
+                b.record()
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+            ms = [a.elapsed_time(b) for a, b in ev]
+            avg = sum(ms) / len(ms)
+            hbm, note = moved_bytes(info, "auto", staged=True)
+            rate = hbm / (avg * 1e-3) / 1e9
+            kind = method[6:]
+            row = {"workload": f"ring_{kind}_R8_f16_{nbytes}B_per_rank_staged_call", "verified": bool(ok),
+                   "verify": {"matches_ring_order_f16" if kind == "reduce_scatter" else "every_output_is_the_concatenation": bool(ok)},
+                   "ms_per_step": round(wall_ms, 4), "kernel_ms_avg": round(avg, 4), "kernel_ms_min": round(min(ms), 4),
+                   "hbm_bytes_per_step": hbm, "algorithmic_bytes_per_step": info["algorithmic_bytes"],
+                   "GB/s": round(rate, 1), "frac": round(rate / PEAK_GBPS, 4), "bytes_counted": note,
+                   "traffic": None, "traffic_source": None}
+            row.update(reference_bandwidths(kind, nbytes, world, wall_ms))
+            out.append(row)
+        finally:
+            eng.close()
+            del x, outs
+            torch.cuda.empty_cache()
+    return out
+
+
+def other_configs(args, dev) -> list:
+    """Configurations 3, 5 (both element types) and the 512 MB pair of 4, each verified and timed like
+    its own `--config` run, for the default run's JSON line."""
+    rows = []
+    saved = args.c5_dtype
+    try:
+        rows.append(brief_inplace(args, workload_c3(args, dev), dev))
+        for dt in ("int32", "float32"):
+            args.c5_dtype = dt
+            rows.append(brief_inplace(args, workload_c5(args, dev), dev))
+        rows.extend(brief_c4(args, dev, 512 << 20))
+    finally:
+        args.c5_dtype = saved
+    return rows
 
 
 # ----------------------------------------------------------------------------------------- c4: message-size sweep
@@ -537,6 +676,7 @@ def run_c4(args, dev) -> int:
                                "channels": 1, "data_ops": info["num_data_ops"], "algorithmic_bytes_per_step": info["algorithmic_bytes"],
                                "hbm_bytes_per_step": hbm, "mode": args.mode, "in_place": False},
                     "latency_us_median": round(ms[len(ms) // 2] * 1e3, 2), "latency_us_min": round(ms[0] * 1e3, 2),
+                    **reference_bandwidths(method[6:], nbytes, world, wall_ms),
                     "algorithmic_equiv_GBps": round(info["algorithmic_bytes"] / (wall_ms * 1e-3) / 1e9, 1),
                     "roofline": {"bound": "hbm", "achieved": round(hbm / (avg * 1e-3) / 1e9, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                                  "frac": round(hbm / (avg * 1e-3) / 1e9 / PEAK_GBPS, 4), "traffic": None, "traffic_source": None,
@@ -570,6 +710,9 @@ def main() -> int:
     ap.add_argument("--no-side-legs", action="store_true", help="skip the op-by-op and single-launch legs of an auto-mode run")
     ap.add_argument("--gpu-inputs", action="store_true",
                     help="c2: draw the inputs with the GPU generator (tuning runs only; not the prescribed inputs)")
+    ap.add_argument("--other-configs", default="auto", choices=["auto", "on", "off"],
+                    help="append configurations 3, 5 and the 512 MB pair of 4 (verified, timed) to the JSON line as "
+                         "'other_configs': auto = only in the plain default run")
     ap.add_argument("--cpu-reps", type=int, default=20)
     ap.add_argument("--calibrate-copy-bytes", type=int, default=0,
                     help="also launch the library's plain copy kernel on this many bytes (3 times): a "

@@ -227,7 +227,9 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * "timing" = "0" | "1" (record HIP events around the program); "vecs_per_thread" = 1 | 2 | 4;
  * "step_tile_bytes" (work item of the level and persistent runners: 0 = chosen from the program's
  * size, 4 to 32 KiB, else a multiple of 4096); "wait_timeout_ms" (how long a persistent launch waits
- * for a predecessor);
+ * for a predecessor); "test_host_epoch_limit" / "test_graph_epoch_limit" (for tests: the launch number
+ * at which the persistent runner's flags are cleared and its numbering restarts, on the host and for
+ * launches recorded into a graph; by default about 2^30 launches apart);
  * "fuse_staging" = "1" | "0" (allreduce-type calls in column mode read the input tensors and write
  * the output tensors directly instead of staging through the engine's rank buffers);
  * "lds_slots" = "1" | "0" (column runner keeps values it re-reads in per-thread LDS slots, so each
@@ -281,10 +283,15 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
  * `stream`), which it refuses to do on a capturing stream (execute once outside the capture first).
  * Calls that overlap in time on one GPU - two streams, two threads - race on the workspace.
  * A recorded launch stays valid while the workspace holds its operation's tables.  Replayed after
- * another operation has taken the workspace over it executes nothing (the kernel compares a tag in
- * its arguments with the one in the workspace before it reads any table) and the next synchronous
- * call or pccl_hip_sync on that GPU's workspace returns PCCL_ERR_INVALID saying so; execute the
- * operation once more through this entry point and the recorded launch works again. */
+ * another operation has taken the workspace over it executes nothing and leaves its rank buffers
+ * exactly as they were (the kernel compares a tag in its arguments with the one in the workspace
+ * before it reads any table).  The library notices at the next look at the workspace (a synchronous
+ * call of this entry point, or pccl_hip_sync): it logs a warning that names the operation, and the
+ * next pccl_hip_sync of THAT operation returns PCCL_ERR_INVALID saying so.  The call that happens to
+ * notice is not failed for it: a call of this entry point that returns 0 has executed and updated its
+ * buffers, one that returns PCCL_ERR_HIP for an expired wait has updated them partially, and every
+ * other error is returned before anything is enqueued.  Execute the operation once more through this
+ * entry point and its recorded launch works again. */
 int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
                                     void* stream, int sync);
 /* Engine::syncOp / Engine::resetSignals (reference csrc/engine_c.cc:562-593). */

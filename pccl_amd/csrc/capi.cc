@@ -343,6 +343,7 @@ struct OpEntry {
     bool timed = false;
     bool ran_persistent = false;          // a persistent launch has not been checked for stalls yet
     bool ran_static = false;              // the same for a launch in the static workspace
+    bool stale_replay = false;            // a recorded launch of this operation was replayed on foreign tables; its next sync says so
     uint64_t generation = 0;              // which host link these tables come from (never reused in the process)
     int epoch = 0;                        // persistent runner: launches so far
     std::vector<int> level_item_begin;    // work-list index where each dependency level starts (+ end)
@@ -376,6 +377,34 @@ struct OpEntry {
 enum class Mode { Auto, Column, Stepwise, Persistent };
 constexpr size_t kMaxSlotLdsBytes = 160 * 1024;   // LDS of one gfx950 CU
 
+// Shape of a slot-runner workgroup for R ranks under the given option values (0 = automatic):
+// threads x vectors per thread (a tile is that many 16-byte vectors of every rank) and the LDS its
+// slots need.  The one place that decides it: linking uses it, and set_option checks a new value
+// against it, so that a combination the LDS cannot hold is refused where it is asked for.
+// Measured on MI355X, same box and call: 8 ranks x 512 MiB bf16 ring 256 x 1 (five per CU) 1.43 ms,
+// 256 x 2 (two per CU, 8 KiB of every rank per tile) 1.39; 32-rank tree 64 x 1 1.19 ms, 128 x 1
+// 1.12; 16 ranks the same from 128 to 512 threads.  One workgroup per CU with larger tiles loses:
+// the program's arithmetic is then not overlapped with anything.
+struct SlotShape { int threads, vecs; size_t need; };
+SlotShape slot_shape(int R, int slot_threads, int slot_vecs, bool slot_direct) {
+    SlotShape sh;
+    sh.threads = R <= 16 ? 256 : R <= 32 ? 128 : 64;
+    sh.vecs = R > 4 && R <= 8 ? 2 : 1;
+    if (slot_threads > 0) { sh.threads = slot_threads; if (slot_vecs == 0) sh.vecs = 1; }
+    if (slot_vecs > 0) sh.vecs = slot_vecs;
+    if (!slot_direct) sh.vecs = 1;   // fetching through registers: one vector per thread
+    sh.need = (size_t)R * sh.vecs * sh.threads * 16;
+    return sh;
+}
+// Empty if the shape can be launched, else why not.
+std::string slot_shape_error(int R, const SlotShape& sh) {
+    if (sh.threads * sh.vecs > 1024) return "slot runner: slot_threads x slot_vecs may not exceed 1024 (" + std::to_string(sh.threads) + " x " + std::to_string(sh.vecs) + ")";
+    if (sh.need > kMaxSlotLdsBytes)
+        return "slot runner: " + std::to_string(R) + " ranks x " + std::to_string(sh.vecs) + " vectors x " + std::to_string(sh.threads) +
+               " threads x 16 bytes exceed the " + std::to_string(kMaxSlotLdsBytes >> 10) + " KiB of LDS a workgroup may use";
+    return "";
+}
+
 }  // namespace
 
 struct pccl_hip_ctx {
@@ -404,6 +433,8 @@ struct pccl_hip_ctx {
     int64_t step_tile_bytes = 0;   // work item of the level and persistent runners; 0 = automatic, 32 KiB for large programs (persistent, headline graph: 3.91 ms at 8 KiB, 3.16 at 16, 3.10 at 32, 3.35 at 64; sizes that do not divide the ops are slower)
     bool fuse_staging = true;             // run staged calls on the caller's tensors when possible
     int wait_timeout_ms = 2000;           // a persistent launch gives up on a dependency after this long
+    int32_t host_epoch_limit = kHostEpochLimit;   // persistent runner: launch number at which the host clears the flags and restarts
+    int32_t graph_epoch_limit = kGraphEpochLimit; // the same for the device-side counter of recorded launches
     hipStream_t last_stream = nullptr;
 };
 
@@ -466,27 +497,13 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
             if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || (in.store & STORE_KIND) == 1) reads_back = true;
         e.slot_threads = 0; e.slot_vecs = 1; e.slot_lds_bytes = 0;
         if (ctx->lds_slots && (ctx->slot_threads > 0 || reads_back || ctx->R <= 16)) {
-            // Shape of a workgroup: threads x vectors per thread (a tile is that many 16-byte vectors of
-            // every rank), chosen so that the slots of a workgroup are 64 KiB at most and at least two
-            // workgroups share a CU - one computes while the other waits for memory.  Measured on
-            // MI355X, same box and call: 8 ranks x 512 MiB bf16 ring 256 x 1 (five per CU) 1.43 ms,
-            // 256 x 2 (two per CU, 8 KiB of every rank per tile) 1.39; 32-rank tree 64 x 1 1.19 ms,
-            // 128 x 1 1.12; 16 ranks the same from 128 to 512 threads.  One workgroup per CU with
-            // larger tiles, which a bare kernel of this traffic shape likes best (1.31 ms for the
-            // ring), loses here: the program's arithmetic is then not overlapped with anything.
             const int R = ctx->R;
-            int threads = R <= 16 ? 256 : R <= 32 ? 128 : 64;
-            int vecs = R > 4 && R <= 8 ? 2 : 1;
-            int lds_kib = 0;
-            if (ctx->slot_threads > 0) { threads = ctx->slot_threads; if (ctx->slot_vecs == 0) vecs = 1; if (ctx->slot_lds_kib == 0) lds_kib = 0; }
-            if (ctx->slot_vecs > 0) vecs = ctx->slot_vecs;
-            if (ctx->slot_lds_kib > 0) lds_kib = ctx->slot_lds_kib;
-            if (!ctx->slot_direct) vecs = 1;
-            if (threads * vecs > 1024) throw Error{PCCL_ERR_INVALID, "slot runner: slot_threads x slot_vecs may not exceed 1024"};
-            const size_t need = (size_t)R * vecs * threads * 16;
-            if (need > kMaxSlotLdsBytes)
-                throw Error{PCCL_ERR_INVALID, "slot runner: " + std::to_string(R) + " ranks x " + std::to_string(vecs) + " vectors x " + std::to_string(threads) +
-                                                  " threads x 16 bytes exceed the " + std::to_string(kMaxSlotLdsBytes >> 10) + " KiB of LDS a workgroup may use"};
+            const SlotShape sh = slot_shape(R, ctx->slot_threads, ctx->slot_vecs, ctx->slot_direct);
+            const std::string why = slot_shape_error(R, sh);
+            if (!why.empty()) throw Error{PCCL_ERR_INVALID, why};
+            const int threads = sh.threads, vecs = sh.vecs;
+            const size_t need = sh.need;
+            const int lds_kib = ctx->slot_lds_kib;
             e.slot_threads = threads; e.slot_vecs = vecs;
             e.slot_lds_bytes = (int)std::min<size_t>(std::max<size_t>(need, (size_t)lds_kib << 10), kMaxSlotLdsBytes);
         }
@@ -719,7 +736,18 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
             // The launch number is a kernel argument, which every replay of a recorded launch would
             // repeat (finding all flags of the previous replay set): on a capturing stream the
             // number comes from a device-side counter that a one-thread kernel advances first.
-            L.epoch = is_capturing(stream) ? 0 : ++e.epoch;
+            if (is_capturing(stream)) L.epoch = 0;
+            else {
+                if (e.epoch >= ctx->host_epoch_limit) {
+                    // the launch numbers have run out: clear the flags and ready words (a fill kernel on the
+                    // stream, behind every earlier launch) and count from 1 again
+                    const int frc = launch_fill_zero((char*)e.state.p + sizeof(StepState), sizeof(int32_t) * ((size_t)P.num_items + P.ops.size() + 1), stream);
+                    if (frc != 0) throw Error{PCCL_ERR_HIP, std::string("clearing the progress flags: ") + hipGetErrorString((hipError_t)frc)};
+                    e.epoch = 0;
+                }
+                L.epoch = ++e.epoch;
+            }
+            L.graph_epoch_limit = ctx->graph_epoch_limit;
             L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
             rc = launch_persistent(L, ptrs, stream);   // sizes the grid to what is resident at once
             e.ran_persistent = true;
@@ -923,28 +951,53 @@ StaticLayout static_layout(const Program& P) {
 }
 
 // A recorded launch that was replayed after the workspace had gone to another operation has left
-// its tag behind (it executed nothing).  Say so once, at the next look at the block.
-void report_stale_launch(StaticWorkspace& ws, const StepState& st) {
+// its tag behind (it executed nothing and touched no buffer).  Whoever looks at the block next
+// notes it: a WARN line that names the operation, the word is cleared, and the operation whose
+// launch it was - if it belongs to this context - hears of it as an error at its own next
+// pccl_hip_sync.  The call that happens to find the word is not failed: it executed normally.
+void note_stale_launch(pccl_hip_ctx* ctx, StaticWorkspace& ws, const StepState& st) {
     if (st.stale_owner == 0) return;
-    ws.owner = 0;                                      // the next call clears the block, this word included
-    throw Error{PCCL_ERR_INVALID, "a recorded launch of pccl_hip_execute_inplace_static was replayed after the static workspace had been taken over "
-                                  "by another operation; it executed nothing.  Execute the operation once through this entry point and record it again"};
+    std::string who = "an operation of another context";
+    for (auto& kv : ctx->ops)
+        if (kv.second.generation != 0 && static_tag(kv.second) == st.stale_owner) {
+            who = "operation '" + kv.first + "'";
+            kv.second.stale_replay = true;
+        }
+    log_line(LOG_WARN, "a recorded launch of pccl_hip_execute_inplace_static (" + who + ") was replayed after the static workspace had been "
+                       "taken over by another operation; that replay executed nothing and left its rank buffers as they were");
+    const uint32_t zero = 0;
+    HIP_TRY(hipMemcpy(ws.ptr + offsetof(StepState, stale_owner), &zero, sizeof(zero), hipMemcpyHostToDevice));
+}
+
+// The progress block of the static workspace after the stream has drained: a stall of THIS launch is
+// an error (checked first, so that a stale replay seen in the same look never hides it); a stale
+// replay is noted as above.
+void read_static_block(pccl_hip_ctx* ctx, StaticWorkspace& ws, const std::string& name) {
+    StepState st;
+    HIP_TRY(hipMemcpy(&st, ws.ptr, sizeof(st), hipMemcpyDeviceToHost));
+    const bool stalled = st.error_op != 0;
+    if (stalled) ws.owner = 0;                         // the next call clears and rewrites everything
+    note_stale_launch(ctx, ws, st);
+    if (stalled)
+        throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting in the static workspace (data op " +
+                                      std::to_string(st.error_op - 1) + " never saw its predecessor " + std::to_string(st.error_dep - 1) +
+                                      " complete); rank buffers are partially updated"};
 }
 
 void check_stall_static(pccl_hip_ctx* ctx, OpEntry& e, const std::string& name) {
-    if (!e.ran_static) return;
-    e.ran_static = false;
-    StaticWorkspace& ws = static_ws(ctx->device);
-    std::lock_guard<std::mutex> lock(ws.mu);
-    if (!ws.ptr || ws.owner != e.generation) return;   // another operation has taken the workspace over since
-    StepState st;
-    HIP_TRY(hipMemcpy(&st, ws.ptr, sizeof(st), hipMemcpyDeviceToHost));
-    report_stale_launch(ws, st);
-    if (st.error_op == 0) return;
-    ws.owner = 0;                                      // the next call clears and rewrites everything
-    throw Error{PCCL_ERR_HIP, "operation '" + name + "': the persistent runner gave up waiting in the static workspace (data op " +
-                                  std::to_string(st.error_op - 1) + " never saw its predecessor " + std::to_string(st.error_dep - 1) +
-                                  " complete); rank buffers are partially updated"};
+    if (e.ran_static) {
+        e.ran_static = false;
+        StaticWorkspace& ws = static_ws(ctx->device);
+        std::lock_guard<std::mutex> lock(ws.mu);
+        // (when another operation has taken the workspace over since, its own look covers the block)
+        if (ws.ptr && ws.owner == e.generation) read_static_block(ctx, ws, name);
+    }
+    if (e.stale_replay) {
+        e.stale_replay = false;
+        throw Error{PCCL_ERR_INVALID, "a recorded launch of operation '" + name + "' (pccl_hip_execute_inplace_static) was replayed after the static "
+                                      "workspace had been taken over by another operation: that replay executed nothing and left its rank buffers "
+                                      "unchanged.  Execute the operation once through that entry point and the recorded launch works again"};
+    }
 }
 
 int register_graph(pccl_hip_ctx* ctx, const char* name, int vrank, RankGraph&& g) {
@@ -1052,12 +1105,23 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
         }
         else if (k == "fuse_staging") ctx->fuse_staging = std::atoi(value) != 0;
         else if (k == "wait_timeout_ms") { ctx->wait_timeout_ms = std::atoi(value); if (ctx->wait_timeout_ms < 0) ctx->wait_timeout_ms = 0; }   // 0: give up on the first predecessor that is not ready
+        else if (k == "test_host_epoch_limit" || k == "test_graph_epoch_limit") {
+            // for tests: bring the point where the persistent runner's launch numbers wrap within reach
+            const long long x = std::atoll(value);
+            if (k == "test_host_epoch_limit") {
+                if (x < 2 || x > kHostEpochLimit) return fail(PCCL_ERR_INVALID, "test_host_epoch_limit must be 2 .. " + std::to_string(kHostEpochLimit));
+                ctx->host_epoch_limit = (int32_t)x;
+            } else {
+                if (x < kGraphEpochBase + 2 || x > kGraphEpochLimit) return fail(PCCL_ERR_INVALID, "test_graph_epoch_limit must be " + std::to_string(kGraphEpochBase + 2) + " .. " + std::to_string(kGraphEpochLimit));
+                ctx->graph_epoch_limit = (int32_t)x;
+            }
+        }
         else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
         else if (k == "vecs_per_thread") {
             int u = std::atoi(value);
             if (u != 1 && u != 2 && u != 4) return fail(PCCL_ERR_INVALID, "vecs_per_thread must be 1, 2 or 4");
             ctx->vecs_per_thread = u; relink = true;
-        } else if (k == "slot_direct") { ctx->slot_direct = std::atoi(value) != 0; relink = true; }
+        }
         else if (k == "slot_store_waves") {
             const int v = std::atoi(value);
             if (v < -1 || v > 1) return fail(PCCL_ERR_INVALID, "slot_store_waves must be -1 (automatic), 0 or 1");
@@ -1065,17 +1129,22 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
         }
         else if (k == "level_graph") ctx->level_graph = std::atoi(value) != 0;
         else if (k == "lds_slots") { ctx->lds_slots = std::atoi(value) != 0; relink = true; }
-        else if (k == "slot_threads") {
-            int t = std::atoi(value);
-            if (t != 0 && t != 64 && t != 128 && t != 256 && t != 512 && t != 1024) return fail(PCCL_ERR_INVALID, "slot_threads must be 0 (automatic), 64, 128, 256, 512 or 1024");
-            if ((size_t)t * ctx->R * 16 * std::max(1, ctx->slot_vecs) > kMaxSlotLdsBytes) return fail(PCCL_ERR_INVALID, "slot_threads x slot_vecs x ranks x 16 bytes exceeds the 160 KiB of LDS a workgroup may use");
-            ctx->slot_threads = t; relink = true;
-        }
-        else if (k == "slot_vecs") {
-            int v = std::atoi(value);
-            if (v != 0 && v != 1 && v != 2 && v != 4) return fail(PCCL_ERR_INVALID, "slot_vecs must be 0 (automatic), 1, 2 or 4");
-            if ((size_t)v * ctx->R * 16 * std::max(64, ctx->slot_threads) > kMaxSlotLdsBytes) return fail(PCCL_ERR_INVALID, "slot_threads x slot_vecs x ranks x 16 bytes exceeds the 160 KiB of LDS a workgroup may use");
-            ctx->slot_vecs = v; relink = true;
+        else if (k == "slot_direct" || k == "slot_threads" || k == "slot_vecs") {
+            // checked against the shape linking would choose with the new value in place
+            int threads = ctx->slot_threads, vecs = ctx->slot_vecs;
+            bool direct = ctx->slot_direct;
+            const int x = std::atoi(value);
+            if (k == "slot_threads") {
+                if (x != 0 && x != 64 && x != 128 && x != 256 && x != 512 && x != 1024) return fail(PCCL_ERR_INVALID, "slot_threads must be 0 (automatic), 64, 128, 256, 512 or 1024");
+                threads = x;
+            } else if (k == "slot_vecs") {
+                if (x != 0 && x != 1 && x != 2 && x != 4) return fail(PCCL_ERR_INVALID, "slot_vecs must be 0 (automatic), 1, 2 or 4");
+                vecs = x;
+            } else direct = x != 0;
+            if (!direct && vecs > 1) return fail(PCCL_ERR_INVALID, "slot_vecs above 1 needs slot_direct=1 (first touches fetched through registers take one vector per thread)");
+            const std::string why = slot_shape_error(ctx->R, slot_shape(ctx->R, threads, vecs, direct));
+            if (!why.empty()) return fail(PCCL_ERR_INVALID, why);
+            ctx->slot_threads = threads; ctx->slot_vecs = vecs; ctx->slot_direct = direct; relink = true;
         }
         else if (k == "slot_lds_kib") {
             int b = std::atoi(value);
@@ -1109,6 +1178,8 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
         else if (k == "fuse_staging") v = std::to_string((int)ctx->fuse_staging);
         else if (k == "wait_timeout_ms") v = std::to_string(ctx->wait_timeout_ms);
         else if (k == "check_races") v = std::to_string((int)ctx->check_races);
+        else if (k == "test_host_epoch_limit") v = std::to_string(ctx->host_epoch_limit);
+        else if (k == "test_graph_epoch_limit") v = std::to_string(ctx->graph_epoch_limit);
         else if (k == "vecs_per_thread") v = std::to_string(ctx->vecs_per_thread);
         else if (k == "slot_direct") v = std::to_string((int)ctx->slot_direct);
         else if (k == "slot_store_waves") v = std::to_string(ctx->slot_store_waves);
@@ -1198,7 +1269,7 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
         if (P.ops.empty()) return 0;
         const bool capturing = is_capturing(s);
         int rc = 0;
-        if (ws.owner != e.generation || ws.epoch >= 0x3FFFFFF0) {
+        if (ws.owner != e.generation || ws.epoch >= ctx->host_epoch_limit) {
             // the workspace holds another operation's tables (or nothing, or the launch numbers have run
             // out): clear the progress block and write this operation's tables, all by kernels on `s`
             if (capturing)
@@ -1222,6 +1293,7 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
         L.dtype = P.dtype; L.num_blocks = ctx->num_blocks;
         L.epoch = capturing ? 0 : ++ws.epoch;            // recorded launches take their number from the device-side counter
         L.owner_tag = static_tag(e);                     // a replay that finds another operation's tables does nothing
+        L.graph_epoch_limit = ctx->graph_epoch_limit;
         L.timeout_ticks = (uint64_t)ctx->wait_timeout_ms * 100000ull;
         {
             TraceRange exe(ctx->trace_ranges, "execute"), range(ctx->trace_ranges, "executor_kernel");
@@ -1232,15 +1304,8 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
         ctx->last_stream = s;
         if (sync) {
             HIP_TRY(hipStreamSynchronize(s));
-            StepState st;
-            HIP_TRY(hipMemcpy(&st, ws.ptr, sizeof(st), hipMemcpyDeviceToHost));
             e.ran_static = false;
-            report_stale_launch(ws, st);
-            if (st.error_op != 0) {
-                ws.owner = 0;
-                return fail(PCCL_ERR_HIP, "operation '" + std::string(name) + "': the persistent runner gave up waiting in the static workspace (data op " +
-                                              std::to_string(st.error_op - 1) + " never saw its predecessor " + std::to_string(st.error_dep - 1) + " complete)");
-            }
+            read_static_block(ctx, ws, name);
         }
         return 0;
     });

@@ -93,7 +93,14 @@ struct StepwiseLaunch {
                               // 0: take it from StepState::graph_epoch, which the launcher advances first
     uint32_t owner_tag;       // persistent runner in a shared block: run only if StepState::owner equals this (0: no check)
     uint64_t timeout_ticks;   // persistent runner: 100 MHz ticks a workgroup may run before a wait gives up
+    int32_t graph_epoch_limit;// recorded launches: where the device-side launch counter wraps (0: kGraphEpochLimit)
 };
+
+// Launch numbers of the persistent runner: the host counts 1 .. kHostEpochLimit and then clears the
+// flags and starts again; recorded launches count kGraphEpochBase + 1 .. kGraphEpochLimit on the device.
+constexpr int32_t kGraphEpochBase = 0x40000000;
+constexpr int32_t kHostEpochLimit = kGraphEpochBase - 16;
+constexpr int32_t kGraphEpochLimit = 0x7FFFFFF0;
 
 // All return a hipError_t value as int (0 = success).
 int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream);

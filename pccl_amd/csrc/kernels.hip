@@ -494,11 +494,25 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(const DevGatherCopy* c
     }
 }
 
-// Launch numbers of recorded launches start here, far from the host's own count (1, 2, ...).
-constexpr int32_t kGraphEpochBase = 0x40000000;
-__global__ void advance_graph_epoch_kernel(StepState* state) {
-    const int32_t e = state->graph_epoch;
-    __hip_atomic_store(&state->graph_epoch, (e < kGraphEpochBase ? kGraphEpochBase : e) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Launch numbers.  Flags and ready words hold the number of the launch that last set them and are
+// never cleared between launches, so every launch needs a number no earlier launch has left in them.
+// The host counts 1, 2, ... up to kHostEpochLimit; launches recorded into a graph (whose arguments
+// every replay repeats) take theirs from a device-side counter that starts at kGraphEpochBase, far
+// from the host's range, and that this kernel advances in front of each of them.  Neither range
+// runs out: the host clears the words and starts again from 1 when it reaches its limit, and this
+// kernel does the same for its counter - all its threads clear the `nwords` flag and ready words
+// behind the block, then the counter restarts at the base (`limit` is a parameter so that a test
+// can bring the wrap within reach).
+__global__ __launch_bounds__(kThreads) void advance_graph_epoch_kernel(StepState* state, int nwords, int32_t limit) {
+    const int32_t e = state->graph_epoch;                 // every thread reads the same word
+    int32_t next = (e < kGraphEpochBase ? kGraphEpochBase : e) + 1;
+    if (next >= limit) {
+        uint32_t* words = reinterpret_cast<uint32_t*>(state + 1);
+        for (int i = threadIdx.x; i < nwords; i += kThreads) words[i] = 0;
+        next = kGraphEpochBase + 1;
+    }
+    __syncthreads();                                      // all reads of the old value and all clears are done
+    if (threadIdx.x == 0) __hip_atomic_store(&state->graph_epoch, next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* dst, int64_t nwords) {
@@ -1015,8 +1029,10 @@ __device__ __forceinline__ void slot_tile(const ColumnLaunch& L, const DevColSeg
             // its own rank-0 slots - slot (0, v) of thread t sits at index v T + t, so the parked
             // values lie in the order of the tile - and after a barrier wave w stores the whole tile
             // to the ranks of the mask that fall to it: 16 T V contiguous bytes of one rank from one
-            // wave, instead of 1 KiB of every rank.  (Measured no faster; kept as an option so that the
-            // comparison can be repeated.)
+            // wave, instead of 1 KiB of every rank.  The host switches this on for plans that write at
+            // least four times what they read in workgroups of four waves or more (an 8-rank 512 MB fp16
+            // allgather 0.82 -> 0.79 ms); plans that read as much as they write are the same either
+            // way, and two-wave workgroups get slower (32-rank tree 1.12 -> 1.28 ms).
 #pragma unroll
             for (int v = 0; v < V; ++v) slots[v * T + tid] = acc[v];
             __syncthreads();
@@ -1217,7 +1233,8 @@ static int launch_persistent_dt(const StepwiseLaunch& L, const RankPtrs& ptrs, h
 int launch_persistent(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream) {
     hipStream_t s = (hipStream_t)stream;
     if (L.epoch == 0) {   // the launch number comes from the device-side counter: advance it first
-        hipLaunchKernelGGL(advance_graph_epoch_kernel, dim3(1), dim3(1), 0, s, L.state);
+        hipLaunchKernelGGL(advance_graph_epoch_kernel, dim3(1), dim3(kThreads), 0, s, L.state, L.num_items + L.num_ops + 1,
+                           L.graph_epoch_limit > 0 ? L.graph_epoch_limit : kGraphEpochLimit);
         hipError_t rc = hipGetLastError();
         if (rc != hipSuccess) return (int)rc;
     }

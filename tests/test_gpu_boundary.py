@@ -216,8 +216,111 @@ def test_slot_runner_workgroup_shapes(engine_factory, seed):
                 outs = eng.execute_operation("ring", [t.cuda() for t in rx])
                 for r in range(world):
                     assert bits_equal(outs[r], ring_want[r]), f"staged ring {what}, rank {r}: {mismatch_report(outs[r], ring_want[r])}"
-        with pytest.raises(PcclError, match="LDS"):
+        with pytest.raises(PcclError, match="may not exceed 1024"):
             eng.set_option("slot_threads", 1024); eng.set_option("slot_vecs", 4)
     finally:
         for key, val in (("slot_vecs", 0), ("slot_threads", 0), ("slot_lds_kib", 0), ("slot_store_waves", -1), ("num_blocks", 0), ("mode", "auto")):
             eng.set_option(key, val)
+
+
+def test_slot_shape_options_are_checked_where_they_are_set(engine_factory):
+    """A workgroup shape that the LDS cannot hold is refused by set_option itself, against the shape
+    linking would choose with the other option left automatic, and the refused value is not kept:
+    the next execution runs with the previous shape."""
+    world, n = 16, 1 << 14
+    jsons = graph_jsons("rhd", "build_allreduce", world, n, "float32", "sm", 1)
+    x = seeded_inputs("randn", world, n, "float32", seed=4)
+    want = oracle_buffers(jsons, x, "float32")
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("rhd", j, r)
+    try:
+        # 16 ranks: the automatic workgroup has 256 threads; 4 vectors per thread would need 256 KiB
+        with pytest.raises(PcclError, match="KiB of LDS"):
+            eng.set_option("slot_vecs", 4)
+        assert eng.get_option("slot_vecs") == "0"
+        eng.set_option("slot_threads", 64)
+        eng.set_option("slot_vecs", 4)                      # 64 x 4 x 16 ranks x 16 B = 64 KiB: fine
+        with pytest.raises(PcclError, match="KiB of LDS"):
+            eng.set_option("slot_threads", 256)             # with the 4 vectors just set
+        assert eng.get_option("slot_threads") == "64"
+        with pytest.raises(PcclError, match="slot_direct=1"):
+            eng.set_option("slot_direct", 0)                # fetching through registers takes one vector per thread
+        assert eng.get_option("slot_direct") == "1"
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("rhd", bufs, sync=True)
+        for r in range(world):
+            assert bits_equal(bufs[r], want[r]), mismatch_report(bufs[r], want[r])
+        eng.set_option("slot_vecs", 1)
+        eng.set_option("slot_direct", 0)
+        with pytest.raises(PcclError, match="slot_direct=1"):
+            eng.set_option("slot_vecs", 2)
+    finally:
+        for key, val in (("slot_direct", 1), ("slot_vecs", 0), ("slot_threads", 0)):
+            eng.set_option(key, val)
+
+
+@pytest.mark.parametrize("entry", ["inplace", "static"])
+def test_launch_numbers_of_the_persistent_runner_wrap(engine_factory, entry):
+    """Flags of the persistent runner hold the number of the launch that set them and are never
+    cleared between launches; when the numbers run out the flags are cleared and the count restarts,
+    on the host (eager launches) and on the device (launches recorded into a graph).  With both
+    limits brought within reach, executions before, at and after each wrap give the oracle's bits."""
+    import ctypes
+    from pccl_amd import _lib
+    world, n = 8, 1 << 15
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2)
+    x = seeded_inputs("randn", world, n, "bfloat16", seed=31)
+    want = oracle_buffers(jsons, x, "bfloat16")
+    eng = engine_factory(world)
+    name = f"wrap_{entry}"
+    for r, j in enumerate(jsons):
+        eng.register_operation_json(name, j, r)
+    src = [t.cuda() for t in x]
+    bufs = [t.clone() for t in src]
+    L = _lib.lib()
+
+    def execute(stream=None, sync=True):
+        ptrs = (ctypes.c_void_p * world)(*[b.data_ptr() for b in bufs])
+        s = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+        f = L.pccl_hip_execute_inplace if entry == "inplace" else L.pccl_hip_execute_inplace_static
+        _lib.check(f(eng._h, name.encode(), ptrs, bufs[0].nbytes, s, 1 if sync else 0))
+
+    eng.set_option("mode", "persistent")
+    eng.set_option("test_host_epoch_limit", 5)
+    eng.set_option("test_graph_epoch_limit", 0x40000000 + 4)
+    try:
+        for i in range(13):                                   # the host's numbers wrap at launches 6 and 11
+            for b, t in zip(bufs, src):
+                b.copy_(t)
+            execute()
+            for r in range(world):
+                assert bits_equal(bufs[r], want[r]), f"eager launch {i}, rank {r}: {mismatch_report(bufs[r], want[r])}"
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for b, t in zip(bufs, src):
+                    b.copy_(t)
+                execute(stream=side.cuda_stream, sync=False)
+        torch.cuda.current_stream().wait_stream(side)
+        for rep in range(9):                                  # the device's counter wraps at every fourth replay
+            for b in bufs:
+                b.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for r in range(world):
+                assert bits_equal(bufs[r], want[r]), f"replay {rep}, rank {r}: {mismatch_report(bufs[r], want[r])}"
+            if rep % 3 == 2:                                  # eager launches between the replays
+                for b, t in zip(bufs, src):
+                    b.copy_(t)
+                execute()
+                for r in range(world):
+                    assert bits_equal(bufs[r], want[r]), f"eager launch after replay {rep}, rank {r}"
+        eng.sync_operation(name)
+    finally:
+        eng.set_option("test_host_epoch_limit", 0x40000000 - 16)
+        eng.set_option("test_graph_epoch_limit", 0x7FFFFFF0)
+        eng.set_option("mode", "auto")

@@ -1,5 +1,5 @@
-"""Graphs that are not single chains, through the level-scheduled runner and (where the ops are
-position-aligned) the column runner: Pipeline-built graphs, fork / join over streams with several
+"""Graphs that are not single chains, through the level-scheduled runner, the persistent
+flag-ordered runner and (where the ops are position-aligned) the column runner: Pipeline-built graphs, fork / join over streams with several
 dependencies and successors per op, and `noop` nodes — the ground the reference covers with its
 DAG kernel (cuda_executor.cu:526-918: remaining_deps counters, up to 8 successors per op).
 """
@@ -25,7 +25,7 @@ def run(engine, name, jsons, inputs, mode):
 
 
 @pytest.mark.parametrize("world,depth,dtype", [(4, 2, "float32"), (8, 3, "bfloat16"), (3, 3, "float16")])
-@pytest.mark.parametrize("mode", ["column", "stepwise"])
+@pytest.mark.parametrize("mode", ["column", "stepwise", "persistent"])
 def test_pipeline_built_ring(engine_factory, world, depth, dtype, mode):
     """Steps rotate over `depth` channels (reference pccl/dsl/pipeline.py); consecutive steps of a
     rank are ordered only through the signal chain around the ring."""
@@ -71,8 +71,9 @@ def fork_join_graph(rank, chunk, dtype):
         return op.get_graph()
 
 
+@pytest.mark.parametrize("mode", ["auto", "stepwise", "persistent"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_fork_join_over_streams(engine_factory, dtype):
+def test_fork_join_over_streams(engine_factory, dtype, mode):
     chunk = 4099          # odd: offsets off 16-byte alignment
     jsons = [compile_to_json_string(fork_join_graph(r, chunk, dtype)) for r in range(2)]
     doc = json.loads(jsons[0])
@@ -81,14 +82,15 @@ def test_fork_join_over_streams(engine_factory, dtype):
     x = seeded_inputs("randn", 2, 9 * chunk, dtype, seed=9)
     want = oracle_buffers(jsons, x, dtype)
     engine = engine_factory(2)
-    got = run(engine, "fj", jsons, x, "auto")
+    got = run(engine, "fj", jsons, x, mode)
     info = engine.op_info("fj")
     assert info["position_aligned"] == 0 and info["num_levels"] == 3
     for r in range(2):
         assert bits_equal(got[r], want[r]), f"rank {r}: {mismatch_report(got[r], want[r])}"
 
 
-def test_noop_nodes_are_contracted(engine_factory):
+@pytest.mark.parametrize("mode", ["stepwise", "persistent", "column"])
+def test_noop_nodes_are_contracted(engine_factory, mode):
     """A `noop` between two data ops keeps their order and costs nothing: the linked program has
     the same data ops and levels as the graph without it."""
     world, n = 2, 4096
@@ -111,7 +113,7 @@ def test_noop_nodes_are_contracted(engine_factory):
     want = oracle_buffers(base, x, "float32")
     assert all(bits_equal(a, b) for a, b in zip(oracle_buffers(with_noop, x, "float32"), want))
     engine = engine_factory(world)
-    got = run(engine, "noop", with_noop, x, "stepwise")
+    got = run(engine, "noop", with_noop, x, mode)
     plain = engine_factory(world)
     for r, j in enumerate(base):
         plain.register_operation_json("plain", j, r)
@@ -122,7 +124,8 @@ def test_noop_nodes_are_contracted(engine_factory):
         assert bits_equal(got[r], want[r])
 
 
-def test_channelized_chain(engine_factory):
+@pytest.mark.parametrize("mode", ["auto", "stepwise", "persistent"])
+def test_channelized_chain(engine_factory, mode):
     """A chain whose data ops the channelize pass (reference pccl/dsl/passes/channelize.py) has
     moved to other channels while their dependencies still cross those channels: the labels change
     the queues the ops sit in, not their order."""
@@ -141,7 +144,7 @@ def test_channelized_chain(engine_factory):
     assert doc["operations"][4]["dependencies"] == [3]          # the chain still crosses the channels
     x = seeded_inputs("randn", world, 2 * pieces * chunk, "float16", seed=11)
     want = oracle_buffers(jsons, x, "float16")
-    got = run(engine_factory(world), "chan", jsons, x, "auto")
+    got = run(engine_factory(world), "chan", jsons, x, mode)
     for r in range(world):
         assert bits_equal(got[r], want[r]), mismatch_report(got[r], want[r])
         assert bits_equal(got[r][pieces * chunk:], x[1 - r][:pieces * chunk])

@@ -1,6 +1,6 @@
 """pccl_hip_execute_inplace_static: the in-place execution for callers that cannot allocate.  Called
-through the C ABI and compared bit for bit with pccl_hip_execute_inplace on the same inputs, on
-calls in a row that share the GPU's static workspace: a larger operation, then a smaller one (whose
+through the C ABI and compared bit for bit with the CPU oracle and with pccl_hip_execute_inplace on
+the same inputs, on calls in a row that share the GPU's static workspace: a larger operation, then a smaller one (whose
 tables replace the first one's and whose flags must not be confused with what the first left
 behind), then the first again, then repeated launches of one operation."""
 import ctypes
@@ -8,7 +8,7 @@ import ctypes
 import pytest
 import torch
 
-from helpers import bits_equal, graph_jsons, mismatch_report, seeded_inputs
+from helpers import bits_equal, graph_jsons, mismatch_report, oracle_buffers, seeded_inputs
 from pccl_amd import _lib
 from pccl_amd._lib import ERR_INVALID
 
@@ -40,15 +40,15 @@ def test_static_workspace_execution_matches_the_allocating_entry_point():
             "small": (graph_jsons("rhd", "build_allreduce", world, 3 * 4096, "float32", "sm", 1), 3 * 4096, "float32", "randn"),
             "tree": (graph_jsons("tree", "build_allreduce", world, 40000, "int32", "sm", 1, reduce_op="max"), 40000, "int32", "randint"),
         }
-        inputs, want = {}, {}
+        inputs, want, oracle_want = {}, {}, {}
         for name, (jsons, n, dtype, kind) in cases.items():
             _register(L, h, name, jsons)
-            inputs[name] = [t.cuda() for t in seeded_inputs(kind, world, n, dtype, seed=len(name))]
-        torch.cuda.synchronize()
-        free_before = torch.cuda.mem_get_info()[0]
+            host = seeded_inputs(kind, world, n, dtype, seed=len(name))
+            oracle_want[name] = oracle_buffers(jsons, host, dtype)
+            inputs[name] = [t.cuda() for t in host]
 
-        def run_static(name):
-            bufs = [t.clone() for t in inputs[name]]
+        def run_static(name, bufs=None):
+            bufs = bufs if bufs is not None else [t.clone() for t in inputs[name]]
             _lib.check(L.pccl_hip_execute_inplace_static(h, name.encode(), _ptrs(bufs), bufs[0].nbytes, _stream(), 1))
             return bufs
 
@@ -59,9 +59,23 @@ def test_static_workspace_execution_matches_the_allocating_entry_point():
         got["large2"] = run_static("large")
         got["tree"] = run_static("tree")
         torch.cuda.synchronize()
-        # nothing of the device's memory was taken by those calls beyond the clones made here
-        clones = sum(t.nbytes for bufs in got.values() for t in bufs)
-        assert free_before - torch.cuda.mem_get_info()[0] <= clones + (64 << 20), "the static entry point seems to have allocated"
+        for key, bufs in got.items():
+            name = "large" if key == "large2" else key
+            for r in range(world):
+                assert bits_equal(bufs[r], oracle_want[name][r]), f"{key} vs the oracle, rank {r}: {mismatch_report(bufs[r], oracle_want[name][r])}"
+
+        # Nothing is allocated: with every kernel of the path loaded by the calls above, alternating
+        # calls - each takes the workspace over from the other: fill, table-write and map kernels -
+        # on buffers made beforehand leave the device's free memory exactly where it was.
+        held = {name: [t.clone() for t in inputs[name]] for name in cases}
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        for i in range(6):
+            for name in ("large", "small", "tree"):
+                run_static(name, held[name])
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before, "the static entry point allocated device memory"
+        del held
 
         # the existing entry point on the same inputs (persistent runner and the default runner)
         for mode in ("persistent", "auto"):
@@ -110,18 +124,23 @@ def test_recorded_launches_and_a_workspace_that_changes_hands():
     a graph of the caller and every replay is compared with pccl_hip_execute_inplace, with eager
     work and synchronisations between the replays.  Then another operation takes the workspace over.
     A replay of the old graph now finds foreign tables behind its kernel arguments: it must execute
-    nothing (the buffers keep what they held), and the next synchronous call reports it.  After an
-    eager call of the first operation the same graph works again."""
+    nothing (the buffers keep what they held); the call that notices it - another operation's - is
+    not failed, and the first operation's next pccl_hip_sync reports it.  After an eager call of the
+    first operation the same graph works again."""
     L = _lib.lib()
     world, n = 8, 1 << 16
     h = ctypes.c_void_p()
     _lib.check(L.pccl_hip_create(ctypes.byref(h), 0, world))
     try:
-        _register(L, h, "a", graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2))
+        jsons_a = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2)
+        _register(L, h, "a", jsons_a)
         _register(L, h, "b", graph_jsons("rhd", "build_allreduce", world, 4096, "float32", "sm", 1))
-        src = [t.cuda() for t in seeded_inputs("randn", world, n, "bfloat16", seed=21)]
+        host_src = seeded_inputs("randn", world, n, "bfloat16", seed=21)
+        src = [t.cuda() for t in host_src]
         want = [t.clone() for t in src]
         _lib.check(L.pccl_hip_execute_inplace(h, b"a", _ptrs(want), want[0].nbytes, _stream(), 1))
+        for r, o in enumerate(oracle_buffers(jsons_a, host_src, "bfloat16")):
+            assert bits_equal(want[r], o), f"execute_inplace vs the oracle, rank {r}: {mismatch_report(want[r], o)}"
         bufs = [t.clone() for t in src]
         _lib.check(L.pccl_hip_execute_inplace_static(h, b"a", _ptrs(bufs), bufs[0].nbytes, _stream(), 1))
         for r in range(world):
@@ -153,8 +172,18 @@ def test_recorded_launches_and_a_workspace_that_changes_hands():
         torch.cuda.synchronize()
         for r in range(world):
             assert bits_equal(bufs[r], src[r]), f"a stale replay touched rank {r}"
-        rc = L.pccl_hip_execute_inplace_static(h, b"b", _ptrs(other), other[0].nbytes, _stream(), 1)
-        assert rc == ERR_INVALID and b"replayed after the static workspace" in L.pccl_hip_last_error()
+        # the operation that owns the workspace now runs normally and gives the same result as before
+        first_b = [t.clone() for t in other]
+        other2 = [t.cuda() for t in seeded_inputs("randn", world, 4096, "float32", seed=22)]
+        _lib.check(L.pccl_hip_execute_inplace_static(h, b"b", _ptrs(other2), other2[0].nbytes, _stream(), 1))
+        for r in range(world):
+            assert bits_equal(other2[r], first_b[r]), "the call that noticed the stale replay did not execute normally"
+        _lib.check(L.pccl_hip_sync(h, b"b"))
+        # the operation whose recorded launch it was hears of it at its own sync, once
+        assert L.pccl_hip_sync(h, b"a") == ERR_INVALID
+        msg = L.pccl_hip_last_error()
+        assert b"operation 'a'" in msg and b"executed nothing" in msg and b"unchanged" in msg, msg
+        _lib.check(L.pccl_hip_sync(h, b"a"))
 
         print("the first operation again, eagerly and from the graph", flush=True)
         again = [t.clone() for t in src]
