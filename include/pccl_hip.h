@@ -159,6 +159,10 @@ typedef struct {
     int32_t order_checked;      /* 1: the pairing of notifies and waits was checked for ambiguity; 0: the
                                    program has too many ops for the check (the pairing of one valid execution
                                    order is then used unverified) */
+    int32_t chain_segments;     /* segments of the column plan in chain form (one accumulator takes every rank's
+                                   original value in turn, the result goes to a set of ranks); equal to num_segments
+                                   when the whole plan can run on the phased runner, else 0 */
+    int32_t staged_chain_segments; /* the same for the plan of a staged call on the caller's tensors */
 } pccl_program_info;
 
 /* One data op of the linked program, for inspection and tests. */
@@ -242,6 +246,14 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * "slot_store_waves" = "-1" | "0" | "1" (1: the final broadcast of a program goes through LDS and each
  * wave stores whole tiles of some ranks; 0: every wave stores a slice of every rank; -1, the default:
  * 1 for plans that write at least four times what they read, such as an allgather);
+ * "phased" = "-1" | "0" | "1" (column plans in chain form - ring allreduce, staged reduce_scatter and
+ * allgather, trees under an operator that may be re-associated - on the phased runner: one persistent
+ * workgroup per CU, the whole chip reads, meets, writes, meets; -1, the default: when the tensors give
+ * every CU at least two 128 KiB chunks of each rank); "phased_shape" = "-1" | "0" | "1" (its workgroup:
+ * 512 threads x 16 vectors, or 256 x 32 with each wave on 32 KiB in a row; -1: by rank count);
+ * "phased_barriers" = "1" | "0" (0: no meetings, for comparison); "phased_timeout_us" (how long a
+ * workgroup waits at a meeting before the launch goes on unsynchronised: meetings order nothing; the
+ * environment variable PCCL_PHASED sets "phased" for new contexts);
  * "level_graph" = "0" | "1" (the level runner launches level by level, or replays the launches of an
  * execution as one HIP graph captured per set of rank pointers);
  * "trace_ranges" = "0" | "1" (host-side roctx ranges around the stages of a call, under the names of

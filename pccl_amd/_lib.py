@@ -50,7 +50,8 @@ class ProgramInfo(ctypes.Structure):
                 ("column_store_bytes", ctypes.c_int64), ("num_items", ctypes.c_int32),
                 ("num_gather_copies", ctypes.c_int32), ("staged_load_bytes", ctypes.c_int64),
                 ("staged_store_bytes", ctypes.c_int64), ("race_checked", ctypes.c_int32),
-                ("order_checked", ctypes.c_int32)]
+                ("order_checked", ctypes.c_int32), ("chain_segments", ctypes.c_int32),
+                ("staged_chain_segments", ctypes.c_int32)]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_ if not n.endswith("_")}

@@ -128,6 +128,8 @@ void fill_info(const Program& p, pccl_program_info* out) {
     out->staged_store_bytes = p.direct_store_bytes;
     out->race_checked = p.race_checked;
     out->order_checked = p.order_checked;
+    out->chain_segments = (int)p.chain_segs.size();
+    out->staged_chain_segments = (int)p.direct_chain_segs.size();
 }
 
 // What a linked program does differently from the reference, said once at link time (WARN, the
@@ -327,12 +329,18 @@ struct OpEntry {
     bool host_linked = false;
     struct HostTables {
         std::vector<DevColSegment> segs, direct_segs;
+        std::vector<DevChainSegment> chain_segs, direct_chain_segs;   // phased runner (empty: the plan is not a chain plan)
+        std::vector<int32_t> chain_srcs;                               // one word per source rank, padded to whole 8-byte words
         std::vector<DevGatherCopy> gather;
         std::vector<DevStepOp> step_ops;
         std::vector<int32_t> item_op;
         std::vector<int32_t> step_deps_padded;   // the dependency lists padded to whole 8-byte words
     } host;
     DevBuf segs, direct_segs, instrs, pre, step_ops, step_deps, item_op, state;
+    DevBuf chain_segs, direct_chain_segs, chain_srcs, phase_sync;
+    int64_t chain_chunks = 0, direct_chain_chunks = 0;   // phased runner: chunks of the two chain plans
+    int chain_seg_chunks = 0, direct_chain_seg_chunks = 0;   // > 0: every segment has this many chunks
+    int chain_tree = 0, direct_chain_tree = 0;               // the plan holds balanced trees: the shape it runs on (0: none)
     int64_t total_tiles = 0, direct_tiles = 0;
     int seg_tiles = 0, direct_seg_tiles = 0;   // > 0: every segment of the plan has this many tiles
     int vecs_per_thread = 0;
@@ -366,6 +374,7 @@ struct OpEntry {
         gather.release(); gather_tiles = 0;
         segs.release(); direct_segs.release(); instrs.release(); pre.release(); step_ops.release(); step_deps.release();
         item_op.release(); state.release();
+        chain_segs.release(); direct_chain_segs.release(); chain_srcs.release(); phase_sync.release();
         if (ev0) (void)hipEventDestroy(ev0);
         if (ev1) (void)hipEventDestroy(ev1);
         ev0 = ev1 = nullptr;
@@ -427,6 +436,11 @@ struct pccl_hip_ctx {
     bool slot_direct = true;              // slot runner fetches first touches straight into LDS
     int slot_store_waves = -1;            // slot runner: broadcast tail through LDS, whole tiles of a rank stored by one wave
                                           // (1), every wave a slice of every rank (0), or chosen from the plan's traffic (-1)
+    int phased = -1;                      // chain plans on the phased runner (whole chip reads, then writes): 1 whenever the
+                                          // plan is a chain plan, 0 never, -1 when it is and the tensors are large enough
+    int phased_shape = -1;                // its workgroup: 0 = 512 threads x 16 vectors, 1 = 256 x 32 (a wave's vectors contiguous), -1 chosen
+    bool phased_barriers = true;          // its workgroups meet between the phases (0: they run free, for comparison)
+    int phased_timeout_us = 1000;         // how long a workgroup waits at a meeting point before the launch goes on unsynchronised
     bool level_graph = false;             // level runner replays its launches as one HIP graph (measured:
                                           // no faster than launching level by level, so off by default)
     hipStream_t capture_stream = nullptr; // private stream the level launches are captured on
@@ -543,6 +557,40 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
         };
         e.host.segs = device_segments(P.segs, &e.total_tiles, &e.seg_tiles);
         if (!P.direct_segs.empty()) e.host.direct_segs = device_segments(P.direct_segs, &e.direct_tiles, &e.direct_seg_tiles);
+        // chain plans for the phased runner (both of its workgroup shapes take chunks of the same size)
+        static_assert(phased_chunk_vecs(0) == phased_chunk_vecs(1), "one chunk table serves both chain shapes");
+        auto chain_segments = [&](const std::vector<ChainSegment>& segs, int64_t* total, int* uniform, int* tree_shape) {
+            std::vector<DevChainSegment> ds(segs.size());
+            int64_t chunks = 0;
+            int depth = 0;
+            for (const ChainSegment& c : segs) depth = std::max(depth, c.tree_depth);
+            // a plan with balanced trees runs on a shape that keeps their partial results in registers:
+            // 16 vectors per thread for f32 trees of up to 16 ranks, 8 for deeper trees and for the
+            // element types whose arithmetic needs registers of its own
+            *tree_shape = depth == 0 ? 0 : depth <= 4 ? 2 : 3;
+            const int64_t chunk_v = phased_chunk_vecs(*tree_shape);
+            for (size_t i = 0; i < segs.size(); ++i) {
+                const ChainSegment& c = segs[i];
+                DevChainSegment& d = ds[i];
+                d.start = c.start; d.end = c.end;
+                d.first_vec = c.start / ve;
+                const int64_t last_vec = (c.end - 1) / ve;
+                d.first_chunk = chunks;
+                chunks += (last_vec - d.first_vec + 1 + chunk_v - 1) / chunk_v;
+                d.src_start = c.src_start; d.n_src = c.n_src; d.redop = c.redop; d.tree_depth = c.tree_depth; d.store_mask = c.store_mask;
+            }
+            *total = chunks;
+            const int64_t per = ds.size() > 1 ? ds[1].first_chunk : chunks;
+            bool same = per > 0 && chunks == per * (int64_t)ds.size() && chunks < ((int64_t)1 << 32) && per <= INT32_MAX;
+            for (size_t i = 0; i < ds.size() && same; ++i) same = ds[i].first_chunk == (int64_t)i * per;
+            *uniform = same ? (int)per : 0;
+            return ds;
+        };
+        e.chain_chunks = e.direct_chain_chunks = 0;
+        e.host.chain_segs = chain_segments(P.chain_segs, &e.chain_chunks, &e.chain_seg_chunks, &e.chain_tree);
+        e.host.direct_chain_segs = chain_segments(P.direct_chain_segs, &e.direct_chain_chunks, &e.direct_chain_seg_chunks, &e.direct_chain_tree);
+        e.host.chain_srcs.assign(P.chain_srcs.begin(), P.chain_srcs.end());
+        if (e.host.chain_srcs.size() % 2) e.host.chain_srcs.push_back(0);
     }
     if (!P.gather.empty()) {
         std::vector<DevGatherCopy> gc(P.gather.size());
@@ -616,6 +664,13 @@ void link_entry(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t stream = nullptr, boo
         e.pre.upload(P.col_pre.data(), P.col_pre.size() * sizeof(uint64_t));
     }
     e.gather.upload(h.gather.data(), h.gather.size() * sizeof(DevGatherCopy));
+    e.chain_segs.upload(h.chain_segs.data(), h.chain_segs.size() * sizeof(DevChainSegment));
+    e.direct_chain_segs.upload(h.direct_chain_segs.data(), h.direct_chain_segs.size() * sizeof(DevChainSegment));
+    e.chain_srcs.upload(h.chain_srcs.data(), h.chain_srcs.size() * sizeof(int32_t));
+    if (!h.chain_segs.empty() || !h.direct_chain_segs.empty()) {
+        const PhaseSync zero{};
+        e.phase_sync.upload(&zero, sizeof(zero));
+    }
     e.step_ops.upload(h.step_ops.data(), h.step_ops.size() * sizeof(DevStepOp));
     e.step_deps.upload(P.step_deps.data(), P.step_deps.size() * sizeof(int32_t));
     e.item_op.upload(h.item_op.data(), h.item_op.size() * sizeof(int32_t));
@@ -693,6 +748,47 @@ int launch_levels(pccl_hip_ctx* ctx, OpEntry& e, const StepwiseLaunch& L, const 
     return (int)hipGraphLaunch(hit->exec, stream);
 }
 
+// Whether a column-mode execution goes to the phased runner, and its launch.  `direct`: the staged
+// call's plan on the caller's tensors.  The phased runner pays when every CU has several chunks to
+// work through; small tensors stay with the slot runner, whose many small workgroups start and end
+// faster.
+bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
+    const int64_t chunks = direct ? e.direct_chain_chunks : e.chain_chunks;
+    const DevBuf& segs = direct ? e.direct_chain_segs : e.chain_segs;
+    if (ctx->phased == 0 || chunks <= 0 || !segs.p || !e.phase_sync.p) return false;
+    if (ctx->phased == 1) return true;
+    // a plan that mostly writes (an allgather: one chunk in, R out) has no read phase to speak of and
+    // is faster with the slot runner's wave-dealt stores (8 x 512 MB fp16: 0.80 against 0.86 ms)
+    const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
+    const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
+    if (2 * loads < stores) return false;
+    // plans with balanced trees: the shapes that hold their partial results are slower than the slot
+    // runner so far (16 ranks x 64 MiB f32 halving-doubling 0.43 against 0.37 ms): only on request
+    if ((direct ? e.direct_chain_tree : e.chain_tree) != 0) return false;
+    return chunks >= 2 * (int64_t)device_cu_count(ctx->device);
+}
+
+int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtrs& ptrs, hipStream_t stream) {
+    const Program& P = e.prog;
+    PhasedLaunch L{};
+    L.segs = (const DevChainSegment*)(direct ? e.direct_chain_segs.p : e.chain_segs.p);
+    L.num_segs = (int)(direct ? P.direct_chain_segs.size() : P.chain_segs.size());
+    L.srcs = (const int32_t*)e.chain_srcs.p;
+    L.total_chunks = direct ? e.direct_chain_chunks : e.chain_chunks;
+    L.seg_chunks = direct ? e.direct_chain_seg_chunks : e.chain_seg_chunks;
+    L.dtype = P.dtype;
+    // 8 ranks and fewer: two waves per SIMD with 16 vectors each; more ranks: one wave per SIMD that
+    // streams 32 KiB of every rank in a row (measured with bare kernels: 8 ranks 80 % against 78 % of
+    // peak, 32 ranks 81 % against 83 %)
+    const int tree_shape = direct ? e.direct_chain_tree : e.chain_tree;
+    L.shape = tree_shape ? tree_shape : ctx->phased_shape >= 0 ? ctx->phased_shape : (ctx->R <= 8 ? 0 : 1);
+    L.num_blocks = ctx->num_blocks;
+    L.barriers = ctx->phased_barriers ? 1 : 0;
+    L.sync = (PhaseSync*)e.phase_sync.p;
+    L.timeout_ticks = (uint64_t)ctx->phased_timeout_us * 100ull;
+    return launch_phased(L, ptrs, stream);
+}
+
 // Enqueue the program on `stream` over the rank buffers `rank_bufs` (R pointers).
 void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t buf_bytes, hipStream_t stream) {
     const Program& P = e.prog;
@@ -717,7 +813,9 @@ void run_program(pccl_hip_ctx* ctx, OpEntry& e, char* const* rank_bufs, size_t b
     if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
     int rc;
     TraceRange range(ctx->trace_ranges, column ? "fused_kernel" : "executor_kernel");
-    if (column) {
+    if (column && wants_phased(ctx, e, false)) {
+        rc = launch_phased_plan(ctx, e, false, ptrs, stream);
+    } else if (column) {
         ColumnLaunch L{};
         L.segs = (const DevColSegment*)e.segs.p; L.num_segs = (int)P.segs.size();
         L.instrs = (const uint64_t*)e.instrs.p; L.pre = (const uint64_t*)e.pre.p;
@@ -791,6 +889,13 @@ bool run_direct(pccl_hip_ctx* ctx, OpEntry& e, const void* const* inputs, void* 
         ptrs.p[PCCL_HIP_MAX_VRANKS + r] = (char*)in_base;
     }
     if (ctx->timing) HIP_TRY(hipEventRecord(e.ev0, stream));
+    if (wants_phased(ctx, e, true)) {
+        TraceRange exe(ctx->trace_ranges, "execute"), range(ctx->trace_ranges, "fused_kernel");
+        const int prc = launch_phased_plan(ctx, e, true, ptrs, stream);
+        if (prc != 0) throw Error{PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)prc)};
+        if (ctx->timing) { HIP_TRY(hipEventRecord(e.ev1, stream)); e.timed = true; }
+        return true;
+    }
     ColumnLaunch L{};
     L.segs = (const DevColSegment*)e.direct_segs.p; L.num_segs = (int)P.direct_segs.size();
     L.instrs = (const uint64_t*)e.instrs.p; L.pre = (const uint64_t*)e.pre.p;
@@ -1048,6 +1153,7 @@ int pccl_hip_create(pccl_hip_ctx** out, int device, int num_vranks) {
         if (const char* nb = std::getenv("PCCL_NUM_BLOCKS")) ctx->num_blocks = std::atoi(nb);
         if (std::getenv("PCCL_DISABLE_FUSED")) ctx->mode = Mode::Stepwise;
         if (const char* tr = std::getenv("PCCL_TRACE_RANGES")) ctx->trace_ranges = std::atoi(tr) != 0;
+        if (const char* ph = std::getenv("PCCL_PHASED")) { const int x = std::atoi(ph); if (x >= -1 && x <= 1) ctx->phased = x; }
         if (log_threshold() <= LOG_INFO)   // reference engine_c.cc:84,163
             log_line(LOG_INFO, "engine context on device " + std::to_string(device) + " with " + std::to_string(num_vranks) + " virtual ranks");
         *out = ctx.release();
@@ -1128,6 +1234,18 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             ctx->slot_store_waves = v;
         }
         else if (k == "level_graph") ctx->level_graph = std::atoi(value) != 0;
+        else if (k == "phased") {
+            const int x = std::atoi(value);
+            if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased must be -1 (automatic), 0 or 1");
+            ctx->phased = x;
+        }
+        else if (k == "phased_shape") {
+            const int x = std::atoi(value);
+            if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased_shape must be -1 (automatic), 0 (512 threads x 16 vectors) or 1 (256 x 32)");
+            ctx->phased_shape = x;
+        }
+        else if (k == "phased_barriers") ctx->phased_barriers = std::atoi(value) != 0;
+        else if (k == "phased_timeout_us") { ctx->phased_timeout_us = std::atoi(value); if (ctx->phased_timeout_us < 0) ctx->phased_timeout_us = 0; }
         else if (k == "lds_slots") { ctx->lds_slots = std::atoi(value) != 0; relink = true; }
         else if (k == "slot_direct" || k == "slot_threads" || k == "slot_vecs") {
             // checked against the shape linking would choose with the new value in place
@@ -1184,6 +1302,10 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
         else if (k == "slot_direct") v = std::to_string((int)ctx->slot_direct);
         else if (k == "slot_store_waves") v = std::to_string(ctx->slot_store_waves);
         else if (k == "level_graph") v = std::to_string((int)ctx->level_graph);
+        else if (k == "phased") v = std::to_string(ctx->phased);
+        else if (k == "phased_shape") v = std::to_string(ctx->phased_shape);
+        else if (k == "phased_barriers") v = std::to_string((int)ctx->phased_barriers);
+        else if (k == "phased_timeout_us") v = std::to_string(ctx->phased_timeout_us);
         else if (k == "lds_slots") v = std::to_string((int)ctx->lds_slots);
         else if (k == "slot_threads") v = std::to_string(ctx->slot_threads);
         else if (k == "slot_vecs") v = std::to_string(ctx->slot_vecs);

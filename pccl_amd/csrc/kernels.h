@@ -79,6 +79,46 @@ struct ColumnLaunch {
     int32_t seg_tiles;        // > 0: every segment has this many tiles (segment = tile / seg_tiles, fewer than 2^32 tiles); 0: search
 };
 
+// One segment of a chain plan (see ChainSegment in program.h) as the phased runner reads it.
+struct DevChainSegment {
+    int64_t start, end;        // element positions
+    int64_t first_vec;         // start / vector elems
+    int64_t first_chunk;       // prefix sum of chunks
+    int32_t src_start, n_src;  // words in PhasedLaunch::srcs: the ranks whose values are combined, in order
+    int32_t redop;
+    int32_t tree_depth;        // 0: a chain; D > 0: a perfectly balanced tree over the 2^D ranks of srcs, left to right
+    uint64_t store_mask;       // ranks that receive the result
+};
+static_assert(sizeof(DevChainSegment) == 56, "DevChainSegment is read 8 bytes at a time");
+
+// Meeting point of the phased runner's workgroups (device memory, zero between launches: the last
+// workgroup to leave a launch clears it).
+struct PhaseSync {
+    int32_t arrive;  int32_t pad0[31];   // arrivals at the current barrier
+    int32_t release; int32_t pad1[31];   // number of the last barrier that everybody has reached
+    int32_t broken;                      // a wait ran out of time: no more waiting in this launch
+    int32_t exited;                      // workgroups that have left the launch
+    int32_t pad2[30];
+};
+
+struct PhasedLaunch {
+    const DevChainSegment* segs;
+    int32_t num_segs;
+    const int32_t* srcs;      // the segments' source ranks, one 32-bit word each
+    int64_t total_chunks;
+    int32_t seg_chunks;       // > 0: every segment has this many chunks; 0: search
+    int32_t dtype;
+    int32_t shape;            // 0: 512 threads x 16 vectors, 1: 256 threads x 32 vectors (each wave a contiguous 32 KiB),
+                              // 2: 1024 threads x 4 vectors, also runs balanced trees of up to 16 ranks,
+                              // 3: 512 threads x 4 vectors, also runs balanced trees of up to 64 ranks
+    int32_t num_blocks;       // 0: one workgroup per CU
+    int32_t barriers;         // 1: all workgroups read together, then write together; 0: no meeting
+    PhaseSync* sync;
+    uint64_t timeout_ticks;   // 100 MHz ticks a workgroup waits at a meeting point before it goes on alone
+};
+// Vectors of every rank one workgroup of the given shape takes per sweep.
+PCCL_HD constexpr int64_t phased_chunk_vecs(int shape) { return shape == 2 ? 1024 * 4 : shape == 3 ? 512 * 4 : 8192; }
+
 struct StepwiseLaunch {
     const DevStepOp* ops;
     int32_t num_ops;
@@ -105,6 +145,7 @@ constexpr int32_t kGraphEpochLimit = 0x7FFFFFF0;
 // All return a hipError_t value as int (0 = success).
 int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream);
 int launch_persistent(const StepwiseLaunch& L, const RankPtrs& ptrs, void* stream);
+int launch_phased(const PhasedLaunch& L, const RankPtrs& ptrs, void* stream);
 // One dependency level: items [item_begin, item_end) of the work list.
 int launch_level(const StepwiseLaunch& L, int item_begin, int item_end, const RankPtrs& ptrs, void* stream);
 int launch_reduce(int dtype, int redop, const void* a, const void* b, void* c, size_t n, void* stream);

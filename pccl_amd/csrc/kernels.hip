@@ -1096,6 +1096,246 @@ __global__ __launch_bounds__(1024 / V) void column_slot_kernel(ColumnLaunch L, R
     }
 }
 
+// ------------------------------------------------------------------------------- phased runner
+//
+// Chain programs - one accumulator per position takes the ranks' original values one after another
+// and the result goes to every rank of a mask: ring allreduce segments, staged reduce_scatter and
+// allgather, trees under an operator that may be re-associated - run on a persistent grid of one
+// workgroup per CU in which the WHOLE CHIP reads together and then writes together.  A workgroup
+// takes a chunk of T x V vectors of every rank per sweep and keeps its V accumulators per thread in
+// registers: read phase = every source rank's chunk streamed in through a small ring of LDS slots
+// and combined; all workgroups meet; write phase = the accumulators stored to every rank of the
+// mask; all meet again.  The memory system then sees long runs of pure reads and pure writes instead
+// of a mix (measured on MI355X with bare kernels of this traffic shape, in place: 8 ranks x 512 MiB
+// 67 % of the 8 TB/s peak without the meetings, 80 % with them, against 77 % for the best
+// one-tile-per-workgroup shape; 32 ranks x 96 MiB 67 / 83 / 73 %).  The traffic is the same as the
+// slot runner's: every rank read once, written once.
+//
+// The meetings order nothing - a workgroup only ever touches its own chunk - so they cannot make a
+// result wrong, and they are bounded: a workgroup that waits longer than `timeout_ticks` (some
+// workgroup is not resident, the GPU is shared) marks the launch as unsynchronised and everybody
+// goes on without further waiting.  The last workgroup to leave clears the meeting block.
+//
+// Chunks that a segment boundary cuts are run vector by vector by the same workgroup (loads and
+// stores of one vector together, cut vectors stored element by element): there are at most two per
+// segment.
+
+// One workgroup per CU: the kernel asks for more than half a CU's LDS, so that two cannot share one.
+constexpr int kPhasedLdsBytes = 84 * 1024;
+
+__device__ __forceinline__ void stv_nt_s(char* uniform_base, uint32_t off, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, %2 sc1 nt\n\ts_nop 0" : : "v"(off), "v"(v), "s"(uniform_base) : "memory");
+}
+__device__ __forceinline__ void load_lds_nt(const char* uniform_base, uint32_t off, u32x4* wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(uniform_base + off),
+                                     (__attribute__((address_space(3))) void*)wave_base, 16, 0, 2 /* nt */);
+}
+
+__device__ __forceinline__ void phase_arrive(PhaseSync* s, int gen, int G) {
+    if (threadIdx.x == 0) {
+        const int old = __hip_atomic_fetch_add(&s->arrive, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old + 1 == gen * G) __hip_atomic_store(&s->release, gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+// Returns false once the launch is unsynchronised (this or another workgroup waited too long).
+__device__ __forceinline__ bool phase_wait(PhaseSync* s, int gen, uint64_t timeout_ticks, int* s_flag) {
+    if (threadIdx.x == 0) {
+        int ok = 1;
+        const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+        while (__hip_atomic_load(&s->release, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gen) {
+            if (__hip_atomic_load(&s->broken, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { ok = 0; break; }
+            if (__builtin_amdgcn_s_memrealtime() - t0 > timeout_ticks) {
+                __hip_atomic_store(&s->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ok = 0;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+        }
+        *s_flag = ok;
+    }
+    __syncthreads();
+    const int ok = __builtin_amdgcn_readfirstlane(*s_flag);
+    __syncthreads();   // the flag may be rewritten by the next meeting
+    return ok != 0;
+}
+
+// Read phase of one chunk: ranks srcs[0 .. n) streamed through a ring of S LDS slots per thread
+// (S divides V, so the slot of vector v is v % S whatever the rank) and combined into acc[].
+// Fetch q = k V + v is issued when fetch q - S has been consumed; loads complete in order, so
+// "at most S - 1 outstanding" means fetch q has landed.
+template <int DT, int OP, int T, int V, int S, int VS, int GR, int TREE>
+__device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int32_t* srcs, int n, int tree_depth, const RankPtrs& ptrs,
+                                           u32x4* lds, int64_t chunk_byte0, uint32_t toff, int tid) {
+    static_assert(V % S == 0 && S <= V && S % GR == 0, "the slot of a vector must not depend on the rank; groups of GR vectors per wait");
+    // trees only arise under an operator whose result depends on the order: sums (maxima, minima and
+    // integer sums are re-associated into chains by the planner)
+    constexpr bool kTrees = TREE > 0 && OP == PCCL_SUM && DT != PCCL_I32;
+    constexpr int kMaxDepth = kTrees ? TREE : 1;
+    // kTrees: the left siblings that wait for their right halves, one per level (a binary counter over
+    // the leaf number: leaf k is combined upwards through every level whose bit is set in k and parked
+    // at the first level whose bit is clear).  All register indices are compile-time; the branches
+    // are uniform.
+    u32x4 parked[kMaxDepth][V];
+    u32x4* const my = lds + (tid & ~63);
+    const u32x4* const mine = lds + tid;
+    const char* cur = ptrs.p[kMaxR + srcs[0]] + chunk_byte0;
+#pragma unroll
+    for (int q = 0; q < S; ++q) load_lds_nt(cur, toff + q * VS, my + q * T);
+    for (int k = 0; k < n; ++k) {
+        const bool last_rank = k + 1 == n;
+        const char* next = ptrs.p[kMaxR + srcs[last_rank ? k : k + 1]] + chunk_byte0;
+#pragma unroll
+        for (int v = 0; v < V; v += GR) {
+            // the GR oldest fetches have landed when at most S - GR are outstanding
+            if (v + S >= V && last_rank) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(S - GR) : "memory");
+            u32x4 x[GR];
+#pragma unroll
+            for (int g = 0; g < GR; ++g) x[g] = mine[((v + g) % S) * T];
+            if (!kTrees || tree_depth == 0) {
+#pragma unroll
+                for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_fast<DT, OP>(x[g], acc[v + g]);
+            } else {
+                // levels this leaf climbs: the trailing one bits of its number (uniform)
+                int climb = __builtin_ctz(~(unsigned)k);
+                if (climb > tree_depth) climb = tree_depth;
+#pragma unroll
+                for (int g = 0; g < GR; ++g) {
+                    u32x4 y = x[g];
+#pragma unroll
+                    for (int lvl = 0; lvl < kMaxDepth; ++lvl)
+                        if (lvl < climb) y = vec_fast<DT, OP>(parked[lvl][v + g], y);
+#pragma unroll
+                    for (int lvl = 0; lvl < kMaxDepth; ++lvl)
+                        if (lvl == climb && lvl < tree_depth) parked[lvl][v + g] = y;
+                    if (climb == tree_depth) acc[v + g] = y;      // the last leaf: the root
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
+#pragma unroll
+            for (int g = 0; g < GR; ++g) {
+                const int w = v + g;
+                if (w + S < V) load_lds_nt(cur, toff + (w + S) * VS, my + (w % S) * T);
+                else if (!last_rank) load_lds_nt(next, toff + (w + S - V) * VS, my + (w % S) * T);
+            }
+        }
+        cur = next;
+    }
+}
+
+template <int DT, int T, int V, int S, bool WAVEC, int GR, int TREE>
+__global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs) {
+    extern __shared__ u32x4 lds[];
+    __shared__ int s_flag;
+    static_assert((size_t)S * T * 16 + 64 <= (size_t)kPhasedLdsBytes, "the fetch ring must fit the LDS the launcher asks for");
+    constexpr int ES = ElemBytes<DT>::value;
+    constexpr int VE = 16 / ES;
+    constexpr int64_t CHUNK_V = (int64_t)T * V;
+    constexpr int VS = WAVEC ? 64 * 16 : T * 16;             // bytes between a thread's consecutive vectors
+    const int tid = threadIdx.x;
+    const int G = gridDim.x;
+    // workgroup b runs on XCD b % 8: every XCD takes a contiguous eighth of each sweep
+    const int place = (G & 7) == 0 ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    // thread's first vector inside a chunk: each wave a contiguous V KiB, or the chunk as V slabs of T vectors
+    const uint32_t tvec = WAVEC ? (uint32_t)(tid >> 6) * V * 64 + (tid & 63) : (uint32_t)tid;
+    const uint32_t toff = tvec * 16;
+    const int64_t sweeps = (L.total_chunks + G - 1) / G;
+    bool meet = L.barriers != 0;
+    int gen = 0;
+    for (int64_t it = 0; it < sweeps; ++it) {
+        const int64_t chunk = it * G + place;
+        const bool live = chunk < L.total_chunks;
+        u32x4 acc[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] = u32x4{0, 0, 0, 0};
+        DevChainSegment seg{};
+        int64_t vbase = 0;
+        bool whole = false;
+        if (live) {
+            int lo = 0;
+            if (L.seg_chunks > 0) {
+                const uint32_t per = (uint32_t)L.seg_chunks;
+                lo = (per & (per - 1)) == 0 ? (int)((uint32_t)chunk >> __builtin_ctz(per)) : (int)((uint32_t)chunk / per);
+            } else {
+                int hi = L.num_segs;
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (as_const(L.segs)[mid].first_chunk <= chunk) lo = mid; else hi = mid;
+                }
+            }
+            seg = load_const(L.segs + lo);
+            vbase = seg.first_vec + (chunk - seg.first_chunk) * CHUNK_V;
+            whole = vbase * VE >= seg.start && (vbase + CHUNK_V) * VE <= seg.end;
+            const PCCL_CONST int32_t* srcs = as_const(L.srcs) + seg.src_start;   // dwords: uniform reads become scalar loads
+            if (whole) {
+                if (seg.redop == PCCL_SUM) chain_read<DT, PCCL_SUM, T, V, S, VS, GR, TREE>(acc, srcs, seg.n_src, seg.tree_depth, ptrs, lds, vbase * 16, toff, tid);
+                else if (seg.redop == PCCL_MAX) chain_read<DT, PCCL_MAX, T, V, S, VS, GR, TREE>(acc, srcs, seg.n_src, seg.tree_depth, ptrs, lds, vbase * 16, toff, tid);
+                else chain_read<DT, PCCL_MIN, T, V, S, VS, GR, TREE>(acc, srcs, seg.n_src, seg.tree_depth, ptrs, lds, vbase * 16, toff, tid);
+            } else {
+                // a chunk that the segment's ends cut: vector by vector, loads and stores together
+                for (int64_t j = tid; j < CHUNK_V; j += T) {
+                    const int64_t vec = vbase + j;
+                    int64_t e0 = vec * VE, e1 = e0 + VE;
+                    if (e0 < seg.start) e0 = seg.start;
+                    if (e1 > seg.end) e1 = seg.end;
+                    if (e0 >= e1) continue;
+                    u32x4 x = ldv(ptrs.p[kMaxR + srcs[0]] + vec * 16);
+                    if (TREE == 0 || seg.tree_depth == 0) {
+                        for (int k = 1; k < seg.n_src; ++k) x = vec_op<DT>(ldv(ptrs.p[kMaxR + srcs[k]] + vec * 16), x, seg.redop);
+                    } else {
+                        u32x4 parked[6];
+                        for (int k = 0; k < seg.n_src; ++k) {
+                            u32x4 y = k == 0 ? x : ldv(ptrs.p[kMaxR + srcs[k]] + vec * 16);
+                            bool placed = false;
+#pragma unroll
+                            for (int lvl = 0; lvl < 6; ++lvl) {
+                                if (!placed && lvl < seg.tree_depth) {
+                                    if (k >> lvl & 1) y = vec_op<DT>(parked[lvl], y, seg.redop);
+                                    else { parked[lvl] = y; placed = true; }
+                                }
+                            }
+                            if (!placed) x = y;
+                        }
+                    }
+                    for (uint64_t m = seg.store_mask; m; m &= m - 1)
+                        store_vector_part<DT>(ptrs.p[__builtin_ctzll(m)] + vec * 16, x, (int)(e0 - vec * VE), (int)(e1 - vec * VE));
+                }
+            }
+        }
+        if (meet) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            ++gen;
+            phase_arrive(L.sync, gen, G);
+            meet = phase_wait(L.sync, gen, L.timeout_ticks, &s_flag);
+        }
+        if (live && whole) {
+            for (uint64_t m = seg.store_mask; m; m &= m - 1) {
+                char* const dst = ptrs.p[__builtin_ctzll(m)] + vbase * 16;
+#pragma unroll
+                for (int v = 0; v < V; ++v) stv_nt_s(dst, toff + v * VS, acc[v]);
+            }
+        }
+        if (meet && it + 1 < sweeps) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            ++gen;
+            phase_arrive(L.sync, gen, G);
+            meet = phase_wait(L.sync, gen, L.timeout_ticks, &s_flag);
+        }
+    }
+    // the last workgroup to leave clears the meeting block for the next launch
+    if (L.barriers != 0 && tid == 0) {
+        const int old = __hip_atomic_fetch_add(&L.sync->exited, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old + 1 == G) {
+            __hip_atomic_store(&L.sync->arrive, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->release, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->broken, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->exited, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------- launchers
 
 // Per-device facts, queried once.  Contexts on different threads may ask at the same time: the
@@ -1193,6 +1433,46 @@ int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
         case PCCL_I32: return launch_column_dt<PCCL_I32>(L, ptrs, s);
         case PCCL_F8E4M3: return launch_column_dt<PCCL_F8E4M3>(L, ptrs, s);
         case PCCL_F8E5M2: return launch_column_dt<PCCL_F8E5M2>(L, ptrs, s);
+        default: return (int)hipErrorInvalidValue;
+    }
+}
+
+template <class K>
+static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads, const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
+    const int dev = current_device();
+    if (!allowed[dev].load(std::memory_order_relaxed)) {
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kPhasedLdsBytes);
+        if (rc != hipSuccess) return (int)rc;
+        allowed[dev].store(1, std::memory_order_relaxed);
+    }
+    int64_t grid = L.num_blocks > 0 ? L.num_blocks : current_cus();
+    if (grid > L.total_chunks) grid = L.total_chunks;
+    if (grid <= 0) return 0;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(threads), (size_t)kPhasedLdsBytes, s, L, ptrs);
+    return (int)hipGetLastError();
+}
+
+template <int DT>
+static int launch_phased_dt(const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
+    static std::atomic<int> allowed[4][kMaxDevices];
+    switch (L.shape) {
+        case 0: return launch_phased_kernel(phased_kernel<DT, 512, 16, 4, false, 2, 0>, allowed[0], 512, L, ptrs, s);
+        case 1: return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, true, 2, 0>, allowed[1], 256, L, ptrs, s);
+        case 2: return launch_phased_kernel(phased_kernel<DT, 1024, 4, 4, false, 2, 4>, allowed[2], 1024, L, ptrs, s);
+        case 3: return launch_phased_kernel(phased_kernel<DT, 512, 4, 4, false, 2, 6>, allowed[3], 512, L, ptrs, s);
+        default: return (int)hipErrorInvalidValue;
+    }
+}
+
+int launch_phased(const PhasedLaunch& L, const RankPtrs& ptrs, void* stream) {
+    hipStream_t s = (hipStream_t)stream;
+    switch (L.dtype) {
+        case PCCL_F32: return launch_phased_dt<PCCL_F32>(L, ptrs, s);
+        case PCCL_F16: return launch_phased_dt<PCCL_F16>(L, ptrs, s);
+        case PCCL_BF16: return launch_phased_dt<PCCL_BF16>(L, ptrs, s);
+        case PCCL_I32: return launch_phased_dt<PCCL_I32>(L, ptrs, s);
+        case PCCL_F8E4M3: return launch_phased_dt<PCCL_F8E4M3>(L, ptrs, s);
+        case PCCL_F8E5M2: return launch_phased_dt<PCCL_F8E5M2>(L, ptrs, s);
         default: return (int)hipErrorInvalidValue;
     }
 }

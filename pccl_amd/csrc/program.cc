@@ -123,6 +123,120 @@ static void count_column_traffic(const Program& P, const ColSegment& seg, int es
             if ((P.col_pre[seg.pre_start + w] >> (8 * j) & 0xFF) != 0xFF) *slot_loads += bytes;
 }
 
+// The chain form of a finished column program, if it has one (see ChainSegment).  The program is
+// evaluated symbolically: every value is a leaf (the original content of a rank) or the combination
+// of two values.  It is a chain when all ranks that are written to memory end up holding one and the
+// same value and that value combines every leaf at most once, either literally as a chain (each
+// combination takes one leaf and the chain so far: any element type and operator, the order is kept)
+// or in any shape under an operator whose result does not depend on the order for this element
+// type: wrapping integer addition, and maximum / minimum of any type (IEEE 754-2019 maximum and
+// minimum are associative and commutative, signed zeros and NaN - written canonically - included),
+// or - third form, reported through depth_out - as a perfectly balanced binary tree, whose shape is
+// kept (floating-point sums of halving-doubling and tree schedules).
+// Operand order within one combination never matters: every operator here is commutative bit for bit.
+static bool chain_form(const Program& P, const ColSegment& seg, int dtype, std::vector<uint8_t>* srcs, int* redop_out, uint64_t* mask_out, int* depth_out) {
+    *depth_out = 0;
+    struct Val { int a = -1, b = -1, leaf = -1, redop = 0; };   // leaf >= 0: original content of that rank
+    std::vector<Val> vals;
+    std::vector<int> cur(PCCL_HIP_MAX_VRANKS);
+    for (int r = 0; r < PCCL_HIP_MAX_VRANKS; ++r) { Val v; v.leaf = r; vals.push_back(v); cur[r] = r; }
+    std::vector<int> final_of(PCCL_HIP_MAX_VRANKS, -1);
+    int acc = -1;
+    for (int k = 0; k < seg.prog_len; ++k) {
+        const ColInstr& in = P.col_instrs[seg.prog_start + k];
+        const int a = in.a_src == SRC_ACC ? acc : cur[in.peer];
+        int res = a;
+        if (in.b_src != SRC_NONE) {
+            const int b = in.b_src == SRC_ACC ? acc : cur[in.self];
+            if (a < 0 || b < 0) return false;
+            Val v; v.a = a; v.b = b; v.redop = in.redop;
+            vals.push_back(v);
+            res = (int)vals.size() - 1;
+        }
+        if (res < 0) continue;   // padding in front of any value (never produced by the planner)
+        acc = res;
+        const int kind = in.store & STORE_KIND;
+        if (kind) cur[in.self] = res;
+        if (kind == 2 || (kind == 1 && (in.store & STORE_LAST))) final_of[in.self] = res;
+    }
+    for (uint64_t m = seg.bcast_mask; m; m &= m - 1) final_of[__builtin_ctzll(m)] = acc;
+    int root = -1;
+    uint64_t mask = 0;
+    for (int r = 0; r < PCCL_HIP_MAX_VRANKS; ++r) {
+        if (final_of[r] < 0) continue;
+        if (root >= 0 && final_of[r] != root) return false;     // different values in different ranks
+        root = final_of[r];
+        mask |= 1ull << r;
+    }
+    if (root < 0) return false;
+    // flatten the root: leaves in chain order, one operator throughout
+    int redop = -1;
+    bool literal = true;          // every combination takes at least one leaf
+    std::vector<uint8_t> leaves;
+    std::vector<int> stack = {root};
+    // literal chains are walked from the root down: the leaf of each combination is met before the
+    // rest of the chain, so the list comes out last-combined first and is reversed at the end
+    while (!stack.empty()) {
+        const int id = stack.back(); stack.pop_back();
+        const Val& v = vals[id];
+        if (v.leaf >= 0) { leaves.push_back((uint8_t)v.leaf); continue; }
+        if (redop >= 0 && v.redop != redop) return false;
+        redop = v.redop;
+        const bool la = vals[v.a].leaf >= 0, lb = vals[v.b].leaf >= 0;
+        if (!la && !lb) literal = false;
+        // push the deeper side first so that it is popped last: [leaf now, rest later]
+        if (la) { stack.push_back(v.b); stack.push_back(v.a); }
+        else { stack.push_back(v.a); stack.push_back(v.b); }
+    }
+    std::reverse(leaves.begin(), leaves.end());
+    uint64_t seen = 0;
+    for (uint8_t r : leaves) { if (seen >> r & 1) return false; seen |= 1ull << r; }
+    if (!literal) {
+        const bool free_order = redop == PCCL_MAX || redop == PCCL_MIN || (redop == PCCL_SUM && dtype == PCCL_I32);
+        if (free_order) std::sort(leaves.begin(), leaves.end());
+        else {
+            // the shape matters: accept a perfectly balanced tree, leaves listed left to right
+            struct Walk {
+                const std::vector<Val>& vals;
+                std::vector<uint8_t> out;
+                int depth_of(int id) {          // depth of a perfect subtree, -1 if it is not perfect
+                    const Val& v = vals[id];
+                    if (v.leaf >= 0) { out.push_back((uint8_t)v.leaf); return 0; }
+                    const int da = depth_of(v.a);
+                    if (da < 0) return -1;
+                    const int db = depth_of(v.b);
+                    return db == da ? da + 1 : -1;
+                }
+            } walk{vals, {}};
+            const int depth = walk.depth_of(root);
+            if (depth < 1 || depth > 6) return false;
+            leaves = walk.out;
+            *depth_out = depth;
+        }
+    }
+    *srcs = leaves; *redop_out = redop < 0 ? PCCL_SUM : redop; *mask_out = mask;
+    return true;
+}
+
+// Chain forms of all segments of a plan, or none.
+static void plan_chains(Program& P, const std::vector<ColSegment>& segs, std::vector<ChainSegment>* out) {
+    out->clear();
+    std::vector<ChainSegment> chains;
+    const size_t srcs_before = P.chain_srcs.size();
+    for (const ColSegment& seg : segs) {
+        std::vector<uint8_t> srcs;
+        int redop = PCCL_SUM, depth = 0;
+        uint64_t mask = 0;
+        if (!chain_form(P, seg, P.dtype, &srcs, &redop, &mask, &depth)) { P.chain_srcs.resize(srcs_before); return; }
+        ChainSegment c;
+        c.start = seg.start; c.end = seg.end; c.redop = redop; c.store_mask = mask; c.tree_depth = depth;
+        c.src_start = (int32_t)P.chain_srcs.size(); c.n_src = (int32_t)srcs.size();
+        P.chain_srcs.insert(P.chain_srcs.end(), srcs.begin(), srcs.end());
+        chains.push_back(c);
+    }
+    *out = std::move(chains);
+}
+
 // The linker: R per-rank graphs in, one Program out.  Each step is a method; they run in the order
 // `run` calls them and hand their results on through the members.
 namespace {
@@ -594,6 +708,7 @@ class Linker {
             }
             for (auto& seg : P.segs)
                 count_column_traffic(P, seg, es, &P.column_load_bytes, &P.column_store_bytes, &P.slot_load_bytes, &P.slot_store_bytes);
+            plan_chains(P, P.segs, &P.chain_segs);
         }
     }
 
@@ -684,6 +799,7 @@ class Linker {
             if (!valid) P.direct_segs.clear();
             for (auto& seg : P.direct_segs)
                 count_column_traffic(P, seg, es, &P.direct_load_bytes, &P.direct_store_bytes, &P.direct_slot_load_bytes, &P.direct_slot_store_bytes);
+            plan_chains(P, P.direct_segs, &P.direct_chain_segs);
         }
     }
 };

@@ -55,6 +55,21 @@ struct ColSegment {
                                            // last instruction (the tail of copies of one value)
 };
 
+// A segment whose column program is one chain: one accumulator takes the original values of the
+// ranks in `srcs` one after another (acc = x[src 0]; acc = x[src k] (op) acc), and the final value
+// is the only thing stored, to every rank of `store_mask`.  What the phased runner executes.
+// Or, tree_depth = D > 0: the value is a perfectly balanced binary tree over 2^D ranks - srcs lists
+// them leaf by leaf, left to right; leaves 2i and 2i + 1 are combined first, then those results in
+// pairs, and so on (halving-doubling and binary-tree schedules under an operator whose rounding makes
+// the shape matter).
+struct ChainSegment {
+    int64_t start = 0, end = 0;          // element positions [start, end)
+    int32_t src_start = 0, n_src = 0;    // ranks in Program::chain_srcs, in the order they are combined
+    int32_t redop = PCCL_SUM;
+    int32_t tree_depth = 0;
+    uint64_t store_mask = 0;
+};
+
 struct StepOpPlan {
     int first_item = 0, ntiles = 0, dep_start = 0, ndeps = 0;
     int lead = 0;   // elements between the item grid's anchor and the op's first element (< tile_elems)
@@ -86,6 +101,11 @@ struct Program {
     int64_t direct_load_bytes = 0, direct_store_bytes = 0;
     int64_t direct_slot_load_bytes = 0, direct_slot_store_bytes = 0;
     std::vector<int64_t> direct_in_start, direct_in_end, direct_out_start, direct_out_end;  // windows per rank
+
+    // chain form of the two column plans: one entry per segment, or empty when some segment is not a
+    // chain (values read back, results stored along the way, different values left in different ranks)
+    std::vector<ChainSegment> chain_segs, direct_chain_segs;
+    std::vector<uint8_t> chain_srcs;
 
     // gather plan of an alltoall graph (valid when non-empty): the staged call as direct copies from
     // the callers' input tensors to their output tensors, element units

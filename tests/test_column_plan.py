@@ -175,3 +175,33 @@ def test_random_aligned_programs(seed, slots_mode):
     run_plan(prog.column_plan(), bufs, bufs, slots_mode)
     for r in range(world):
         assert np.array_equal(bufs[r], want[r]), f"rank {r}"
+
+
+# ---------------------------------------------------------------------------------------------
+# Chain form of the plans (what the phased runner executes)
+
+def _info(alg, method, world, n, dtype, channels=1, **ext):
+    graphs = [HostGraph.from_json(j) for j in graph_jsons(alg, method, world, n, dtype, "sm", channels, **ext)]
+    return HostProgram(graphs).info()
+
+
+def test_which_plans_are_chains():
+    """A plan is a chain plan when every segment leaves one value - every contributing rank combined
+    once - in all the ranks it writes: ring allreduces literally; trees and halving-doubling when the
+    operator may be re-associated for the element type (integer sums, maxima, minima), else as
+    balanced trees; a staged reduce_scatter but not the in-place one, which leaves its partial sums
+    in the other ranks."""
+    ring = _info("ring", "build_allreduce", 8, 1 << 16, "bfloat16", 4)
+    assert ring["chain_segments"] == ring["num_segments"] == 32 and ring["staged_chain_segments"] == 32
+    rs = _info("ring", "build_reduce_scatter", 8, 1 << 16, "float16")
+    assert rs["chain_segments"] == 0 and rs["staged_chain_segments"] == 8
+    ag = _info("ring", "build_allgather", 8, 1 << 16, "float16")
+    assert ag["chain_segments"] == 8 and ag["staged_chain_segments"] == 8
+    for dtype, op in (("int32", "sum"), ("float32", "max"), ("bfloat16", "min"), ("float32", "sum"), ("float16", "sum")):
+        tree = _info("tree", "build_allreduce", 32, 1 << 12, dtype, reduce_op=op)
+        assert tree["chain_segments"] == tree["num_segments"] == 1, (dtype, op)
+    rhd = _info("rhd", "build_allreduce", 16, 1 << 16, "float32", 2)
+    assert rhd["chain_segments"] == rhd["num_segments"]
+    # a reduce-only ring (no allgather phase) leaves a different value in every rank
+    with_partials = random_program(77, 4, 5000, 30, "int32", True)
+    assert HostProgram([HostGraph.from_json(j) for j in with_partials]).info()["chain_segments"] == 0

@@ -1,0 +1,193 @@
+"""The phased runner: chain plans (one accumulator per position, the result to a set of ranks) and
+balanced trees on a persistent grid whose workgroups read together, meet, write together, meet.
+Everything is compared with the CPU oracle bit for bit through the engine's C-ABI calls; the
+meetings order nothing, so results must also be exact when they time out or are switched off."""
+import pytest
+import torch
+
+from helpers import bits_equal, graph_jsons, mismatch_report, oracle_buffers, random_program, seeded_inputs
+
+pytestmark = pytest.mark.gpu
+
+CHUNK_VECS = 8192      # 16-byte vectors of every rank one workgroup takes per sweep (chain shapes)
+
+
+def _register(eng, name, jsons):
+    for r, j in enumerate(jsons):
+        eng.register_operation_json(name, j, r)
+
+
+def _check(got, want, what):
+    for r, (g, w) in enumerate(zip(got, want)):
+        assert bits_equal(g, w), f"{what}, rank {r}: {mismatch_report(g, w)}"
+
+
+CASES = [
+    # alg, method, world, elements, dtype, channels, extra, input kind, chain?, tree?
+    ("ring", "build_allreduce", 8, 8 * 3 * 65536 + 8 * 24, "bfloat16", 4, {}, "randn", True, False),
+    ("ring", "build_allreduce", 3, 3 * 100003, "float32", 1, {}, "randn", True, False),
+    ("ring", "build_allreduce", 16, 16 * 40000, "float16", 2, {}, "randn", True, False),
+    ("ring", "build_allreduce", 5, 5 * 77777, "float8_e4m3", 1, {}, "randn", True, False),
+    ("tree", "build_allreduce", 32, 300007, "int32", 1, {"reduce_op": "sum"}, "randint", True, False),
+    ("tree", "build_allreduce", 16, 250001, "float32", 1, {"reduce_op": "max"}, "randn", True, False),
+    ("tree", "build_allreduce", 8, 131072 + 5, "bfloat16", 1, {"reduce_op": "min"}, "randn", True, False),
+    ("rhd", "build_allreduce", 16, 16 * 50000, "int32", 1, {}, "randint", True, False),
+    ("rhd", "build_allreduce", 16, 16 * 40960, "float32", 2, {}, "uniform", True, True),
+    ("rhd", "build_allreduce", 8, 8 * 30000, "bfloat16", 1, {}, "randn", True, True),
+    ("tree", "build_allreduce", 32, 200003, "float32", 1, {"reduce_op": "sum"}, "randn", True, True),
+    ("tree", "build_allreduce", 64, 70001, "float16", 1, {"reduce_op": "sum"}, "randn0.1", True, True),
+    ("tree", "build_allreduce", 2, 90001, "float32", 1, {"reduce_op": "sum"}, "randn", True, False),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: f"{c[0]}-R{c[2]}-{c[4]}-{c[6].get('reduce_op', 'sum')}")
+def test_chain_and_tree_plans_in_place_and_staged(engine_factory, case):
+    alg, method, world, n, dtype, channels, ext, kind, chain, tree = case
+    jsons = graph_jsons(alg, method, world, n, dtype, "sm", channels, **ext)
+    x = seeded_inputs(kind, world, n, dtype, seed=world + n % 97)
+    want = oracle_buffers(jsons, x, dtype)
+    eng = engine_factory(world)
+    name = f"ph_{alg}_{world}_{dtype}_{ext.get('reduce_op', '')}"
+    _register(eng, name, jsons)
+    info = eng.op_info(name)
+    assert (info["chain_segments"] == info["num_segments"]) == chain
+    assert info["staged_chain_segments"] == info["chain_segments"]
+    eng.set_option("phased", 1)
+    try:
+        # grids: one workgroup per CU; 5 workgroups (not a multiple of the XCD count, many sweeps and
+        # meetings); meetings off; a wait that gives up at once
+        for blocks, barriers, timeout in ((0, 1, 1000), (5, 1, 1000), (8, 0, 1000), (16, 1, 0)):
+            for shape in ((-1,) if tree else (0, 1)):
+                what = f"blocks={blocks} barriers={barriers} timeout={timeout} shape={shape}"
+                print(f"{name}: {what}", flush=True)
+                eng.set_option("num_blocks", blocks); eng.set_option("phased_barriers", barriers)
+                eng.set_option("phased_timeout_us", timeout); eng.set_option("phased_shape", shape)
+                bufs = [t.cuda() for t in x]
+                eng.execute_inplace(name, bufs, sync=True)
+                _check(bufs, want, f"in place, {what}")
+                outs = eng.execute_operation(name, [t.cuda() for t in x])
+                _check(outs, want, f"staged, {what}")
+    finally:
+        for key, val in (("phased", -1), ("num_blocks", 0), ("phased_barriers", 1), ("phased_timeout_us", 1000), ("phased_shape", -1)):
+            eng.set_option(key, val)
+
+
+@pytest.mark.parametrize("method", ["build_reduce_scatter", "build_allgather"])
+def test_staged_reduce_scatter_and_allgather(engine_factory, method):
+    """The staged plans of a ring reduce_scatter (eight ranks read, one written per chunk) and of an
+    allgather (one read, eight written) are chains; in place a reduce_scatter leaves its partial sums
+    in the other ranks and is not."""
+    world, n = 8, 8 * (3 * CHUNK_VECS * 8 + 1000)     # fp16: 8 elements per vector; chunks cut by the chunk ends
+    jsons = graph_jsons("ring", method, world, n, "float16", "sm", 1)
+    chunk = n // world
+    in_elems = n if method == "build_reduce_scatter" else chunk
+    x = seeded_inputs("randn0.1", world, in_elems, "float16", seed=7)
+    eng = engine_factory(world)
+    name = "ph_" + method
+    _register(eng, name, jsons)
+    info = eng.op_info(name)
+    assert info["staged_chain_segments"] == world
+    assert info["chain_segments"] == (0 if method == "build_reduce_scatter" else world)
+    # the staged call on the oracle: inputs placed in the rank buffers, the program, the output windows
+    if method == "build_reduce_scatter":
+        full = oracle_buffers(jsons, x, "float16")
+        want = [full[r][r * chunk:(r + 1) * chunk] for r in range(world)]
+    else:
+        want = oracle_buffers(jsons, x, "float16", buffer_elems=n, place=lambda r: r * chunk)
+        whole = torch.cat(x)
+        for w in want:
+            assert bits_equal(w, whole)
+    eng.set_option("phased", 1)
+    try:
+        for blocks in (0, 7):
+            eng.set_option("num_blocks", blocks)
+            out_elems = chunk if method == "build_reduce_scatter" else n
+            outs = [torch.empty(out_elems, dtype=torch.float16, device="cuda") for _ in range(world)]
+            eng.execute_operation(name, [t.cuda() for t in x], outs)
+            _check(outs, want, f"{method} blocks={blocks}")
+    finally:
+        eng.set_option("phased", -1); eng.set_option("num_blocks", 0)
+
+
+def test_automatic_choice_and_what_is_not_a_chain(engine_factory):
+    """Large chain plans go to the phased runner by themselves; a program that leaves different values
+    in different ranks, or stores along the way, is not a chain plan and keeps running on the slot
+    runner whatever the option says."""
+    world = 8
+    n = 4 * 256 * CHUNK_VECS * 8                         # bf16: 4 chunks per CU on a 256-CU GPU
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2)
+    eng = engine_factory(world)
+    _register(eng, "ph_auto", jsons)
+    x = seeded_inputs("randn", world, n, "bfloat16", seed=3)
+    want = oracle_buffers(jsons, x, "bfloat16")
+    bufs = [t.cuda() for t in x]
+    eng.execute_inplace("ph_auto", bufs, sync=True)
+    _check(bufs, want, "automatic")
+    rnd = random_program(4242, 4, 50000, 40, "float32", True)
+    _register(eng4 := engine_factory(4), "ph_rnd", rnd)
+    assert eng4.op_info("ph_rnd")["chain_segments"] == 0
+    xr = seeded_inputs("randn", 4, 50000, "float32", seed=5)
+    wr = oracle_buffers(rnd, xr, "float32")
+    eng4.set_option("phased", 1)
+    try:
+        b = [t.cuda() for t in xr]
+        eng4.execute_inplace("ph_rnd", b, sync=True)
+        _check(b, wr, "not a chain plan")
+    finally:
+        eng4.set_option("phased", -1)
+
+
+def test_more_workgroups_than_fit_at_once(engine_factory):
+    """With more workgroups than the GPU holds at once a meeting cannot complete: the waits run out,
+    the launch goes on unsynchronised and finishes with exact results, and the next launch meets
+    normally again (the last workgroup to leave clears the meeting block)."""
+    world, n = 8, 1200 * CHUNK_VECS * 8              # bf16: 1200 chunks of every rank
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 1)
+    x = seeded_inputs("randn", world, n, "bfloat16", seed=9)
+    want = oracle_buffers(jsons, x, "bfloat16")
+    eng = engine_factory(world)
+    _register(eng, "ph_many", jsons)
+    eng.set_option("phased", 1)
+    try:
+        for blocks, timeout in ((1100, 50), (0, 1000), (1100, 0), (0, 1000)):
+            eng.set_option("num_blocks", blocks); eng.set_option("phased_timeout_us", timeout)
+            bufs = [t.cuda() for t in x]
+            eng.execute_inplace("ph_many", bufs, sync=True)
+            _check(bufs, want, f"blocks={blocks} timeout={timeout}")
+    finally:
+        eng.set_option("phased", -1); eng.set_option("num_blocks", 0); eng.set_option("phased_timeout_us", 1000)
+
+
+def test_phased_launches_recorded_into_a_graph(engine_factory):
+    """A phased launch is one kernel and needs no set-up per launch (the meeting block cleans itself),
+    so it can be recorded and replayed; every replay against the oracle, eager work in between."""
+    world, n = 8, 16 * CHUNK_VECS * 8                  # 16 chunks
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2)
+    x = seeded_inputs("randn", world, n, "bfloat16", seed=13)
+    want = oracle_buffers(jsons, x, "bfloat16")
+    eng = engine_factory(world)
+    _register(eng, "ph_graph", jsons)
+    eng.set_option("phased", 1)
+    try:
+        src = [t.cuda() for t in x]
+        bufs = [t.clone() for t in src]
+        eng.execute_inplace("ph_graph", bufs, sync=True)
+        _check(bufs, want, "eager")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for b, t in zip(bufs, src):
+                    b.copy_(t)
+                eng.execute_inplace("ph_graph", bufs)
+        torch.cuda.current_stream().wait_stream(side)
+        for rep in range(4):
+            for b in bufs:
+                b.fill_(float(rep))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            _check(bufs, want, f"replay {rep}")
+    finally:
+        eng.set_option("phased", -1)
