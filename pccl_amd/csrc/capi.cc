@@ -558,16 +558,16 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
         e.host.segs = device_segments(P.segs, &e.total_tiles, &e.seg_tiles);
         if (!P.direct_segs.empty()) e.host.direct_segs = device_segments(P.direct_segs, &e.direct_tiles, &e.direct_seg_tiles);
         // chain plans for the phased runner (both of its workgroup shapes take chunks of the same size)
-        static_assert(phased_chunk_vecs(0) == phased_chunk_vecs(1), "one chunk table serves both chain shapes");
+        static_assert(phased_chunk_vecs(0) == phased_chunk_vecs(1) && phased_chunk_vecs(0) == phased_chunk_vecs(2), "one chunk table serves all shapes");
         auto chain_segments = [&](const std::vector<ChainSegment>& segs, int64_t* total, int* uniform, int* tree_shape) {
             std::vector<DevChainSegment> ds(segs.size());
             int64_t chunks = 0;
             int depth = 0;
             for (const ChainSegment& c : segs) depth = std::max(depth, c.tree_depth);
-            // a plan with balanced trees runs on a shape that keeps their partial results in registers:
-            // 16 vectors per thread for f32 trees of up to 16 ranks, 8 for deeper trees and for the
-            // element types whose arithmetic needs registers of its own
-            *tree_shape = depth == 0 ? 0 : depth <= 4 ? 2 : 3;
+            // a plan with balanced trees runs on the shape that has the code for them (not built for the
+            // 8-bit floats, whose arithmetic leaves no registers for it: those stay with the slot runner)
+            *tree_shape = depth == 0 ? 0 : 2;
+            if (depth > 0 && (P.dtype == PCCL_F8E4M3 || P.dtype == PCCL_F8E5M2)) { *total = 0; *uniform = 0; return std::vector<DevChainSegment>(); }
             const int64_t chunk_v = phased_chunk_vecs(*tree_shape);
             for (size_t i = 0; i < segs.size(); ++i) {
                 const ChainSegment& c = segs[i];
@@ -762,9 +762,6 @@ bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
     const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
     if (2 * loads < stores) return false;
-    // plans with balanced trees: the shapes that hold their partial results are slower than the slot
-    // runner so far (16 ranks x 64 MiB f32 halving-doubling 0.43 against 0.37 ms): only on request
-    if ((direct ? e.direct_chain_tree : e.chain_tree) != 0) return false;
     return chunks >= 2 * (int64_t)device_cu_count(ctx->device);
 }
 

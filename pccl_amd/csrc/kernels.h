@@ -109,15 +109,14 @@ struct PhasedLaunch {
     int32_t seg_chunks;       // > 0: every segment has this many chunks; 0: search
     int32_t dtype;
     int32_t shape;            // 0: 512 threads x 16 vectors, 1: 256 threads x 32 vectors (each wave a contiguous 32 KiB),
-                              // 2: 1024 threads x 4 vectors, also runs balanced trees of up to 16 ranks,
-                              // 3: 512 threads x 4 vectors, also runs balanced trees of up to 64 ranks
+                              // 2: 256 x 32 with the code for balanced trees as well
     int32_t num_blocks;       // 0: one workgroup per CU
     int32_t barriers;         // 1: all workgroups read together, then write together; 0: no meeting
     PhaseSync* sync;
     uint64_t timeout_ticks;   // 100 MHz ticks a workgroup waits at a meeting point before it goes on alone
 };
 // Vectors of every rank one workgroup of the given shape takes per sweep.
-PCCL_HD constexpr int64_t phased_chunk_vecs(int shape) { return shape == 2 ? 1024 * 4 : shape == 3 ? 512 * 4 : 8192; }
+PCCL_HD constexpr int64_t phased_chunk_vecs(int shape) { (void)shape; return 8192; }
 
 struct StepwiseLaunch {
     const DevStepOp* ops;

@@ -10,6 +10,7 @@
 
 #include <atomic>
 #include <cstring>
+#include <utility>
 
 #include "kernels.h"
 
@@ -179,45 +180,37 @@ __device__ __forceinline__ u32x4 vec_fast(u32x4 a, u32x4 b) {
         }
         return r;
     } else if constexpr (DT == PCCL_BF16) {
-        u32x4 r;
+        // word by word, no arrays: everything stays in registers whatever the surrounding code looks like
         uint64_t nan = 0;
-        const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
-        uint32_t rw[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float lo = f32_comb<OP>(as_f32(aw[i] << 16), as_f32(bw[i] << 16));
-            const float hi = f32_comb<OP>(as_f32(aw[i] & 0xFFFF0000u), as_f32(bw[i] & 0xFFFF0000u));
+        auto word = [&](uint32_t x, uint32_t y) {
+            const float lo = f32_comb<OP>(as_f32(x << 16), as_f32(y << 16));
+            const float hi = f32_comb<OP>(as_f32(x & 0xFFFF0000u), as_f32(y & 0xFFFF0000u));
             nan |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(lo, hi));
             const f32x2 pair = {lo, hi};
-            rw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
-        }
-        if (__builtin_expect(nan != 0, 0)) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if ((rw[i] & 0x7FFFu) > 0x7F80u) rw[i] = (rw[i] & 0xFFFF0000u) | 0x7FFFu;
-                if ((rw[i] & 0x7FFF0000u) > 0x7F800000u) rw[i] = (rw[i] & 0x0000FFFFu) | 0x7FFF0000u;
-            }
-        }
-        r.x = rw[0]; r.y = rw[1]; r.z = rw[2]; r.w = rw[3];
+            return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
+        };
+        auto repair = [](uint32_t w) {
+            if ((w & 0x7FFFu) > 0x7F80u) w = (w & 0xFFFF0000u) | 0x7FFFu;
+            if ((w & 0x7FFF0000u) > 0x7F800000u) w = (w & 0x0000FFFFu) | 0x7FFF0000u;
+            return w;
+        };
+        u32x4 r = {word(a.x, b.x), word(a.y, b.y), word(a.z, b.z), word(a.w, b.w)};
+        if (__builtin_expect(nan != 0, 0)) { r.x = repair(r.x); r.y = repair(r.y); r.z = repair(r.z); r.w = repair(r.w); }
         return r;
     } else if constexpr (DT == PCCL_F16) {
-        const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
-        uint32_t rw[4];
         uint64_t nan = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const h2 s = f16x2_comb<OP>(__builtin_bit_cast(h2, aw[i]), __builtin_bit_cast(h2, bw[i]));
+        auto word = [&](uint32_t x, uint32_t y) {
+            const h2 s = f16x2_comb<OP>(__builtin_bit_cast(h2, x), __builtin_bit_cast(h2, y));
             nan |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(s[0], s[1]));
-            rw[i] = __builtin_bit_cast(uint32_t, s);
-        }
-        if (__builtin_expect(nan != 0, 0)) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if ((rw[i] & 0x7FFFu) > 0x7C00u) rw[i] = (rw[i] & 0xFFFF0000u) | 0x7FFFu;
-                if ((rw[i] & 0x7FFF0000u) > 0x7C000000u) rw[i] = (rw[i] & 0x0000FFFFu) | 0x7FFF0000u;
-            }
-        }
-        u32x4 r = {rw[0], rw[1], rw[2], rw[3]};
+            return __builtin_bit_cast(uint32_t, s);
+        };
+        auto repair = [](uint32_t w) {
+            if ((w & 0x7FFFu) > 0x7C00u) w = (w & 0xFFFF0000u) | 0x7FFFu;
+            if ((w & 0x7FFF0000u) > 0x7C000000u) w = (w & 0x0000FFFFu) | 0x7FFF0000u;
+            return w;
+        };
+        u32x4 r = {word(a.x, b.x), word(a.y, b.y), word(a.z, b.z), word(a.w, b.w)};
+        if (__builtin_expect(nan != 0, 0)) { r.x = repair(r.x); r.y = repair(r.y); r.z = repair(r.z); r.w = repair(r.w); }
         return r;
     } else {
         return vec_op_words<DT>(a, b, OP);
@@ -1163,19 +1156,10 @@ __device__ __forceinline__ bool phase_wait(PhaseSync* s, int gen, uint64_t timeo
 // (S divides V, so the slot of vector v is v % S whatever the rank) and combined into acc[].
 // Fetch q = k V + v is issued when fetch q - S has been consumed; loads complete in order, so
 // "at most S - 1 outstanding" means fetch q has landed.
-template <int DT, int OP, int T, int V, int S, int VS, int GR, int TREE>
-__device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int32_t* srcs, int n, int tree_depth, const RankPtrs& ptrs,
+template <int DT, int OP, int T, int V, int S, int VS, int GR>
+__device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int32_t* srcs, int n, const RankPtrs& ptrs,
                                            u32x4* lds, int64_t chunk_byte0, uint32_t toff, int tid) {
     static_assert(V % S == 0 && S <= V && S % GR == 0, "the slot of a vector must not depend on the rank; groups of GR vectors per wait");
-    // trees only arise under an operator whose result depends on the order: sums (maxima, minima and
-    // integer sums are re-associated into chains by the planner)
-    constexpr bool kTrees = TREE > 0 && OP == PCCL_SUM && DT != PCCL_I32;
-    constexpr int kMaxDepth = kTrees ? TREE : 1;
-    // kTrees: the left siblings that wait for their right halves, one per level (a binary counter over
-    // the leaf number: leaf k is combined upwards through every level whose bit is set in k and parked
-    // at the first level whose bit is clear).  All register indices are compile-time; the branches
-    // are uniform.
-    u32x4 parked[kMaxDepth][V];
     u32x4* const my = lds + (tid & ~63);
     const u32x4* const mine = lds + tid;
     const char* cur = ptrs.p[kMaxR + srcs[0]] + chunk_byte0;
@@ -1192,25 +1176,8 @@ __device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int
             u32x4 x[GR];
 #pragma unroll
             for (int g = 0; g < GR; ++g) x[g] = mine[((v + g) % S) * T];
-            if (!kTrees || tree_depth == 0) {
 #pragma unroll
-                for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_fast<DT, OP>(x[g], acc[v + g]);
-            } else {
-                // levels this leaf climbs: the trailing one bits of its number (uniform)
-                int climb = __builtin_ctz(~(unsigned)k);
-                if (climb > tree_depth) climb = tree_depth;
-#pragma unroll
-                for (int g = 0; g < GR; ++g) {
-                    u32x4 y = x[g];
-#pragma unroll
-                    for (int lvl = 0; lvl < kMaxDepth; ++lvl)
-                        if (lvl < climb) y = vec_fast<DT, OP>(parked[lvl][v + g], y);
-#pragma unroll
-                    for (int lvl = 0; lvl < kMaxDepth; ++lvl)
-                        if (lvl == climb && lvl < tree_depth) parked[lvl][v + g] = y;
-                    if (climb == tree_depth) acc[v + g] = y;      // the last leaf: the root
-                }
-            }
+            for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_fast<DT, OP>(x[g], acc[v + g]);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
 #pragma unroll
             for (int g = 0; g < GR; ++g) {
@@ -1223,11 +1190,79 @@ __device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int
     }
 }
 
-template <int DT, int T, int V, int S, bool WAVEC, int GR, int TREE>
+template <int V, class F, int... Vs>
+__device__ __forceinline__ void fill_by_index(u32x4 (&out)[V], F&& f, std::integer_sequence<int, Vs...>) {
+    ((out[Vs] = f(Vs)), ...);
+}
+
+// Read phase of one chunk whose value is a perfectly balanced tree over n = 2^depth ranks, depth >= 2:
+// vector by vector, all n leaves of a vector before the next vector, four leaves at a time - a quad
+// ((l0 + l1) + (l2 + l3)) is combined at once, and the quads' results climb the remaining levels like
+// a binary counter over the quad number: quad j is combined with the parked left siblings of every
+// level whose bit is set in j and is parked at the first level whose bit is clear.  The waiting left
+// siblings are thus `depth - 2` vectors per thread whatever V is.  Fetch q = v n + k goes to slot
+// q % S.  The leaves' base addresses sit in the lanes of one register pair (lane i: leaf i) and are
+// picked with v_readlane: no memory access stands between two fetches.
+template <int DT, int T, int V, int S, int VS>
+__device__ __forceinline__ void tree_read(u32x4 (&acc)[V], const PCCL_CONST int32_t* srcs, int n, int depth, const RankPtrs& ptrs,
+                                          u32x4* lds, int64_t chunk_byte0, uint32_t toff, int tid) {
+    static_assert(S % 4 == 0 && S >= 8, "a quad is consumed while the next one is in flight");
+    constexpr int kMaxUpper = 4;                 // levels above the quads: trees of up to 64 ranks
+    u32x4* const my = lds + (tid & ~63);
+    const u32x4* const mine = lds + tid;
+    uint32_t lp_lo = 0, lp_hi = 0;
+    for (int i = 0; i < n; ++i) {
+        const uint64_t p = (uint64_t)(ptrs.p[kMaxR + srcs[i]] + chunk_byte0);
+        if ((tid & 63) == i) { lp_lo = (uint32_t)p; lp_hi = (uint32_t)(p >> 32); }
+    }
+    auto leaf_base = [&](int k) {
+        // (the builtin returns a signed int: without the casts a low word with its top bit set would
+        // smear ones over the high word)
+        const uint64_t p = (uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)lp_lo, k) |
+                           ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)lp_hi, k) << 32);
+        return (const char*)p;
+    };
+    const int total = V * n;                     // fetches of this chunk; total >= S because n >= 4 and V >= 2
+    auto fetch = [&](int q) {                    // q uniform: leaf q % n of vector q / n into slot q % S
+        load_lds_nt(leaf_base(q & (n - 1)), toff + (uint32_t)(q >> depth) * VS, my + (q & (S - 1)) * T);
+    };
+    for (int q = 0; q < S; ++q) fetch(q);
+    const int upper = depth - 2;                 // levels the quads' results still have to climb
+    u32x4 parked[kMaxUpper];
+    // one vector: all its leaves, quad by quad; returns the root
+    auto one_vector = [&](int v) __attribute__((always_inline)) {
+        u32x4 root = u32x4{0, 0, 0, 0};
+        for (int k = 0; k < n; k += 4) {
+            const int q = v * n + k;
+            if (q + S >= total) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(S - 4) : "memory");
+            const u32x4 l0 = mine[(q & (S - 1)) * T], l1 = mine[((q + 1) & (S - 1)) * T];
+            const u32x4 l2 = mine[((q + 2) & (S - 1)) * T], l3 = mine[((q + 3) & (S - 1)) * T];
+            u32x4 y = vec_fast<DT, PCCL_SUM>(vec_fast<DT, PCCL_SUM>(l0, l1), vec_fast<DT, PCCL_SUM>(l2, l3));
+            int climb = __builtin_ctz(~(unsigned)(k >> 2));      // trailing one bits of the quad number (uniform)
+            if (climb > upper) climb = upper;
+#pragma unroll
+            for (int lvl = 0; lvl < kMaxUpper; ++lvl)
+                if (lvl < climb) y = vec_fast<DT, PCCL_SUM>(parked[lvl], y);
+#pragma unroll
+            for (int lvl = 0; lvl < kMaxUpper; ++lvl)
+                if (lvl == climb && lvl < upper) parked[lvl] = y;
+            if (climb == upper) root = y;                        // the last quad carries the root
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
+            if (q + S < total) { fetch(q + S); fetch(q + S + 1); fetch(q + S + 2); fetch(q + S + 3); }
+        }
+        return root;
+    };
+    // a fold over the vector numbers: every index of acc[] is a compile-time constant whatever the
+    // optimiser makes of the loops inside
+    fill_by_index(acc, one_vector, std::make_integer_sequence<int, V>{});
+}
+
+template <int DT, int T, int V, int S, bool WAVEC, int GR, bool TREE>
 __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs) {
     extern __shared__ u32x4 lds[];
     __shared__ int s_flag;
-    static_assert((size_t)S * T * 16 + 64 <= (size_t)kPhasedLdsBytes, "the fetch ring must fit the LDS the launcher asks for");
+    static_assert((size_t)S * T * 16 <= 160u * 1024, "the fetch ring must fit a CU's LDS");
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
     constexpr int64_t CHUNK_V = (int64_t)T * V;
@@ -1268,9 +1303,14 @@ __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs
             whole = vbase * VE >= seg.start && (vbase + CHUNK_V) * VE <= seg.end;
             const PCCL_CONST int32_t* srcs = as_const(L.srcs) + seg.src_start;   // dwords: uniform reads become scalar loads
             if (whole) {
-                if (seg.redop == PCCL_SUM) chain_read<DT, PCCL_SUM, T, V, S, VS, GR, TREE>(acc, srcs, seg.n_src, seg.tree_depth, ptrs, lds, vbase * 16, toff, tid);
-                else if (seg.redop == PCCL_MAX) chain_read<DT, PCCL_MAX, T, V, S, VS, GR, TREE>(acc, srcs, seg.n_src, seg.tree_depth, ptrs, lds, vbase * 16, toff, tid);
-                else chain_read<DT, PCCL_MIN, T, V, S, VS, GR, TREE>(acc, srcs, seg.n_src, seg.tree_depth, ptrs, lds, vbase * 16, toff, tid);
+                bool done = false;
+                if constexpr (TREE) {
+                    if (seg.tree_depth > 1) { tree_read<DT, T, V, S, VS>(acc, srcs, seg.n_src, seg.tree_depth, ptrs, lds, vbase * 16, toff, tid); done = true; }
+                }
+                if (done) {}
+                else if (seg.redop == PCCL_SUM) chain_read<DT, PCCL_SUM, T, V, S, VS, GR>(acc, srcs, seg.n_src, ptrs, lds, vbase * 16, toff, tid);
+                else if (seg.redop == PCCL_MAX) chain_read<DT, PCCL_MAX, T, V, S, VS, GR>(acc, srcs, seg.n_src, ptrs, lds, vbase * 16, toff, tid);
+                else chain_read<DT, PCCL_MIN, T, V, S, VS, GR>(acc, srcs, seg.n_src, ptrs, lds, vbase * 16, toff, tid);
             } else {
                 // a chunk that the segment's ends cut: vector by vector, loads and stores together
                 for (int64_t j = tid; j < CHUNK_V; j += T) {
@@ -1280,7 +1320,7 @@ __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs
                     if (e1 > seg.end) e1 = seg.end;
                     if (e0 >= e1) continue;
                     u32x4 x = ldv(ptrs.p[kMaxR + srcs[0]] + vec * 16);
-                    if (TREE == 0 || seg.tree_depth == 0) {
+                    if (!TREE || seg.tree_depth == 0) {
                         for (int k = 1; k < seg.n_src; ++k) x = vec_op<DT>(ldv(ptrs.p[kMaxR + srcs[k]] + vec * 16), x, seg.redop);
                     } else {
                         u32x4 parked[6];
@@ -1438,28 +1478,34 @@ int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
 }
 
 template <class K>
-static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads, const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
+static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads, int ring_slots, const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
     const int dev = current_device();
+    // the fetch ring, and never less than what keeps a second workgroup off the CU
+    const int lds = std::max(kPhasedLdsBytes, ring_slots * threads * 16);
     if (!allowed[dev].load(std::memory_order_relaxed)) {
-        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kPhasedLdsBytes);
+        hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (rc != hipSuccess) return (int)rc;
         allowed[dev].store(1, std::memory_order_relaxed);
     }
     int64_t grid = L.num_blocks > 0 ? L.num_blocks : current_cus();
     if (grid > L.total_chunks) grid = L.total_chunks;
     if (grid <= 0) return 0;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(threads), (size_t)kPhasedLdsBytes, s, L, ptrs);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(threads), (size_t)lds, s, L, ptrs);
     return (int)hipGetLastError();
 }
 
 template <int DT>
 static int launch_phased_dt(const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
-    static std::atomic<int> allowed[4][kMaxDevices];
+    static std::atomic<int> allowed[3][kMaxDevices];
+    // integer sums never arrive as trees (the planner re-associates them into chains), and the 8-bit
+    // floats' arithmetic leaves no registers for the tree code
+    constexpr bool kNoTrees = DT == PCCL_I32 || DT == PCCL_F8E4M3 || DT == PCCL_F8E5M2;
     switch (L.shape) {
-        case 0: return launch_phased_kernel(phased_kernel<DT, 512, 16, 4, false, 2, 0>, allowed[0], 512, L, ptrs, s);
-        case 1: return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, true, 2, 0>, allowed[1], 256, L, ptrs, s);
-        case 2: return launch_phased_kernel(phased_kernel<DT, 1024, 4, 4, false, 2, 4>, allowed[2], 1024, L, ptrs, s);
-        case 3: return launch_phased_kernel(phased_kernel<DT, 512, 4, 4, false, 2, 6>, allowed[3], 512, L, ptrs, s);
+        case 0: return launch_phased_kernel(phased_kernel<DT, 512, 16, 4, false, 2, false>, allowed[0], 512, 4, L, ptrs, s);
+        case 1: return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, true, 2, false>, allowed[1], 256, 8, L, ptrs, s);
+        case 2:
+            if constexpr (kNoTrees) return (int)hipErrorInvalidValue;
+            else return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, true, 2, true>, allowed[2], 256, 8, L, ptrs, s);
         default: return (int)hipErrorInvalidValue;
     }
 }
