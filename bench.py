@@ -366,7 +366,8 @@ def run_inplace(args, wl: Workload, dev) -> int:
         eng.set_option(key, val)
     info = eng.op_info("bench")
     alg_bytes = info["algorithmic_bytes"]
-    log(f"program: {info}")
+    runner_kernel = eng.get_option("runner_inplace:bench")      # the kernel the library launches for this plan, size and options
+    log(f"program: {info}; runner: {runner_kernel}")
 
     t0 = time.perf_counter()
     pristine = wl.make_inputs()
@@ -446,9 +447,8 @@ def run_inplace(args, wl: Workload, dev) -> int:
         persistent = side_leg(eng, "bench", bufs, "persistent", reps, alg_bytes)
         persistent["note"] += "; one launch for the whole graph, ordering by device-side flags (one per work item, one ready word per op)"
 
-    default_runner = not any(kv.split("=")[0].startswith(("lds_slots", "slot_")) for kv in args.option)
-    column = args.mode in ("auto", "column") and info["position_aligned"]
-    kernel = "column_slot_kernel" if column else "level_kernel" if args.mode == "stepwise" else "persistent_kernel"
+    default_runner = not any(kv.split("=")[0].startswith(("lds_slots", "slot_", "phased")) for kv in args.option)
+    kernel = runner_kernel
     traffic, traffic_source = committed_traffic(kernel, wl.traffic_stem) if default_runner else (None, None)
     if traffic is not None and kernel == "level_kernel":
         traffic *= info["num_levels"]      # the profile gives one launch; an execution is one launch per level
@@ -521,8 +521,9 @@ def brief_inplace(args, wl: Workload, dev) -> dict:
         avg_ms = sum(kern_ms) / len(kern_ms)
         hbm_bytes, note = moved_bytes(info, "auto")
         rate = hbm_bytes / (avg_ms * 1e-3) / 1e9
-        traffic, source = committed_traffic("column_slot_kernel", wl.traffic_stem)
-        out = {"workload": wl.name, "verified": bool(ok), "verify": verify, "ms_per_step": round(ms_per_step, 4),
+        kernel = eng.get_option("runner_inplace:bench")
+        traffic, source = committed_traffic(kernel, wl.traffic_stem)
+        out = {"workload": wl.name, "kernel": kernel, "verified": bool(ok), "verify": verify, "ms_per_step": round(ms_per_step, 4),
                "kernel_ms_avg": round(avg_ms, 4), "kernel_ms_min": round(min(kern_ms), 4),
                "hbm_bytes_per_step": hbm_bytes, "algorithmic_bytes_per_step": info["algorithmic_bytes"],
                "GB/s": round(rate, 1), "frac": round(rate / PEAK_GBPS, 4), "bytes_counted": note,
@@ -582,7 +583,7 @@ def brief_c4(args, dev, nbytes: int) -> list:
             hbm, note = moved_bytes(info, "auto", staged=True)
             rate = hbm / (avg * 1e-3) / 1e9
             kind = method[6:]
-            row = {"workload": f"ring_{kind}_R8_f16_{nbytes}B_per_rank_staged_call", "verified": bool(ok),
+            row = {"workload": f"ring_{kind}_R8_f16_{nbytes}B_per_rank_staged_call", "kernel": eng.get_option("runner_staged:bench"), "verified": bool(ok),
                    "verify": {"matches_ring_order_f16" if kind == "reduce_scatter" else "every_output_is_the_concatenation": bool(ok)},
                    "ms_per_step": round(wall_ms, 4), "kernel_ms_avg": round(avg, 4), "kernel_ms_min": round(min(ms), 4),
                    "hbm_bytes_per_step": hbm, "algorithmic_bytes_per_step": info["algorithmic_bytes"],
@@ -654,6 +655,19 @@ def run_c4(args, dev) -> int:
                 for _ in range(args.warmup):
                     call()
                 torch.cuda.synchronize()
+                if args.c4_graph:
+                    # the prepared call recorded once into a graph (one kernel node in column mode) and replayed
+                    side = torch.cuda.Stream()
+                    side.wait_stream(torch.cuda.current_stream())
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.stream(side):
+                        with torch.cuda.graph(graph, stream=side):
+                            call()
+                    torch.cuda.current_stream().wait_stream(side)
+                    call = graph.replay
+                    for _ in range(args.warmup):
+                        call()
+                    torch.cuda.synchronize()
                 ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
                 t0 = time.perf_counter()
                 for a, b in ev:
@@ -674,7 +688,8 @@ def run_c4(args, dev) -> int:
                     "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
                     "config": {"workload": f"ring_{method[6:]}_R8_f16_{nbytes}B_per_rank", "virtual_ranks": world, "bytes_per_rank": nbytes,
                                "channels": 1, "data_ops": info["num_data_ops"], "algorithmic_bytes_per_step": info["algorithmic_bytes"],
-                               "hbm_bytes_per_step": hbm, "mode": args.mode, "in_place": False},
+                               "hbm_bytes_per_step": hbm, "mode": args.mode, "in_place": False, "graph_replay": bool(args.c4_graph)},
+                    "wall_us_per_call": round(wall_ms * 1e3, 2),
                     "latency_us_median": round(ms[len(ms) // 2] * 1e3, 2), "latency_us_min": round(ms[0] * 1e3, 2),
                     **reference_bandwidths(method[6:], nbytes, world, wall_ms),
                     "algorithmic_equiv_GBps": round(info["algorithmic_bytes"] / (wall_ms * 1e-3) / 1e9, 1),
@@ -699,6 +714,7 @@ def main() -> int:
     ap.add_argument("--channels", type=int, default=4, help="c2: channels of the ring")
     ap.add_argument("--c5-dtype", default="int32", choices=["int32", "float32"], help="c5: int32 SUM or float32 MAX")
     ap.add_argument("--c4-bytes", default="", help="c4: comma-separated bytes per rank instead of the full sweep")
+    ap.add_argument("--c4-graph", action="store_true", help="c4: record the prepared call into a HIP graph once and time its replays")
     ap.add_argument("--vecs-per-thread", type=int, default=0)
     ap.add_argument("--num-blocks", type=int, default=-1)
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
@@ -717,7 +733,18 @@ def main() -> int:
     ap.add_argument("--calibrate-copy-bytes", type=int, default=0,
                     help="also launch the library's plain copy kernel on this many bytes (3 times): a "
                          "known-traffic reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--probe", default="", metavar="'RANKS BYTES CASE ...'",
+                    help="run the memory-system probe (pccl_amd/csrc/stream_probe.hip: bare kernels of the runners' traffic "
+                         "shapes) with these arguments instead of a benchmark; prints its JSON lines")
     args = ap.parse_args()
+    if args.probe:
+        # a child process, started before anything here touches the GPU
+        import subprocess
+        from pccl_amd import build as lib_build
+        if not os.path.exists(lib_build.PROBE):
+            print("bench.py: the probe is not built (python pccl_amd/build.py)", file=sys.stderr)
+            return 1
+        return subprocess.run([lib_build.PROBE] + args.probe.split()).returncode
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU: the R ranks are virtual ranks resident in one "
               "MI355X's HBM and no multi-GPU path exists; run with --gpus 1", file=sys.stderr)

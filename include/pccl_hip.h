@@ -263,7 +263,10 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * persistent runners; the marker library is loaded at run time and PCCL_ERR_UNSUPPORTED is returned
  * if there is none; the environment variable PCCL_TRACE_RANGES=1 sets it for new contexts). */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
-/* The current value of an option as text (the keys of pccl_hip_set_option, and "num_vranks"): what the
+/* The current value of an option as text (the keys of pccl_hip_set_option, "num_vranks", and
+ * "runner_inplace:NAME" / "runner_staged:NAME": the kernel an in-place / staged execution of operation
+ * NAME would launch now - "phased_kernel", "column_slot_kernel", "column_kernel", "level_kernel",
+ * "persistent_kernel", "gather_kernel", or "staging + ..." - which links the operation): what the
  * environment switches PCCL_NUM_BLOCKS / PCCL_DISABLE_FUSED / PCCL_TRACE_RANGES left in a new context
  * can be read back here.  No counterpart in the reference. */
 int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t cap);

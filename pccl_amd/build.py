@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "lib")
 OUT = os.path.join(OUT_DIR, "libpccl_hip.so")
 SOURCES = ["graph.cc", "program.cc", "capi.cc", "kernels.hip"]
-HEADERS = ["graph.h", "program.h", "kernels.h", "json_min.h", "../../include/pccl_hip.h"]
+HEADERS = ["graph.h", "program.h", "kernels.h", "json_min.h", "../../include/pccl_hip.h", "stream_probe.hip"]
 
 
 def is_stale() -> bool:
@@ -55,7 +55,22 @@ def build(force: bool = True, verbose: bool = False) -> str:
     if failed:
         raise RuntimeError("hipcc failed")
     subprocess.run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", OUT] + objs, check=True)
+    build_probe(hipcc, common)
     return OUT
+
+
+PROBE = os.path.join(OUT_DIR, "stream_probe")
+
+
+def build_probe(hipcc: str, common) -> str:
+    """The memory-system probe (bare kernels of the runners' traffic shapes; `bench.py --probe`): a
+    standalone program, not part of the library."""
+    cmd = [hipcc] + [c for c in common if c != "-fPIC"] + [os.path.join(CSRC, "stream_probe.hip"), "-o", PROBE]
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    if out.returncode != 0:
+        sys.stderr.write(out.stdout.decode())
+        raise RuntimeError("hipcc failed on stream_probe.hip")
+    return PROBE
 
 
 if __name__ == "__main__":

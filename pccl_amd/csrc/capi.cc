@@ -749,9 +749,10 @@ int launch_levels(pccl_hip_ctx* ctx, OpEntry& e, const StepwiseLaunch& L, const 
 }
 
 // Whether a column-mode execution goes to the phased runner, and its launch.  `direct`: the staged
-// call's plan on the caller's tensors.  The phased runner pays when every CU has several chunks to
-// work through; small tensors stay with the slot runner, whose many small workgroups start and end
-// faster.
+// call's plan on the caller's tensors.  The phased runner pays from about one 128 KiB chunk of every
+// rank per CU on (8-rank bf16 ring allreduce, in place: 16 MiB per rank 54 us on either runner, 32 MiB
+// 88 against 97 us, 128 MiB 0.344 against 0.359 ms); smaller tensors stay with the slot runner, whose
+// many small workgroups start and end faster (4 MiB per rank: 17 against 44 us).
 bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     const int64_t chunks = direct ? e.direct_chain_chunks : e.chain_chunks;
     const DevBuf& segs = direct ? e.direct_chain_segs : e.chain_segs;
@@ -762,7 +763,7 @@ bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
     const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
     if (2 * loads < stores) return false;
-    return chunks >= 2 * (int64_t)device_cu_count(ctx->device);
+    return chunks >= (int64_t)device_cu_count(ctx->device);
 }
 
 int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtrs& ptrs, hipStream_t stream) {
@@ -780,7 +781,11 @@ int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtr
     const int tree_shape = direct ? e.direct_chain_tree : e.chain_tree;
     L.shape = tree_shape ? tree_shape : ctx->phased_shape >= 0 ? ctx->phased_shape : (ctx->R <= 8 ? 0 : 1);
     L.num_blocks = ctx->num_blocks;
-    L.barriers = ctx->phased_barriers ? 1 : 0;
+    // a plan that mostly reads (a reduce_scatter: R chunks in, one out) gains nothing from meeting:
+    // its write phases are too short to matter (8 x 64 MB fp16: 89 us without, 94 us with)
+    const int64_t loads = direct ? P.direct_slot_load_bytes : P.slot_load_bytes;
+    const int64_t stores = direct ? P.direct_slot_store_bytes : P.slot_store_bytes;
+    L.barriers = ctx->phased_barriers && loads < 4 * stores ? 1 : 0;
     L.sync = (PhaseSync*)e.phase_sync.p;
     L.timeout_ticks = (uint64_t)ctx->phased_timeout_us * 100ull;
     return launch_phased(L, ptrs, stream);
@@ -1309,6 +1314,22 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
         else if (k == "slot_lds_kib") v = std::to_string(ctx->slot_lds_kib);
         else if (k == "step_tile_bytes") v = std::to_string(ctx->step_tile_bytes);
         else if (k == "num_vranks") v = std::to_string(ctx->R);
+        else if (k.rfind("runner_inplace:", 0) == 0 || k.rfind("runner_staged:", 0) == 0) {
+            // which kernel an execution of that operation would launch now, given its plan, the tensors'
+            // size and the options (16-byte aligned, non-overlapping tensors assumed)
+            const bool staged = k[7] == 's';
+            OpEntry& e = find_entry(ctx, k.c_str() + (staged ? 14 : 15));
+            HIP_TRY(hipSetDevice(ctx->device));
+            link_entry(ctx, e);
+            const Program& P = e.prog;
+            const bool column_ok = ctx->mode == Mode::Auto || ctx->mode == Mode::Column;
+            if (staged && P.collective_type == "alltoall" && ctx->fuse_staging && e.gather.p && ctx->mode == Mode::Auto) v = "gather_kernel";
+            else if (staged && !(ctx->fuse_staging && column_ok && P.position_aligned && !P.direct_segs.empty()))
+                v = std::string("staging + ") + (ctx->mode == Mode::Persistent ? "persistent_kernel" : (P.position_aligned && column_ok) ? "column" : "level_kernel");
+            else if (!column_ok || !P.position_aligned) v = ctx->mode == Mode::Persistent ? "persistent_kernel" : "level_kernel";
+            else if (wants_phased(ctx, e, staged)) v = "phased_kernel";
+            else v = e.slot_threads > 0 ? "column_slot_kernel" : "column_kernel";
+        }
         else return fail(PCCL_ERR_INVALID, "unknown option '" + k + "'");
         if (v.size() + 1 > cap) return fail(PCCL_ERR_INVALID, "value buffer too small");
         std::memcpy(value, v.c_str(), v.size() + 1);
