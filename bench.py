@@ -289,6 +289,13 @@ def committed_traffic(kernel: str, stem: str | None):
         return None, None
 
 
+def c4_traffic(kernel: str, kind: str, nbytes: int):
+    """Counter-measured traffic of a staged reduce_scatter / allgather call: only the 512 MB size has a profile."""
+    if nbytes != 536870912:
+        return None, None
+    return committed_traffic(kernel, f"ring_{kind}_R8_f16_512MB_staged")
+
+
 def timed_inplace(eng, name, bufs, steps, warmup):
     """K timed executions in place: wall time per step and per-launch HIP-event times."""
     import torch
@@ -462,6 +469,7 @@ def run_inplace(args, wl: Workload, dev) -> int:
                    "hbm_bytes_per_step": hbm_bytes, "mode": args.mode, "in_place": True},
         "pct_of_hbm_peak": round(100 * value / PEAK_GBPS, 1),
         "algorithmic_equiv_GBps": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        **reference_bandwidths("allreduce", wl.n * (2 if wl.dtype in ("bf16", "f16") else 4), wl.world, ms_per_step),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "bytes_counted": hbm_note, "kernel": kernel,
@@ -587,8 +595,8 @@ def brief_c4(args, dev, nbytes: int) -> list:
                    "verify": {"matches_ring_order_f16" if kind == "reduce_scatter" else "every_output_is_the_concatenation": bool(ok)},
                    "ms_per_step": round(wall_ms, 4), "kernel_ms_avg": round(avg, 4), "kernel_ms_min": round(min(ms), 4),
                    "hbm_bytes_per_step": hbm, "algorithmic_bytes_per_step": info["algorithmic_bytes"],
-                   "GB/s": round(rate, 1), "frac": round(rate / PEAK_GBPS, 4), "bytes_counted": note,
-                   "traffic": None, "traffic_source": None}
+                   "GB/s": round(rate, 1), "frac": round(rate / PEAK_GBPS, 4), "bytes_counted": note}
+            row["traffic"], row["traffic_source"] = c4_traffic(row["kernel"], kind, nbytes)
             row.update(reference_bandwidths(kind, nbytes, world, wall_ms))
             out.append(row)
         finally:
@@ -679,6 +687,8 @@ def run_c4(args, dev) -> int:
                 ms = sorted(a.elapsed_time(b) for a, b in ev)
                 avg = sum(ms) / len(ms)
                 hbm, note = moved_bytes(info, args.mode, staged=True)
+                c4_kernel = eng.get_option("runner_staged:bench")
+                c4_tr = c4_traffic(c4_kernel, method[6:], nbytes) if args.mode == "auto" and not args.option else (None, None)
                 if args.mode in ("stepwise", "persistent"):
                     hbm += 2 * 2 * world * (in_elems + out_elems)  # the two batched staging copies: read + write, 2 bytes per element
                     note += " plus the input and output staging copies"
@@ -694,8 +704,8 @@ def run_c4(args, dev) -> int:
                     **reference_bandwidths(method[6:], nbytes, world, wall_ms),
                     "algorithmic_equiv_GBps": round(info["algorithmic_bytes"] / (wall_ms * 1e-3) / 1e9, 1),
                     "roofline": {"bound": "hbm", "achieved": round(hbm / (avg * 1e-3) / 1e9, 1), "peak": PEAK_GBPS, "unit": "GB/s",
-                                 "frac": round(hbm / (avg * 1e-3) / 1e9 / PEAK_GBPS, 4), "traffic": None, "traffic_source": None,
-                                 "bytes_counted": note, "kernel_ms_avg": round(avg, 5)}}), flush=True)
+                                 "frac": round(hbm / (avg * 1e-3) / 1e9 / PEAK_GBPS, 4), **dict(zip(("traffic", "traffic_source"), c4_tr)),
+                                 "kernel": c4_kernel, "bytes_counted": note, "kernel_ms_avg": round(avg, 5)}}), flush=True)
             finally:
                 eng.close()
     return 0
