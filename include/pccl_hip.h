@@ -144,7 +144,7 @@ typedef struct {
     int32_t num_levels;         /* longest dependency chain over data ops */
     int32_t position_aligned;   /* 1 if every data op reads and writes the same element positions */
     int32_t num_segments;       /* column plan: maximal position ranges with one op list */
-    int32_t residual_signals;   /* semaphores left non-zero by one execution (0 for balanced graphs) */
+    int32_t residual_signals;   /* semaphores one execution leaves at another count than it found (0 for balanced graphs) */
     int64_t buffer_elems;       /* rank-buffer elements the graphs address (max offset+size) */
     int64_t algorithmic_bytes;  /* sum over data ops: reduce 3*n*esize, copy 2*n*esize */
     int64_t column_load_bytes;  /* bytes the column plan loads / stores from memory per execution */
@@ -177,6 +177,18 @@ typedef struct {
  * dependencies, detect deadlock and unordered conflicting accesses.  No reference counterpart:
  * the reference runs one process per rank and synchronises at run time. */
 int pccl_program_link(const pccl_graph* const* graphs, int num_vranks, pccl_program** out);
+/* The same for an execution that finds semaphores above zero: `carried` holds num_carried triples
+ * (rank, signal id, count), the state earlier executions left in the engine's signal region (the
+ * reference zeroes it only in Engine::resetSignals, csrc/engine_c.cc:576-593).  The first `count`
+ * waits on such a semaphore pass without a notify of this execution (cuda_executor.cu:425-445) and
+ * are ordered after none.  An engine does this by itself (pccl_hip_execute*); this entry point is for
+ * inspection and tests. */
+int pccl_program_link_carried(const pccl_graph* const* graphs, int num_vranks, const int32_t* carried, int num_carried,
+                              pccl_program** out);
+/* The semaphores a program touches: quadruples (rank, signal id, notifies, waits) of one execution,
+ * ordered by (rank, id); returns their number (fills at most `cap`).  One execution changes the count
+ * of each by notifies - waits. */
+int pccl_program_get_signals(const pccl_program* p, int32_t* out, int cap);
 void pccl_program_free(pccl_program* p);
 int pccl_program_get_info(const pccl_program* p, pccl_program_info* out);
 int pccl_program_get_ops(const pccl_program* p, pccl_linked_op* out, int cap);
@@ -263,7 +275,9 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * persistent runners; the marker library is loaded at run time and PCCL_ERR_UNSUPPORTED is returned
  * if there is none; the environment variable PCCL_TRACE_RANGES=1 sets it for new contexts). */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
-/* The current value of an option as text (the keys of pccl_hip_set_option, "num_vranks", and
+/* The current value of an option as text (the keys of pccl_hip_set_option, "num_vranks", "signals" -
+ * the semaphores that executions so far have left above zero, as "rank:id=count" joined by commas in
+ * (rank, id) order, empty when there are none; PCCL_ERR_INVALID if `cap` is too small for the text -, and
  * "runner_inplace:NAME" / "runner_staged:NAME": the kernel an in-place / staged execution of operation
  * NAME would launch now - "phased_kernel", "column_slot_kernel", "column_kernel", "level_kernel",
  * "persistent_kernel", "gather_kernel", or "staging + ..." - which links the operation): what the
@@ -309,8 +323,22 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
  * entry point and its recorded launch works again. */
 int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* const* bufs, size_t buf_bytes,
                                     void* stream, int sync);
-/* Engine::syncOp / Engine::resetSignals (reference csrc/engine_c.cc:562-593). */
+/* Engine::syncOp (reference csrc/engine_c.cc:562-574). */
 int pccl_hip_sync(pccl_hip_ctx* ctx, const char* name);
+/* Engine::resetSignals (reference csrc/engine_c.cc:576-593): zero the engine's counting semaphores.
+ * As in the reference they are one state per engine, shared by all registered operations, and live
+ * from one execution to the next: a notify that no wait consumed is found by the next execution, of
+ * any operation, that waits on that semaphore (a wait passes on a count above zero and takes one,
+ * cuda_executor.cu:425-445).  This library resolves notifies and waits when it links an operation, so
+ * it keeps the counts on the host (updated when an execution is issued; the caller orders executions
+ * by the streams it issues them to), links an operation for the counts it finds, and links it again
+ * when a later execution finds others (an operation whose notifies and waits balance, on semaphores
+ * nobody left counts on - every schedule template - is linked once).  What follows from a count: a
+ * wait with no notify of its own execution passes once per count and deadlocks (PCCL_ERR_LINK, before
+ * anything runs) without one; a wait that passes on a carried count is ordered after nothing, so data
+ * it was meant to guard may now race (reported as a data race at link time).  An execution that would
+ * move or use counts is refused on a capturing stream (PCCL_ERR_INVALID): a replay could not follow
+ * them.  A name that is not registered is ignored, like in the reference. */
 int pccl_hip_reset_signals(pccl_hip_ctx* ctx, const char* name);
 
 int pccl_hip_op_info(pccl_hip_ctx* ctx, const char* name, pccl_program_info* out);

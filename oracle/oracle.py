@@ -114,10 +114,20 @@ class Graph:
             return cls(json.load(f))
 
 
+NUM_SIGNALS = 4096    # semaphores per rank (include/common/config.h:24)
+
+
+def new_signals(world: int) -> np.ndarray:
+    """The semaphore state of an engine with ``world`` ranks, all zero: pass it to consecutive
+    ``run`` calls to carry counts from one execution into the next (csrc/engine_c.cc:576-593)."""
+    return np.zeros((world, NUM_SIGNALS), dtype=np.int32)
+
+
 def run(graphs: Sequence[Graph], bufs: List[np.ndarray], sched_seed: int = 0,
-        threads: int = 0) -> OracleStats:
+        threads: int = 0, signals: np.ndarray = None) -> OracleStats:
     """Execute the R graphs in place on ``bufs`` (one contiguous array per rank, raw storage:
-    float32/int32 as themselves, float16/bfloat16 as uint16 bit patterns)."""
+    float32/int32 as themselves, float16/bfloat16 as uint16 bit patterns).  ``signals`` (from
+    ``new_signals``) is the semaphore state to start from, updated in place; None starts from zero."""
     L = lib()
     R = len(graphs)
     dtype = graphs[0].dtype
@@ -130,8 +140,11 @@ def run(graphs: Sequence[Graph], bufs: List[np.ndarray], sched_seed: int = 0,
                                              for g in graphs])
     ptrs = (ctypes.c_void_p * R)(*[b.ctypes.data for b in bufs])
     st = OracleStats()
-    rc = L.pccl_oracle_run(R, nops, tabs, dtype, ptrs, ctypes.c_int64(nelems),
-                           ctypes.c_uint32(sched_seed), threads, ctypes.byref(st))
+    if signals is not None:
+        assert signals.dtype == np.int32 and signals.shape == (R, NUM_SIGNALS) and signals.flags["C_CONTIGUOUS"]
+    rc = L.pccl_oracle_run_carry(R, nops, tabs, dtype, ptrs, ctypes.c_int64(nelems),
+                                 ctypes.c_uint32(sched_seed), threads,
+                                 ctypes.c_void_p(signals.ctypes.data if signals is not None else None), ctypes.byref(st))
     if rc != 0:
         raise OracleError(L.pccl_oracle_last_error().decode())
     return st

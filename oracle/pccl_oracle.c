@@ -40,6 +40,14 @@
  *   signals + runner   counting semaphores.  PINNED by the closed forms of the reference's own
  *                      correctness script (tests/test_correctness.py:142-289) and by brute-force
  *                      evaluation of each schedule's per-element reduction order.
+ *   counts carried     pccl_oracle_run_carry: the semaphore region outlives an execution and is
+ *   over               shared by all operations of an engine (engine_c.cc:131-146, cleared only by
+ *                      resetSignals :576-593).  The reference has no test of it; PINNED by known
+ *                      answers that follow from executeWaitNotify / executeNotify alone: a wait with
+ *                      no notify anywhere deadlocks from zero and passes, once per count, on what an
+ *                      earlier execution left; the state after k executions of an operation with
+ *                      n notifies and w waits on a semaphore is k (n - w); resetSignals restores
+ *                      the deadlock (tests/test_oracle.py).
  *   tails              the reference drops the last n % (16/sizeof T) elements of every chunk and
  *                      issues unconditional 16-byte loads (compute.h:26,52; vec.h:25-28), so sizes
  *                      and offsets that are not multiples of 16 bytes have no defined reference
@@ -302,9 +310,27 @@ static uint32_t lcg(uint32_t* s) { *s = *s * 1664525u + 1013904223u; return *s >
  *   threads          OpenMP threads for the element loops (<=0: library default)
  * Returns 0 on success, -1 bad argument / out-of-range access, -2 deadlock.
  */
+int pccl_oracle_run_carry(int R, const int32_t* nops, const oracle_op* const* ops, int dtype,
+                          void* const* bufs, int64_t buf_elems, uint32_t sched_seed, int threads,
+                          int32_t* signals_io, oracle_stats* stats);
+
 int pccl_oracle_run(int R, const int32_t* nops, const oracle_op* const* ops, int dtype,
                     void* const* bufs, int64_t buf_elems, uint32_t sched_seed, int threads,
                     oracle_stats* stats) {
+    return pccl_oracle_run_carry(R, nops, ops, dtype, bufs, buf_elems, sched_seed, threads, NULL, stats);
+}
+
+/*
+ * The same with the semaphores handed in and out: signals_io holds R x ORACLE_NUM_SIGNALS counts
+ * (rank-major), read as the state the execution starts from and left as the state it ends in.  The
+ * reference keeps one signal region per engine for all registered operations and clears it only in
+ * Engine::resetSignals (csrc/engine_c.cc:576-593): counts that one execution leaves above zero are
+ * what the waits of the next execution, of any operation, find (cuda_executor.cu:425-445: a wait
+ * passes on a positive count and takes one).  NULL: start from zero and forget, as pccl_oracle_run.
+ */
+int pccl_oracle_run_carry(int R, const int32_t* nops, const oracle_op* const* ops, int dtype,
+                          void* const* bufs, int64_t buf_elems, uint32_t sched_seed, int threads,
+                          int32_t* signals_io, oracle_stats* stats) {
     int es = pccl_oracle_elem_size(dtype);
     if (R <= 0 || !es) { snprintf(g_err, sizeof g_err, "bad R=%d or dtype=%d", R, dtype); return -1; }
 #ifdef _OPENMP
@@ -312,7 +338,7 @@ int pccl_oracle_run(int R, const int32_t* nops, const oracle_op* const* ops, int
 #endif
     oracle_stats st; memset(&st, 0, sizeof st);
     int rc = 0;
-    int32_t* signals = calloc((size_t)R * ORACLE_NUM_SIGNALS, sizeof(int32_t));
+    int32_t* signals = signals_io ? signals_io : calloc((size_t)R * ORACLE_NUM_SIGNALS, sizeof(int32_t));
     int** remaining = calloc(R, sizeof(int*));
     fifo* queues = calloc((size_t)R * ORACLE_MAX_CHANNELS, sizeof(fifo));
     int64_t total = 0, done = 0;
@@ -406,7 +432,8 @@ out:
         if (remaining[r]) free(remaining[r]);
         for (int c = 0; c < ORACLE_MAX_CHANNELS; c++) free(queues[r * ORACLE_MAX_CHANNELS + c].q);
     }
-    free(remaining); free(queues); free(signals);
+    free(remaining); free(queues);
+    if (!signals_io) free(signals);
     if (stats) *stats = st;
     return rc;
 }

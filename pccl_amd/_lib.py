@@ -83,6 +83,7 @@ EXPORTS = [
     "pccl_graph_load_file", "pccl_graph_load_json", "pccl_graph_from_triggers", "pccl_graph_free",
     "pccl_graph_num_ops", "pccl_graph_dtype", "pccl_graph_tensor_elems", "pccl_graph_collective_type",
     "pccl_graph_get_triggers", "pccl_graph_get_meta", "pccl_graph_fused_steps", "pccl_program_link",
+    "pccl_program_link_carried", "pccl_program_get_signals",
     "pccl_program_free", "pccl_program_get_info", "pccl_program_get_ops", "pccl_program_get_column",
     "pccl_hip_create",
     "pccl_hip_destroy", "pccl_hip_register_file", "pccl_hip_register_json", "pccl_hip_register_triggers",
@@ -121,6 +122,8 @@ def lib() -> ctypes.CDLL:
         "pccl_graph_get_meta": (i32, [vp, P(PrimitiveMeta), i32]),
         "pccl_graph_fused_steps": (i32, [vp, P(FusedStep), i32, P(ctypes.c_int), P(ctypes.c_int)]),
         "pccl_program_link": (i32, [P(vp), i32, P(vp)]),
+        "pccl_program_link_carried": (i32, [P(vp), i32, P(ctypes.c_int32), i32, P(vp)]),
+        "pccl_program_get_signals": (i32, [vp, P(ctypes.c_int32), i32]),
         "pccl_program_free": (None, [vp]),
         "pccl_program_get_info": (i32, [vp, P(ProgramInfo)]),
         "pccl_program_get_ops": (i32, [vp, P(LinkedOp), i32]),
@@ -231,12 +234,23 @@ class HostGraph:
 class HostProgram:
     """R graphs linked into one program (host side only)."""
 
-    def __init__(self, graphs):
+    def __init__(self, graphs, carried=None):
+        """``carried``: ``{(rank, signal_id): count}`` left by earlier executions (default: none)."""
         arr = (ctypes.c_void_p * len(graphs))(*[g._h for g in graphs])
         h = ctypes.c_void_p()
-        check(lib().pccl_program_link(arr, len(graphs), ctypes.byref(h)))
+        flat = [v for (rank, sid), count in sorted((carried or {}).items()) for v in (rank, sid, count)]
+        trip = (ctypes.c_int32 * max(len(flat), 1))(*flat)
+        check(lib().pccl_program_link_carried(arr, len(graphs), trip, len(flat) // 3, ctypes.byref(h)))
         self._h = h
         self._graphs = graphs
+
+    def signals(self) -> dict:
+        """``{(rank, signal_id): (notifies, waits)}`` of one execution."""
+        L = lib()
+        n = L.pccl_program_get_signals(self._h, None, 0)
+        buf = (ctypes.c_int32 * max(4 * n, 1))()
+        L.pccl_program_get_signals(self._h, buf, n)
+        return {(buf[4 * i], buf[4 * i + 1]): (buf[4 * i + 2], buf[4 * i + 3]) for i in range(n)}
 
     def __del__(self):
         if getattr(self, "_h", None) and _lib is not None:

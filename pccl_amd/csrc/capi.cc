@@ -132,16 +132,18 @@ void fill_info(const Program& p, pccl_program_info* out) {
     out->staged_chain_segments = (int)p.direct_chain_segs.size();
 }
 
-// What a linked program does differently from the reference, said once at link time (WARN, the
+// What a reader of the log should know about a linked program, said once at link time (WARN, the
 // default threshold).  The reference keeps its counting semaphores across executions and across
 // operations (zeroed only by resetSignals, csrc/engine_c.cc:576-593; a wait passes on any count
-// above zero, csrc/plugins/cuda/cuda_executor.cu:425-445): a notify nobody awaits would there be
-// carried into the next execution, here every execution starts from zero.
+// above zero and takes one, csrc/plugins/cuda/cuda_executor.cu:425-445), and so does an engine
+// here: a notify nobody awaits is found by the next execution that waits on that semaphore.
 void warn_about(const Program& p, const std::string& what, bool races_wanted) {
     if (p.residual_signals != 0)
-        log_line(LOG_WARN, what + ": " + std::to_string(p.residual_signals) + " semaphore(s) are left above zero by one execution "
-                               "(a notify without a wait); the reference would carry those counts into the next execution, "
-                               "this executor starts every execution from zero");
+        log_line(LOG_WARN, what + ": one execution leaves " + std::to_string(p.residual_signals) + " semaphore(s) at another count than it "
+                               "found them (notifies and waits do not balance); the counts are carried into the next execution of any "
+                               "operation on this engine, as in the reference, until reset_signals");
+    if (p.carried_waits != 0)
+        log_line(LOG_INFO, what + ": " + std::to_string(p.carried_waits) + " wait(s) pass on counts that earlier executions left behind");
     if (!p.order_checked)
         log_line(LOG_WARN, what + ": " + std::to_string(p.num_all_ops) + " ops are too many for the notify/wait ambiguity check and the "
                                "data-race check; the pairing of one valid execution order is used unverified");
@@ -247,6 +249,36 @@ int pccl_program_link(const pccl_graph* const* graphs, int num_vranks, pccl_prog
     });
 }
 
+int pccl_program_link_carried(const pccl_graph* const* graphs, int num_vranks, const int32_t* carried, int num_carried,
+                              pccl_program** out) {
+    return guarded([&] {
+        if (!graphs || !out || (num_carried > 0 && !carried) || num_carried < 0) return fail(PCCL_ERR_INVALID, "null argument");
+        std::vector<const RankGraph*> gs;
+        for (int r = 0; r < num_vranks; ++r) gs.push_back(graphs[r] ? &graphs[r]->g : nullptr);
+        LinkOptions opt;
+        for (int i = 0; i < num_carried; ++i) {
+            const int32_t* c = carried + 3 * (size_t)i;
+            if (c[0] < 0 || c[0] >= num_vranks || c[2] < 0)
+                return fail(PCCL_ERR_INVALID, "carried count " + std::to_string(i) + ": rank " + std::to_string(c[0]) + ", count " + std::to_string(c[2]));
+            opt.carried.push_back({{(int)c[0], (int)c[1]}, (int)c[2]});
+        }
+        auto p = std::make_unique<pccl_program>();
+        p->p = link_program(gs, opt);
+        warn_about(p->p, "linked program", true);
+        *out = p.release();
+        return 0;
+    });
+}
+
+int pccl_program_get_signals(const pccl_program* p, int32_t* out, int cap) {
+    if (!p || (!out && cap > 0)) return fail(PCCL_ERR_INVALID, "null argument");
+    const std::vector<SignalUse>& u = p->p.signals;
+    for (size_t i = 0; i < u.size() && (int)i < cap; ++i) {
+        out[4 * i] = u[i].rank; out[4 * i + 1] = u[i].id; out[4 * i + 2] = u[i].notifies; out[4 * i + 3] = u[i].waits;
+    }
+    return (int)u.size();
+}
+
 void pccl_program_free(pccl_program* p) { delete p; }
 
 int pccl_program_get_info(const pccl_program* p, pccl_program_info* out) {
@@ -327,6 +359,9 @@ struct OpEntry {
     // half (the tables uploaded: allocations and copies).  Inspection needs the first only; the
     // second happens at the first execution, and not on a stream that is being captured.
     bool host_linked = false;
+    bool uses_scanned = false;
+    std::vector<SignalUse> sig_uses;      // the semaphores the graphs touch (depends on the graphs only)
+    std::vector<int> link_carried;        // per sig_uses entry: the carried count the current link was made for
     struct HostTables {
         std::vector<DevColSegment> segs, direct_segs;
         std::vector<DevChainSegment> chain_segs, direct_chain_segs;   // phased runner (empty: the plan is not a chain plan)
@@ -450,6 +485,11 @@ struct pccl_hip_ctx {
     int32_t host_epoch_limit = kHostEpochLimit;   // persistent runner: launch number at which the host clears the flags and restarts
     int32_t graph_epoch_limit = kGraphEpochLimit; // the same for the device-side counter of recorded launches
     hipStream_t last_stream = nullptr;
+    // Counting semaphores above zero, (rank, id) -> count: what executions so far have left behind.
+    // One state per engine, shared by all operations, cleared by pccl_hip_reset_signals - the
+    // reference's signal region (csrc/engine_c.cc:131-146, 576-593).  Updated when an execution is
+    // issued: executions are ordered by the streams they are issued to, as the caller orders them.
+    std::map<std::pair<int, int>, int> signals;
 };
 
 namespace {
@@ -483,6 +523,64 @@ void ensure_buffers(pccl_hip_ctx* ctx, size_t bytes, hipStream_t stream) {
     ctx->buf_bytes = rounded;
 }
 
+// The counts an execution of `e` would find now on the semaphores it touches, one per entry of
+// e.sig_uses, cut off at the number of waits it has there (a higher count changes nothing for it).
+std::vector<int> carried_now(pccl_hip_ctx* ctx, OpEntry& e) {
+    if (!e.uses_scanned) {
+        std::vector<const RankGraph*> gs;
+        for (int r = 0; r < ctx->R; ++r) gs.push_back(r < (int)e.graphs.size() ? e.graphs[r].get() : nullptr);
+        e.sig_uses = signal_uses(gs);
+        e.uses_scanned = true;
+    }
+    std::vector<int> out;
+    out.reserve(e.sig_uses.size());
+    for (const SignalUse& u : e.sig_uses) {
+        auto it = ctx->signals.find(std::make_pair((int)u.rank, (int)u.id));
+        out.push_back(it == ctx->signals.end() ? 0 : std::min(it->second, (int)u.waits));
+    }
+    return out;
+}
+
+// Before an execution or an inspection of `e`: its link has to be the one for the counts its
+// semaphores hold now.  A program whose waits find other counts than its link assumed pairs its
+// notifies and waits differently (and may deadlock or race where it did not), so it is linked again;
+// operations whose notifies and waits balance, on semaphores nobody left counts on - every schedule
+// template - never come here twice.
+void refresh_link(pccl_hip_ctx* ctx, OpEntry& e, hipStream_t s, bool executing, bool may_free_device = true) {
+    const std::vector<int> now = carried_now(ctx, e);
+    bool moves = false, carried = false;
+    for (size_t i = 0; i < now.size(); ++i) {
+        moves = moves || e.sig_uses[i].notifies != e.sig_uses[i].waits;
+        carried = carried || now[i] > 0;
+    }
+    if (executing && (moves || carried) && is_capturing(s))
+        throw Error{PCCL_ERR_INVALID, "the stream is capturing and this operation's semaphores carry counts from one execution to the next "
+                                      "(its notifies and waits do not balance, or an earlier execution left counts on them): a recorded launch "
+                                      "could not follow them.  Execute it outside the capture, or call reset_signals first if the counts are not wanted"};
+    if ((e.host_linked || e.linked) && now != e.link_carried) {
+        if (e.linked) {
+            if (!may_free_device)
+                throw Error{PCCL_ERR_INVALID, "the semaphore counts this operation finds have changed since it was linked and its plan tables on the "
+                                              "device would have to be replaced, which this entry point may not do (it frees nothing): execute the "
+                                              "operation once through pccl_hip_execute_inplace, or call reset_signals"};
+            HIP_TRY(hipDeviceSynchronize());
+        }
+        e.release();
+    }
+}
+
+// An execution of `e` has been issued: its notifies and waits are now part of the engine's state.
+void commit_signals(pccl_hip_ctx* ctx, const OpEntry& e) {
+    for (const SignalUse& u : e.sig_uses) {
+        const int d = u.notifies - u.waits;
+        if (d == 0) continue;
+        const auto key = std::make_pair((int)u.rank, (int)u.id);
+        int& c = ctx->signals[key];
+        c += d;
+        if (c <= 0) ctx->signals.erase(key);     // never below zero: the link would have reported a deadlock
+    }
+}
+
 // Host half of linking: the program, the shape of the slot runner's workgroups, the tables as the
 // kernels read them.  No HIP call.
 void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
@@ -493,6 +591,10 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
     LinkOptions opt;
     opt.check_races = ctx->check_races;
     opt.step_tile_bytes = ctx->step_tile_bytes;
+    const std::vector<int> carried = carried_now(ctx, e);
+    for (size_t i = 0; i < carried.size(); ++i)
+        if (carried[i] > 0) opt.carried.push_back({{(int)e.sig_uses[i].rank, (int)e.sig_uses[i].id}, carried[i]});
+    e.link_carried = carried;
     e.prog = link_program(gs, opt);
     const Program& P = e.prog;
     const int es = elem_size(P.dtype);
@@ -1116,6 +1218,7 @@ int register_graph(pccl_hip_ctx* ctx, const char* name, int vrank, RankGraph&& g
     if (e.graphs.empty()) e.graphs.resize(ctx->R);
     if (e.linked) HIP_TRY(hipDeviceSynchronize());
     if (e.linked || e.host_linked) e.release();  // re-registration replaces the op
+    e.uses_scanned = false;
     e.graphs[vrank] = std::make_unique<RankGraph>(std::move(g));
     if (log_threshold() <= LOG_INFO)   // reference engine_c.cc:168,199
         log_line(LOG_INFO, std::string("operation '") + name + "' registered for virtual rank " + std::to_string(vrank) + ": " +
@@ -1314,12 +1417,17 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
         else if (k == "slot_lds_kib") v = std::to_string(ctx->slot_lds_kib);
         else if (k == "step_tile_bytes") v = std::to_string(ctx->step_tile_bytes);
         else if (k == "num_vranks") v = std::to_string(ctx->R);
+        else if (k == "signals") {   // the semaphores above zero, "rank:id=count" joined by commas, ordered by (rank, id)
+            for (const auto& kv : ctx->signals)
+                v += (v.empty() ? "" : ",") + std::to_string(kv.first.first) + ":" + std::to_string(kv.first.second) + "=" + std::to_string(kv.second);
+        }
         else if (k.rfind("runner_inplace:", 0) == 0 || k.rfind("runner_staged:", 0) == 0) {
             // which kernel an execution of that operation would launch now, given its plan, the tensors'
             // size and the options (16-byte aligned, non-overlapping tensors assumed)
             const bool staged = k[7] == 's';
             OpEntry& e = find_entry(ctx, k.c_str() + (staged ? 14 : 15));
             HIP_TRY(hipSetDevice(ctx->device));
+            refresh_link(ctx, e, nullptr, false);
             link_entry(ctx, e);
             const Program& P = e.prog;
             const bool column_ok = ctx->mode == Mode::Auto || ctx->mode == Mode::Column;
@@ -1345,6 +1453,7 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
         hipStream_t s = (hipStream_t)stream;
+        refresh_link(ctx, e, s, true);
         link_entry(ctx, e, s, true);
         for (int r = 0; r < ctx->R; ++r)
             if (!inputs[r] || !outputs[r]) return fail(PCCL_ERR_INVALID, "null tensor for virtual rank " + std::to_string(r));
@@ -1352,6 +1461,7 @@ int pccl_hip_execute(pccl_hip_ctx* ctx, const char* name, const void* const* inp
         if (!run_direct(ctx, e, inputs, outputs, in_bytes, out_bytes, s) &&
             !run_gather(ctx, e, inputs, outputs, in_bytes, out_bytes, s))
             run_staged(ctx, e, inputs, outputs, in_bytes, out_bytes, s);
+        commit_signals(ctx, e);
         ctx->last_stream = s;
         if (sync) { HIP_TRY(hipStreamSynchronize(s)); check_stall(e, name); }
         return 0;
@@ -1366,11 +1476,13 @@ int pccl_hip_execute_inplace(pccl_hip_ctx* ctx, const char* name, void* const* b
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
         hipStream_t s = (hipStream_t)stream;
+        refresh_link(ctx, e, s, true);
         link_entry(ctx, e, s, true);
         {
             TraceRange exe(ctx->trace_ranges, "execute");
             run_program(ctx, e, (char* const*)bufs, buf_bytes, s);
         }
+        commit_signals(ctx, e);
         ctx->last_stream = s;
         if (sync) { HIP_TRY(hipStreamSynchronize(s)); check_stall(e, name); }
         return 0;
@@ -1384,9 +1496,10 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
         std::lock_guard<std::mutex> lock(ctx->mu);
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
+        hipStream_t s = (hipStream_t)stream;
+        refresh_link(ctx, e, s, true, false);            // never frees device memory here
         link_host(ctx, e);                               // host memory only
         const Program& P = e.prog;
-        hipStream_t s = (hipStream_t)stream;
         StaticWorkspace& ws = static_ws(ctx->device);
         std::lock_guard<std::mutex> wlock(ws.mu);
         if (!ws.ptr) return fail(PCCL_ERR_HIP, "the static workspace of this GPU has no address");
@@ -1440,6 +1553,7 @@ int pccl_hip_execute_inplace_static(pccl_hip_ctx* ctx, const char* name, void* c
             rc = launch_persistent(L, ptrs, s);
         }
         if (rc) { ws.owner = 0; return fail(PCCL_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString((hipError_t)rc)); }
+        commit_signals(ctx, e);
         e.ran_static = true;
         ctx->last_stream = s;
         if (sync) {
@@ -1473,8 +1587,11 @@ int pccl_hip_reset_signals(pccl_hip_ctx* ctx, const char* name) {
         if (it == ctx->ops.end()) return 0;
         HIP_TRY(hipSetDevice(ctx->device));
         HIP_TRY(hipStreamSynchronize(ctx->last_stream));
-        // Semaphores are resolved at link time, so no signal array survives an execution; what can
-        // be left over is the runner's progress block after an aborted launch.
+        // The reference clears the engine's whole signal region, whichever operation is named
+        // (csrc/engine_c.cc:576-593): every carried count goes.  Operations that were linked for other
+        // counts are linked again when they are next executed.  What else can be left over is the
+        // runner's progress block after an aborted launch.
+        ctx->signals.clear();
         OpEntry& e = it->second;
         if (e.linked && e.state.p) {
             int rc = launch_fill_zero(e.state.p, e.state.bytes, ctx->last_stream);
@@ -1492,6 +1609,7 @@ int pccl_hip_op_info(pccl_hip_ctx* ctx, const char* name, pccl_program_info* out
         std::lock_guard<std::mutex> lock(ctx->mu);
         HIP_TRY(hipSetDevice(ctx->device));
         OpEntry& e = find_entry(ctx, name);
+        refresh_link(ctx, e, nullptr, false);
         link_host(ctx, e);      // inspection needs no device memory
         fill_info(e.prog, out);
         if (e.slot_threads > 0) {   // the traffic of the runner this context would launch

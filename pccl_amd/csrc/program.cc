@@ -237,6 +237,23 @@ static void plan_chains(Program& P, const std::vector<ColSegment>& segs, std::ve
     *out = std::move(chains);
 }
 
+std::vector<SignalUse> signal_uses(const std::vector<const RankGraph*>& graphs) {
+    std::map<std::pair<int, int>, SignalUse> uses;
+    for (size_t r = 0; r < graphs.size(); ++r) {
+        if (!graphs[r]) continue;
+        for (const GraphOp& o : graphs[r]->ops) {
+            if (o.kind != OpKind::Wait && o.kind != OpKind::Notify) continue;
+            const auto key = std::make_pair(o.kind == OpKind::Wait ? (int)r : (int)o.peer, (int)o.off0);
+            SignalUse& u = uses[key];
+            u.rank = key.first; u.id = key.second;
+            (o.kind == OpKind::Wait ? u.waits : u.notifies) += 1;
+        }
+    }
+    std::vector<SignalUse> out;
+    for (const auto& kv : uses) out.push_back(kv.second);
+    return out;
+}
+
 // The linker: R per-rank graphs in, one Program out.  Each step is a method; they run in the order
 // `run` calls them and hand their results on through the members.
 namespace {
@@ -334,6 +351,12 @@ class Linker {
             }
         // per (target rank, id): notify nodes not yet consumed, in arrival order
         std::map<std::pair<int, int>, std::deque<int>> pending;
+        // counts carried in from earlier executions: a wait takes one of these before it takes a notify
+        // of this execution (the waits on one semaphore are ordered among themselves, so the first
+        // ones are the ones that pass unconditionally at run time too)
+        std::map<std::pair<int, int>, int> credit;
+        for (const auto& c : opt.carried)
+            if (c.second > 0) credit[c.first] += c.second;
         exec_order.reserve(N);
         int done = 0;
         while (done < N) {
@@ -347,10 +370,16 @@ class Linker {
                         int id = base[r] + i;
                         if (o.kind == OpKind::Wait) {
                             auto key = std::make_pair(r, (int)o.off0);
-                            auto it = pending.find(key);
-                            if (it == pending.end() || it->second.empty()) break;  // blocked
-                            nodes[id].preds.push_back(it->second.front());
-                            it->second.pop_front();
+                            auto cr = credit.find(key);
+                            if (cr != credit.end() && cr->second > 0) {
+                                --cr->second;                    // passes on a carried count: ordered after nothing here
+                                ++P.carried_waits;
+                            } else {
+                                auto it = pending.find(key);
+                                if (it == pending.end() || it->second.empty()) break;  // blocked
+                                nodes[id].preds.push_back(it->second.front());
+                                it->second.pop_front();
+                            }
                             wait_seq[key].push_back(id);
                         } else if (o.kind == OpKind::Notify) {
                             auto key = std::make_pair(o.peer, (int)o.off0);
@@ -377,7 +406,9 @@ class Linker {
                 throw Error{PCCL_ERR_LINK, "deadlock: " + std::to_string(done) + " of " + std::to_string(N) + " ops can run; blocked: " + blocked};
             }
         }
-        for (auto& kv : pending) if (!kv.second.empty()) P.residual_signals++;
+        std::vector<const RankGraph*> gs(graphs.begin(), graphs.end());
+        P.signals = signal_uses(gs);
+        for (const SignalUse& u : P.signals) if (u.notifies != u.waits) P.residual_signals++;
     }
 
     // Reachability (happens-before) over all ops, in execution order.

@@ -75,6 +75,13 @@ struct StepOpPlan {
     int lead = 0;   // elements between the item grid's anchor and the op's first element (< tile_elems)
 };
 
+// One semaphore a program touches: how often one execution notifies it and waits on it.  The counts a
+// program leaves behind are (carried in) + notifies - waits, whatever order the ranks ran in.
+struct SignalUse {
+    int32_t rank = 0, id = 0;       // the semaphore: signal `id` of rank `rank`
+    int32_t notifies = 0, waits = 0;
+};
+
 struct Program {
     int R = 0;
     int dtype = PCCL_F32;
@@ -83,7 +90,9 @@ struct Program {
     std::vector<LinkedOp> ops;  // topological order: (level, rank, channel, position)
     int num_all_ops = 0;
     int num_levels = 0;
-    int residual_signals = 0;
+    int residual_signals = 0;       // semaphores one execution leaves at another count than it found
+    std::vector<SignalUse> signals; // every semaphore the program touches, ordered by (rank, id)
+    int carried_waits = 0;          // waits that passed on a count carried in (LinkOptions::carried)
     int64_t buffer_elems = 0;
     int64_t algorithmic_bytes = 0;
     bool race_checked = false;    // the data-race check ran over every pair of conflicting accesses
@@ -123,7 +132,15 @@ struct LinkOptions {
     bool check_races = true;
     bool conflict_deps = true;     // order data ops by memory conflicts instead of raw chain order
     int64_t step_tile_bytes = 0;   // bytes per work item of the stepwise plan; 0 = chosen from the program's size
+    // Semaphore counts this execution finds, left by earlier executions on the same engine (the
+    // reference clears its signal region only in Engine::resetSignals, csrc/engine_c.cc:576-593):
+    // ((rank, id), count) for the counts above zero.  The first `count` waits on such a semaphore
+    // pass without a notify of this execution and get no ordering from one.
+    std::vector<std::pair<std::pair<int, int>, int>> carried;
 };
+
+// The semaphores the graphs touch, without linking them (registration order does not matter).
+std::vector<SignalUse> signal_uses(const std::vector<const RankGraph*>& graphs);
 
 // Throws Error (PCCL_ERR_LINK for deadlock, ambiguous signal pairing, races, bad ranks).
 Program link_program(const std::vector<const RankGraph*>& graphs, const LinkOptions& opt);

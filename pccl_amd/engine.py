@@ -102,7 +102,7 @@ class Engine:
         _lib.check(self._L.pccl_hip_set_option(self._h, key.encode(), str(value).encode()))
 
     def get_option(self, key: str) -> str:
-        buf = ctypes.create_string_buffer(64)
+        buf = ctypes.create_string_buffer(65536 if key == "signals" else 64)
         _lib.check(self._L.pccl_hip_get_option(self._h, key.encode(), buf, len(buf)))
         return buf.value.decode()
 
@@ -195,7 +195,20 @@ class Engine:
         _lib.check(self._L.pccl_hip_sync(self._h, name.encode()))
 
     def reset_signals(self, name: str) -> None:
+        """Zero every counting semaphore of the engine (reference ``Engine::resetSignals``,
+        ``csrc/engine_c.cc:576-593``: the signal region is one per engine, whichever operation is named)."""
         _lib.check(self._L.pccl_hip_reset_signals(self._h, name.encode()))
+
+    def signals(self) -> dict:
+        """The semaphores that executions so far have left above zero: ``{(rank, signal_id): count}``.
+        The next execution of any operation finds them (a wait passes on a count above zero and takes
+        one, reference ``csrc/plugins/cuda/cuda_executor.cu:425-445``)."""
+        out = {}
+        for item in filter(None, self.get_option("signals").split(",")):
+            key, _, count = item.partition("=")
+            rank, _, sid = key.partition(":")
+            out[(int(rank), int(sid))] = int(count)
+        return out
 
     def op_info(self, name: str) -> dict:
         out = _lib.ProgramInfo()

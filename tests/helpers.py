@@ -154,6 +154,56 @@ def random_program(seed: int, world: int, n: int, num_ops: int, dtype: str, alig
     return out
 
 
+def carry_ops(n: int = 64, dtype: str = "float32") -> dict:
+    """Two-rank operations whose notifies and waits do not balance, for the semaphore state that the
+    reference keeps from one execution to the next (csrc/engine_c.cc:576-593).  h = n / 2.
+      give  rank 0: own[0:h] <- rank 1's [0:h]; notify (1, 5) twice.   rank 1: wait 5; own[h:n] <- rank 0's [h:n].
+            One notify is left over: (1, 5) goes up by one.
+      take  rank 0: own[h:n] <- rank 1's [h:n].   rank 1: wait 5 (nobody notifies it here); own[0:h] += rank 0's [0:h].
+            Runs only on a count that an earlier execution left: (1, 5) goes down by one.
+      pair  rank 0: own[0:h] += rank 1's [0:h]; notify (1, 5).   rank 1: wait 5; own[h:n] <- rank 0's [0:h].
+            Balanced, and race-free from zero; on a carried count the wait passes before the notify and
+            rank 1's copy is no longer ordered after rank 0's reduce: a data race."""
+    h = n // 2
+
+    def build(rank, body):
+        with CommunicationOp(name=f"carry{rank}") as op:
+            op.tensor(dtype=dtype, shape=(n,))
+            body(op)
+        return compile_to_json_string(op.get_graph())
+
+    return {
+        "give": [build(0, lambda op: (op.sm_copy(source_rank=1, src_offset=0, dst_offset=0, size=h),
+                                      op.notify(signal_id=5, target_rank=1), op.notify(signal_id=5, target_rank=1))),
+                 build(1, lambda op: (op.wait_notify(signal_id=5, source_rank=0),
+                                      op.sm_copy(source_rank=0, src_offset=h, dst_offset=h, size=n - h)))],
+        "take": [build(0, lambda op: op.sm_copy(source_rank=1, src_offset=h, dst_offset=h, size=n - h)),
+                 build(1, lambda op: (op.wait_notify(signal_id=5, source_rank=0),
+                                      op.sm_reduce(source_rank=0, remote_offset=0, src_offset=0, dst_offset=0, count=h)))],
+        "pair": [build(0, lambda op: (op.sm_reduce(source_rank=1, remote_offset=0, src_offset=0, dst_offset=0, count=h),
+                                      op.notify(signal_id=5, target_rank=1))),
+                 build(1, lambda op: (op.wait_notify(signal_id=5, source_rank=0),
+                                      op.sm_copy(source_rank=0, src_offset=0, dst_offset=h, size=h)))],
+    }
+
+
+def carry_expected(name: str, bufs: Sequence[np.ndarray]) -> List[np.ndarray]:
+    """What one execution of a ``carry_ops`` operation leaves in the two rank buffers, written from the
+    operation's description with numpy (float32 or int32 arrays)."""
+    a, b = bufs[0].copy(), bufs[1].copy()
+    h = len(a) // 2
+    if name == "give":
+        a[:h], b[h:] = bufs[1][:h], bufs[0][h:]
+    elif name == "take":
+        a[h:], b[:h] = bufs[1][h:], bufs[0][:h] + bufs[1][:h]
+    elif name == "pair":
+        a[:h] = bufs[1][:h] + bufs[0][:h]
+        b[h:2 * h] = a[:h]
+    else:
+        raise KeyError(name)
+    return [a, b]
+
+
 def to_raw(t: torch.Tensor) -> np.ndarray:
     """CPU tensor -> numpy array of its storage bits (bf16/f16 as uint16)."""
     t = t.contiguous()

@@ -354,12 +354,72 @@ def test_residual_signals_are_counted():
     assert info["race_checked"] == 1 and info["order_checked"] == 1
 
 
-def test_linker_warns_where_an_execution_would_differ_from_the_reference():
-    """A notify without a wait leaves its semaphore above zero; the reference carries that count into
-    the next execution (signals are only zeroed by resetSignals, csrc/engine_c.cc:576-593, and a wait
-    passes on any count above zero, cuda_executor.cu:425-445), this executor starts from zero every
-    time: said at WARN level when the program is linked.  A balanced graph links silently.  A program
-    too large for the ambiguity and race checks says that they were skipped."""
+def test_linking_for_counts_that_earlier_executions_left():
+    """The linker given the semaphore state an execution finds (reference: one signal region per
+    engine, cleared only by resetSignals, csrc/engine_c.cc:576-593; a wait passes on a count above
+    zero and takes one, cuda_executor.cu:425-445) against the oracle given the same state: the same
+    programs run or deadlock, and counts move by notifies - waits."""
+    import json
+    import numpy as np
+    from helpers import carry_ops, oracle
+    n = 64
+    jsons = carry_ops(n)
+    hg = {k: [HostGraph.from_json(j) for j in v] for k, v in jsons.items()}
+    og = {k: [oracle.Graph(json.loads(j)) for j in v] for k, v in jsons.items()}
+    uses = {k: HostProgram(v, {(1, 5): 1} if k == "take" else None).signals() for k, v in hg.items()}
+    assert uses == {"give": {(1, 5): (2, 1)}, "take": {(1, 5): (0, 1)}, "pair": {(1, 5): (1, 1)}}
+    for count in range(0, 4):
+        for name in ("give", "take", "pair"):
+            carried = {(1, 5): count} if count else {}
+            sig = oracle.new_signals(2)
+            sig[1, 5] = count
+            bufs = [np.zeros(n, dtype=np.float32) for _ in range(2)]
+            try:
+                oracle.run(og[name], bufs, signals=sig)
+                oracle_runs = True
+            except oracle.OracleError as e:
+                assert "deadlock" in str(e)
+                oracle_runs = False
+            try:
+                prog = HostProgram(hg[name], carried)
+                links, msg = True, ""
+            except PcclError as e:
+                links, msg = False, str(e)
+            if name == "pair" and count > 0:
+                # the oracle runs it in one of the orders the semaphores allow; the linker sees that the
+                # copy is no longer ordered after the reduce it reads from
+                assert oracle_runs and not links and "data race" in msg
+                continue
+            assert links == oracle_runs, (name, count, msg)
+            if links:
+                notifies, waits = prog.signals()[(1, 5)]
+                assert int(sig[1, 5]) == count + notifies - waits
+                assert prog.info()["residual_signals"] == (0 if notifies == waits else 1)
+            else:
+                assert "deadlock" in msg and "signal 5" in msg
+    # a count on another semaphore, or on the same id of the other rank, changes nothing
+    assert "deadlock" in _link_err_carried(hg["take"], {(0, 5): 3, (1, 6): 2})
+    # the two leftover waits of two ranks are told apart: one count lets one wait through
+    both = _two_rank(lambda op, me, other: (op.wait_notify(signal_id=2, source_rank=other),
+                                            op.sm_copy(source_rank=other, src_offset=32 * other, dst_offset=32 * other, size=32)))
+    hb = [HostGraph.from_json(j) for j in both]
+    assert "rank 1" in _link_err_carried(hb, {(0, 2): 1})
+    assert HostProgram(hb, {(0, 2): 1, (1, 2): 4}).info()["num_data_ops"] == 2
+
+
+def _link_err_carried(graphs, carried):
+    with pytest.raises(PcclError) as e:
+        HostProgram(graphs, carried)
+    assert e.value.code == ERR_LINK
+    return str(e.value)
+
+
+def test_linker_says_when_semaphores_do_not_balance():
+    """A notify without a wait leaves its semaphore above zero, and the next execution of any
+    operation finds it there (signals are only zeroed by resetSignals, csrc/engine_c.cc:576-593, and a
+    wait passes on any count above zero, cuda_executor.cu:425-445): said at WARN level when the
+    program is linked.  A balanced graph links silently.  A program too large for the ambiguity and
+    race checks says that they were skipped."""
     import subprocess
     import sys
     code = ("import sys, json; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
@@ -387,7 +447,7 @@ def test_linker_warns_where_an_execution_would_differ_from_the_reference():
 
     vals, err = run("unbalanced")
     assert vals == ["2", "1", "1"]
-    assert "[pccl] [warning]" in err and "2 semaphore(s) are left above zero" in err and "reference would carry" in err
+    assert "[pccl] [warning]" in err and "leaves 2 semaphore(s) at another count" in err and "carried into the next execution" in err
     vals, err = run("balanced")
     assert vals == ["0", "1", "1"] and "[pccl]" not in err
     vals, err = run("big")     # 64 ranks x 4 channels: more ops than the quadratic checks take

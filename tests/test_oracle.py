@@ -9,8 +9,8 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import (FP8_MAX, TORCH_DTYPE, bits_equal, from_raw, graph_jsons, mismatch_report, oracle,
-                     oracle_buffers, seeded_inputs, to_raw)
+from helpers import (FP8_MAX, TORCH_DTYPE, bits_equal, carry_expected, carry_ops, from_raw, graph_jsons, mismatch_report,
+                     oracle, oracle_buffers, seeded_inputs, to_raw)
 
 
 # ------------------------------------------------------------------------------- element arithmetic
@@ -361,6 +361,49 @@ def test_wait_without_notify_is_reported_as_deadlock():
     graphs = [oracle.Graph(json.loads(j)) for j in jsons]
     with pytest.raises(oracle.OracleError, match="deadlock"):
         oracle.run(graphs, [np.zeros(16, dtype=np.float32) for _ in range(2)])
+
+
+def test_counts_carried_from_one_execution_to_the_next():
+    """The reference keeps one signal region per engine and clears it only in Engine::resetSignals
+    (csrc/engine_c.cc:131-146, 576-593); a wait passes on a count above zero and takes one
+    (cuda_executor.cu:425-445).  Known answers that follow from those two functions alone: an
+    operation whose only wait has no notify deadlocks from zero and runs, once per count, on what
+    earlier executions left; k executions of an operation with n notifies and w waits on a semaphore
+    move it by k (n - w); clearing the region brings the deadlock back.  Buffers against numpy."""
+    n = 64
+    ops = {k: [oracle.Graph(json.loads(j)) for j in v] for k, v in carry_ops(n).items()}
+    rng = np.random.default_rng(5)
+    bufs = [rng.standard_normal(n).astype(np.float32) for _ in range(2)]
+    sig = oracle.new_signals(2)
+
+    def state():
+        return {(int(r), int(i)): int(sig[r, i]) for r, i in zip(*np.nonzero(sig))}
+
+    def step(name):
+        nonlocal bufs
+        want = carry_expected(name, bufs)
+        oracle.run(ops[name], bufs, signals=sig)
+        for got, w in zip(bufs, want):
+            assert np.array_equal(got.view(np.int32), w.view(np.int32)), name
+    with pytest.raises(oracle.OracleError, match="deadlock"):
+        oracle.run(ops["take"], [b.copy() for b in bufs], signals=oracle.new_signals(2))
+    step("give"); assert state() == {(1, 5): 1}
+    step("take"); assert state() == {}
+    with pytest.raises(oracle.OracleError, match="deadlock"):
+        oracle.run(ops["take"], [b.copy() for b in bufs], signals=sig.copy())
+    for k in range(1, 4):
+        step("give"); assert state() == {(1, 5): k}
+    step("pair"); assert state() == {(1, 5): 3}          # balanced: leaves what it found
+    for k in (2, 1, 0):
+        step("take"); assert state() == ({(1, 5): k} if k else {})
+    # without a state handed in every execution starts from zero, as before
+    oracle.run(ops["give"], bufs)
+    with pytest.raises(oracle.OracleError, match="deadlock"):
+        oracle.run(ops["take"], bufs)
+    # resetSignals: the region is zeroed, the deadlock is back
+    step("give"); sig[:] = 0
+    with pytest.raises(oracle.OracleError, match="deadlock"):
+        oracle.run(ops["take"], bufs, signals=sig)
 
 
 def test_out_of_range_access_is_an_error():
