@@ -259,13 +259,17 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * wave stores whole tiles of some ranks; 0: every wave stores a slice of every rank; -1, the default:
  * 1 for plans that write at least four times what they read, such as an allgather);
  * "phased" = "-1" | "0" | "1" (column plans in chain form - ring allreduce, staged reduce_scatter and
- * allgather, trees under an operator that may be re-associated - on the phased runner: one persistent
- * workgroup per CU, the whole chip reads, meets, writes, meets; -1, the default: when the tensors give
- * every CU at least two 128 KiB chunks of each rank); "phased_shape" = "-1" | "0" | "1" (its workgroup:
- * 512 threads x 16 vectors, or 256 x 32 with each wave on 32 KiB in a row; -1: by rank count);
- * "phased_barriers" = "1" | "0" (0: no meetings, for comparison); "phased_timeout_us" (how long a
- * workgroup waits at a meeting before the launch goes on unsynchronised: meetings order nothing; the
- * environment variable PCCL_PHASED sets "phased" for new contexts);
+ * allgather, trees under an operator that may be re-associated, balanced trees of float sums - on the
+ * phased runner: one persistent workgroup per CU, the whole chip reads, meets, writes, meets; -1, the
+ * default: when the tensors give every CU at least one 128 KiB chunk of each rank and the plan does
+ * not store more than twice what it loads, which leaves an allgather on the slot runner);
+ * "phased_shape" = "-1" | "0" | "1" (its workgroup: 512 threads x 16 vectors, or 256 x 32; -1: by rank
+ * count); "phased_exchange" = "-1" | "0" | "1" (the 256 x 32 shape on chains: 1, and -1, read as slabs
+ * and write with each wave on 32 KiB in a row, the sums changing hands through LDS in between; 0: each
+ * wave on 32 KiB in a row for reads as well); "phased_barriers" = "1" | "0" (0: no meetings, for
+ * comparison); "phased_timeout_us" (how long a workgroup waits at a meeting before the launch goes on
+ * unsynchronised: meetings order nothing; the environment variable PCCL_PHASED sets "phased" for new
+ * contexts);
  * "level_graph" = "0" | "1" (the level runner launches level by level, or replays the launches of an
  * execution as one HIP graph captured per set of rank pointers);
  * "trace_ranges" = "0" | "1" (host-side roctx ranges around the stages of a call, under the names of

@@ -473,6 +473,7 @@ struct pccl_hip_ctx {
                                           // (1), every wave a slice of every rank (0), or chosen from the plan's traffic (-1)
     int phased = -1;                      // chain plans on the phased runner (whole chip reads, then writes): 1 whenever the
                                           // plan is a chain plan, 0 never, -1 when it is and the tensors are large enough
+    int phased_exchange = -1;             // 256 x 32 shapes: the sums change hands through LDS between read and write phase (-1 chosen, 0, 1)
     int phased_shape = -1;                // its workgroup: 0 = 512 threads x 16 vectors, 1 = 256 x 32 (a wave's vectors contiguous), -1 chosen
     bool phased_barriers = true;          // its workgroups meet between the phases (0: they run free, for comparison)
     int phased_timeout_us = 1000;         // how long a workgroup waits at a meeting point before the launch goes on unsynchronised
@@ -882,6 +883,10 @@ int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtr
     // peak, 32 ranks 81 % against 83 %)
     const int tree_shape = direct ? e.direct_chain_tree : e.chain_tree;
     L.shape = tree_shape ? tree_shape : ctx->phased_shape >= 0 ? ctx->phased_shape : (ctx->R <= 8 ? 0 : 1);
+    // 256 x 32 chains read as slabs and write with each wave on 32 KiB in a row, the sums changing hands
+    // through LDS between the phases (32 ranks x 96 MiB: int32 SUM 0.822 -> 0.842 of peak, f32 MAX
+    // 0.820 -> 0.840; 16-rank bf16 ring 0.335 -> 0.327 ms); trees gain nothing from it and keep their shape
+    if (ctx->phased_exchange != 0 && L.shape == 1) L.shape = 3;
     L.num_blocks = ctx->num_blocks;
     // a plan that mostly reads (a reduce_scatter: R chunks in, one out) gains nothing from meeting:
     // its write phases are too short to matter (8 x 64 MB fp16: 89 us without, 94 us with)
@@ -1349,6 +1354,11 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased_shape must be -1 (automatic), 0 (512 threads x 16 vectors) or 1 (256 x 32)");
             ctx->phased_shape = x;
         }
+        else if (k == "phased_exchange") {
+            const int x = std::atoi(value);
+            if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased_exchange must be -1 (automatic), 0 or 1");
+            ctx->phased_exchange = x;
+        }
         else if (k == "phased_barriers") ctx->phased_barriers = std::atoi(value) != 0;
         else if (k == "phased_timeout_us") { ctx->phased_timeout_us = std::atoi(value); if (ctx->phased_timeout_us < 0) ctx->phased_timeout_us = 0; }
         else if (k == "lds_slots") { ctx->lds_slots = std::atoi(value) != 0; relink = true; }
@@ -1409,6 +1419,7 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
         else if (k == "level_graph") v = std::to_string((int)ctx->level_graph);
         else if (k == "phased") v = std::to_string(ctx->phased);
         else if (k == "phased_shape") v = std::to_string(ctx->phased_shape);
+        else if (k == "phased_exchange") v = std::to_string(ctx->phased_exchange);
         else if (k == "phased_barriers") v = std::to_string((int)ctx->phased_barriers);
         else if (k == "phased_timeout_us") v = std::to_string(ctx->phased_timeout_us);
         else if (k == "lds_slots") v = std::to_string((int)ctx->lds_slots);

@@ -217,6 +217,63 @@ __device__ __forceinline__ u32x4 vec_fast(u32x4 a, u32x4 b) {
     }
 }
 
+// The arithmetic of vec_fast with nothing done about NaN results, and the canonicalisation as a step
+// of its own.  A NaN never turns back into a number under SUM, MAX or MIN (IEEE 754-2019 maximum and
+// minimum propagate it, as addition does, and the bf16 rounding keeps a quiet NaN a NaN), so a chain or
+// tree of these operations gives a NaN at its end exactly when one of its steps did, and making only the
+// end result canonical gives the bits that canonicalising after every step gives.  The read phases of
+// the phased runner use this: their loops then hold no branch, and the loads of the next vectors are
+// not held up behind a test of this one's result.  Not for a value that no operation produced (a
+// copied NaN keeps its payload), and not for the 8-bit floats (their clamp would lose a NaN).
+template <int DT, int OP>
+__device__ __forceinline__ u32x4 vec_bare(u32x4 a, u32x4 b) {
+    if constexpr (DT == PCCL_F32) {
+        return u32x4{as_u32(f32_comb<OP>(as_f32(a.x), as_f32(b.x))), as_u32(f32_comb<OP>(as_f32(a.y), as_f32(b.y))),
+                     as_u32(f32_comb<OP>(as_f32(a.z), as_f32(b.z))), as_u32(f32_comb<OP>(as_f32(a.w), as_f32(b.w)))};
+    } else if constexpr (DT == PCCL_BF16) {
+        auto word = [](uint32_t x, uint32_t y) {
+            const f32x2 pair = {f32_comb<OP>(as_f32(x << 16), as_f32(y << 16)), f32_comb<OP>(as_f32(x & 0xFFFF0000u), as_f32(y & 0xFFFF0000u))};
+            return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
+        };
+        return u32x4{word(a.x, b.x), word(a.y, b.y), word(a.z, b.z), word(a.w, b.w)};
+    } else if constexpr (DT == PCCL_F16) {
+        auto word = [](uint32_t x, uint32_t y) {
+            return __builtin_bit_cast(uint32_t, f16x2_comb<OP>(__builtin_bit_cast(h2, x), __builtin_bit_cast(h2, y)));
+        };
+        return u32x4{word(a.x, b.x), word(a.y, b.y), word(a.z, b.z), word(a.w, b.w)};
+    } else {
+        return vec_fast<DT, OP>(a, b);
+    }
+}
+// f32 and f16 chains and trees run with the deferred form (16-rank halving-doubling 0.762 -> 0.786 of
+// peak, 32-rank f32 MAX 0.796 -> 0.840, f16 reduce_scatter 0.800 -> 0.807).  bf16 keeps the test per
+// step: its arithmetic is seven instructions per element pair, and without a branch after every vector
+// the compiler gathers the arithmetic of a whole rank behind that rank's last fetch, where no fetch
+// overlaps it (headline 0.791 -> 0.767; with the arithmetic pinned after each group of fetches 0.781).
+template <int DT> constexpr bool kDeferredNan = DT == PCCL_F32 || DT == PCCL_F16;
+template <int DT, int OP>
+__device__ __forceinline__ u32x4 vec_phase(u32x4 a, u32x4 b) {
+    if constexpr (kDeferredNan<DT>) return vec_bare<DT, OP>(a, b); else return vec_fast<DT, OP>(a, b);
+}
+
+template <int DT>
+__device__ __forceinline__ u32x4 canon_nan(u32x4 r) {
+    if constexpr (DT == PCCL_F32) {
+        auto word = [](uint32_t w) { return (w & 0x7FFFFFFFu) > 0x7F800000u ? 0x7FFFFFFFu : w; };
+        return u32x4{word(r.x), word(r.y), word(r.z), word(r.w)};
+    } else if constexpr (DT == PCCL_BF16 || DT == PCCL_F16) {
+        constexpr uint32_t inf = DT == PCCL_BF16 ? 0x7F80u : 0x7C00u;
+        auto word = [](uint32_t w) {
+            if ((w & 0x7FFFu) > inf) w = (w & 0xFFFF0000u) | 0x7FFFu;
+            if ((w & 0x7FFF0000u) > (inf << 16)) w = (w & 0x0000FFFFu) | 0x7FFF0000u;
+            return w;
+        };
+        return u32x4{word(r.x), word(r.y), word(r.z), word(r.w)};
+    } else {
+        return r;
+    }
+}
+
 // One decision on the operator per vector: each branch below inlines the word code with a
 // constant operator, so the four words run back to back without tests in between.
 template <int DT>
@@ -1112,6 +1169,14 @@ __global__ __launch_bounds__(1024 / V) void column_slot_kernel(ColumnLaunch L, R
 // Chunks that a segment boundary cuts are run vector by vector by the same workgroup (loads and
 // stores of one vector together, cut vectors stored element by element): there are at most two per
 // segment.
+//
+// Which vectors of its chunk a thread holds (LAY): 0 = the chunk as V slabs of T vectors, thread t
+// vector t of every slab (all waves of a workgroup read and write one 1 KiB-per-wave slab together);
+// 1 = each wave V KiB in a row, for reads and writes; 2 = read as slabs, written with each wave on
+// V KiB in a row: the sums change hands through LDS between the two phases (T x V x 16 bytes, the
+// fetch ring's space included).  Reads are fastest as slabs and writes with long runs per wave
+// (bare kernels, 32 ranks x 96 MiB: read phases 6.9-7.0 against 6.8 TB/s, write phases 6.5 against
+// 5.6-6.0); what the exchange costs is two LDS passes per sweep, about a microsecond in 80 to 330.
 
 // One workgroup per CU: the kernel asks for more than half a CU's LDS, so that two cannot share one.
 constexpr int kPhasedLdsBytes = 84 * 1024;
@@ -1177,7 +1242,7 @@ __device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int
 #pragma unroll
             for (int g = 0; g < GR; ++g) x[g] = mine[((v + g) % S) * T];
 #pragma unroll
-            for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_fast<DT, OP>(x[g], acc[v + g]);
+            for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_phase<DT, OP>(x[g], acc[v + g]);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
 #pragma unroll
             for (int g = 0; g < GR; ++g) {
@@ -1187,6 +1252,12 @@ __device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int
             }
         }
         cur = next;
+    }
+    if constexpr (kDeferredNan<DT>) {
+        if (n > 1) {      // a single source is a copy: its bits are kept as they are
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v] = canon_nan<DT>(acc[v]);
+        }
     }
 }
 
@@ -1238,16 +1309,16 @@ __device__ __forceinline__ void tree_read(u32x4 (&acc)[V], const PCCL_CONST int3
             else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(S - 4) : "memory");
             const u32x4 l0 = mine[(q & (S - 1)) * T], l1 = mine[((q + 1) & (S - 1)) * T];
             const u32x4 l2 = mine[((q + 2) & (S - 1)) * T], l3 = mine[((q + 3) & (S - 1)) * T];
-            u32x4 y = vec_fast<DT, PCCL_SUM>(vec_fast<DT, PCCL_SUM>(l0, l1), vec_fast<DT, PCCL_SUM>(l2, l3));
+            u32x4 y = vec_phase<DT, PCCL_SUM>(vec_phase<DT, PCCL_SUM>(l0, l1), vec_phase<DT, PCCL_SUM>(l2, l3));
             int climb = __builtin_ctz(~(unsigned)(k >> 2));      // trailing one bits of the quad number (uniform)
             if (climb > upper) climb = upper;
 #pragma unroll
             for (int lvl = 0; lvl < kMaxUpper; ++lvl)
-                if (lvl < climb) y = vec_fast<DT, PCCL_SUM>(parked[lvl], y);
+                if (lvl < climb) y = vec_phase<DT, PCCL_SUM>(parked[lvl], y);
 #pragma unroll
             for (int lvl = 0; lvl < kMaxUpper; ++lvl)
                 if (lvl == climb && lvl < upper) parked[lvl] = y;
-            if (climb == upper) root = y;                        // the last quad carries the root
+            if (climb == upper) root = kDeferredNan<DT> ? canon_nan<DT>(y) : y;   // the last quad carries the root
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
             if (q + S < total) { fetch(q + S); fetch(q + S + 1); fetch(q + S + 2); fetch(q + S + 3); }
         }
@@ -1258,22 +1329,25 @@ __device__ __forceinline__ void tree_read(u32x4 (&acc)[V], const PCCL_CONST int3
     fill_by_index(acc, one_vector, std::make_integer_sequence<int, V>{});
 }
 
-template <int DT, int T, int V, int S, bool WAVEC, int GR, bool TREE>
+template <int DT, int T, int V, int S, int LAY, int GR, bool TREE>
 __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs) {
     extern __shared__ u32x4 lds[];
     __shared__ int s_flag;
-    static_assert((size_t)S * T * 16 <= 160u * 1024, "the fetch ring must fit a CU's LDS");
+    static_assert((size_t)S * T * 16 <= 159u * 1024, "the fetch ring must fit a CU's LDS");
+    static_assert(LAY != 2 || ((size_t)T * V * 16 <= 159u * 1024 && S <= V), "so must a chunk's sums when they change hands through it");
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
     constexpr int64_t CHUNK_V = (int64_t)T * V;
-    constexpr int VS = WAVEC ? 64 * 16 : T * 16;             // bytes between a thread's consecutive vectors
+    constexpr int VS = LAY == 1 ? 64 * 16 : T * 16;          // bytes between a thread's consecutive vectors while it reads
+    constexpr int WVS = LAY >= 1 ? 64 * 16 : T * 16;         // ... and while it writes
     const int tid = threadIdx.x;
     const int G = gridDim.x;
     // workgroup b runs on XCD b % 8: every XCD takes a contiguous eighth of each sweep
     const int place = (G & 7) == 0 ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
     // thread's first vector inside a chunk: each wave a contiguous V KiB, or the chunk as V slabs of T vectors
-    const uint32_t tvec = WAVEC ? (uint32_t)(tid >> 6) * V * 64 + (tid & 63) : (uint32_t)tid;
-    const uint32_t toff = tvec * 16;
+    const uint32_t wavec = (uint32_t)(tid >> 6) * V * 64 + (tid & 63);
+    const uint32_t toff = (LAY == 1 ? wavec : (uint32_t)tid) * 16;
+    const uint32_t wtoff = (LAY >= 1 ? wavec : (uint32_t)tid) * 16;
     const int64_t sweeps = (L.total_chunks + G - 1) / G;
     bool meet = L.barriers != 0;
     int gen = 0;
@@ -1342,6 +1416,19 @@ __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs
                 }
             }
         }
+        if constexpr (LAY == 2) {
+            if (live && whole) {            // uniform over the workgroup: the barriers are reached by all or by none
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();            // every wave has consumed its ring slots: the space is free
+#pragma unroll
+                for (int v = 0; v < V; ++v) lds[v * T + tid] = acc[v];          // position v T + t of the chunk
+                __syncthreads();
+#pragma unroll
+                for (int v = 0; v < V; ++v) acc[v] = lds[wavec + v * 64];
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __syncthreads();            // all have their sums before the next sweep's fetches land here
+            }
+        }
         if (meet) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
@@ -1353,7 +1440,7 @@ __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs
             for (uint64_t m = seg.store_mask; m; m &= m - 1) {
                 char* const dst = ptrs.p[__builtin_ctzll(m)] + vbase * 16;
 #pragma unroll
-                for (int v = 0; v < V; ++v) stv_nt_s(dst, toff + v * VS, acc[v]);
+                for (int v = 0; v < V; ++v) stv_nt_s(dst, wtoff + v * WVS, acc[v]);
             }
         }
         if (meet && it + 1 < sweeps) {
@@ -1478,10 +1565,11 @@ int launch_column(const ColumnLaunch& L, const RankPtrs& ptrs, void* stream) {
 }
 
 template <class K>
-static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads, int ring_slots, const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
+static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads, int lds_vectors, const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
     const int dev = current_device();
-    // the fetch ring, and never less than what keeps a second workgroup off the CU
-    const int lds = std::max(kPhasedLdsBytes, ring_slots * threads * 16);
+    // the fetch ring (or a chunk's sums where they change hands through LDS), and never less than what
+    // keeps a second workgroup off the CU
+    const int lds = std::max(kPhasedLdsBytes, lds_vectors * threads * 16);
     if (!allowed[dev].load(std::memory_order_relaxed)) {
         hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (rc != hipSuccess) return (int)rc;
@@ -1496,16 +1584,17 @@ static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads
 
 template <int DT>
 static int launch_phased_dt(const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
-    static std::atomic<int> allowed[3][kMaxDevices];
+    static std::atomic<int> allowed[4][kMaxDevices];
     // integer sums never arrive as trees (the planner re-associates them into chains), and the 8-bit
     // floats' arithmetic leaves no registers for the tree code
     constexpr bool kNoTrees = DT == PCCL_I32 || DT == PCCL_F8E4M3 || DT == PCCL_F8E5M2;
     switch (L.shape) {
-        case 0: return launch_phased_kernel(phased_kernel<DT, 512, 16, 4, false, 2, false>, allowed[0], 512, 4, L, ptrs, s);
-        case 1: return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, true, 2, false>, allowed[1], 256, 8, L, ptrs, s);
+        case 0: return launch_phased_kernel(phased_kernel<DT, 512, 16, 4, 0, 2, false>, allowed[0], 512, 4, L, ptrs, s);
+        case 1: return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, 1, 2, false>, allowed[1], 256, 8, L, ptrs, s);
         case 2:
             if constexpr (kNoTrees) return (int)hipErrorInvalidValue;
-            else return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, true, 2, true>, allowed[2], 256, 8, L, ptrs, s);
+            else return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, 1, 2, true>, allowed[2], 256, 8, L, ptrs, s);
+        case 3: return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, 2, 2, false>, allowed[3], 256, 32, L, ptrs, s);
         default: return (int)hipErrorInvalidValue;
     }
 }

@@ -57,18 +57,22 @@ def test_chain_and_tree_plans_in_place_and_staged(engine_factory, case):
         # grids: one workgroup per CU; 5 workgroups (not a multiple of the XCD count, many sweeps and
         # meetings); meetings off; a wait that gives up at once
         for blocks, barriers, timeout in ((0, 1, 1000), (5, 1, 1000), (8, 0, 1000), (16, 1, 0)):
-            for shape in ((-1,) if tree else (0, 1)):
-                what = f"blocks={blocks} barriers={barriers} timeout={timeout} shape={shape}"
+            # shapes: 512 x 16; 256 x 32 with each wave on 32 KiB in a row; the same read as slabs, the sums
+            # changing hands through LDS before they are written (trees choose their shape themselves)
+            for shape, exchange in (((-1, -1),) if tree else ((0, 0), (1, 0), (1, 1))):
+                what = f"blocks={blocks} barriers={barriers} timeout={timeout} shape={shape} exchange={exchange}"
                 print(f"{name}: {what}", flush=True)
                 eng.set_option("num_blocks", blocks); eng.set_option("phased_barriers", barriers)
                 eng.set_option("phased_timeout_us", timeout); eng.set_option("phased_shape", shape)
+                eng.set_option("phased_exchange", exchange)
                 bufs = [t.cuda() for t in x]
                 eng.execute_inplace(name, bufs, sync=True)
                 _check(bufs, want, f"in place, {what}")
                 outs = eng.execute_operation(name, [t.cuda() for t in x])
                 _check(outs, want, f"staged, {what}")
     finally:
-        for key, val in (("phased", -1), ("num_blocks", 0), ("phased_barriers", 1), ("phased_timeout_us", 1000), ("phased_shape", -1)):
+        for key, val in (("phased", -1), ("num_blocks", 0), ("phased_barriers", 1), ("phased_timeout_us", 1000), ("phased_shape", -1),
+                         ("phased_exchange", -1)):
             eng.set_option(key, val)
 
 
@@ -191,3 +195,66 @@ def test_phased_launches_recorded_into_a_graph(engine_factory):
             _check(bufs, want, f"replay {rep}")
     finally:
         eng.set_option("phased", -1)
+
+
+SPECIAL_BITS = {   # quiet NaNs with payloads, a signalling NaN, infinities, zeros, the smallest denormal, the largest finite values
+    "float32": [0x7FC00000, 0x7FC12345, 0xFFC00001, 0x7F800001, 0x7F800000, 0xFF800000, 0x00000000, 0x80000000, 0x00000001, 0x7F7FFFFF, 0xFF7FFFFF],
+    "bfloat16": [0x7FC0, 0x7FC5, 0xFFC1, 0x7F81, 0x7F80, 0xFF80, 0x0000, 0x8000, 0x0001, 0x7F7F, 0xFF7F],
+    "float16": [0x7E00, 0x7E05, 0xFE01, 0x7C01, 0x7C00, 0xFC00, 0x0000, 0x8000, 0x0001, 0x7BFF, 0xFBFF],
+}
+
+
+def _with_specials(x, dtype, seed):
+    """One element in a hundred of every rank replaced by a special bit pattern."""
+    import numpy as np
+    from helpers import from_raw, to_raw
+    rng = np.random.default_rng(seed)
+    out = []
+    for t in x:
+        raw = to_raw(t).copy()
+        where = rng.random(raw.shape[0]) < 0.01
+        raw[where] = rng.choice(np.array(SPECIAL_BITS[dtype], dtype=raw.dtype), int(where.sum()))
+        out.append(from_raw(raw, dtype))
+    return out
+
+
+@pytest.mark.parametrize("case", [
+    ("ring", "build_allreduce", 8, "bfloat16", "sum"), ("ring", "build_allreduce", 4, "float16", "sum"),
+    ("ring", "build_allreduce", 16, "float32", "sum"), ("tree", "build_allreduce", 16, "float32", "max"),
+    ("tree", "build_allreduce", 8, "float16", "min"), ("tree", "build_allreduce", 32, "bfloat16", "max"),
+    ("rhd", "build_allreduce", 16, "float32", "sum"), ("tree", "build_allreduce", 32, "bfloat16", "sum"),
+    ("rhd", "build_allreduce", 8, "float16", "sum"), ("ring", "build_allgather", 8, "float32", "sum"),
+], ids=lambda c: f"{c[0]}-{c[1][6:]}-R{c[2]}-{c[3]}-{c[4]}")
+def test_nans_infinities_and_zeros_through_chains_and_trees(engine_factory, case):
+    """The read phases canonicalise NaN results once, at the end of a chain or tree, instead of after
+    every step: same bits as the oracle, which does it step by step - NaN payloads and signalling
+    NaNs among the inputs, infinities of both signs meeting in a sum, signed zeros under MAX and MIN.
+    An allgather only copies: its NaNs keep their payloads."""
+    alg, method, world, dtype, op = case
+    per = {"float32": 4, "bfloat16": 8, "float16": 8}[dtype]
+    n = world * (2 * CHUNK_VECS * per + 40)              # chunks cut by the ends, for the vector-by-vector path too
+    ext = {} if method == "build_allgather" else {"reduce_op": op}
+    jsons = graph_jsons(alg, method, world, n, dtype, "sm", 1, **ext)
+    gather = method == "build_allgather"
+    chunk = n // world
+    x = _with_specials(seeded_inputs("randn", world, chunk if gather else n, dtype, seed=world), dtype, seed=17 + world)
+    want = oracle_buffers(jsons, x, dtype, buffer_elems=n, place=(lambda r: r * chunk) if gather else None)
+    eng = engine_factory(world)
+    name = f"nan_{alg}_{method}_{world}_{dtype}_{op}"
+    _register(eng, name, jsons)
+    assert eng.op_info(name)["chain_segments" if not gather else "staged_chain_segments"] > 0
+    eng.set_option("phased", 1)
+    try:
+        for exchange in (0, 1):
+            eng.set_option("phased_exchange", exchange)
+            if gather:
+                outs = [torch.empty(n, dtype=x[0].dtype, device="cuda") for _ in range(world)]
+                eng.execute_operation(name, [t.cuda() for t in x], outs)
+                _check(outs, want, f"staged, exchange={exchange}")
+            else:
+                bufs = [t.cuda() for t in x]
+                eng.execute_inplace(name, bufs, sync=True)
+                _check(bufs, want, f"in place, exchange={exchange}")
+                assert eng.get_option(f"runner_inplace:{name}") == "phased_kernel"
+    finally:
+        eng.set_option("phased", -1); eng.set_option("phased_exchange", -1)
