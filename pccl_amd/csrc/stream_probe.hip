@@ -10,7 +10,9 @@
 //                            shape); W = 1: the final stores dealt to the waves
 //          phased:T:V:S:M:L  one persistent workgroup per CU, sums of T x V vectors in registers, ring
 //                            of S slots; M = 0 no meetings, 1 all workgroups meet after the reads and after
-//                            the writes, 2 meet before the reads only; L = 1: a wave's vectors contiguous
+//                            the writes, 2 meet before the reads only; L = 1: a wave's vectors contiguous;
+//                            L = 2: read as slabs, written with a wave's vectors contiguous (the sums
+//                            change hands through LDS between the phases)
 //          read:T / write:T / copy:T   streams only: every workgroup of T threads reads (writes) one
 //                            1 KiB-per-wave tile of every rank; copy: rank r to rank (r + ranks / 2)
 // Every case prints one JSON line; results are checked on the host for the cases that compute.
@@ -127,7 +129,7 @@ __device__ __forceinline__ void meet_wait(Meet* s, int gen) {     // bounded: 0.
     __syncthreads();
 }
 
-template <int T, int V, int S, bool WAVEC>
+template <int T, int V, int S, int LAY>
 __global__ __launch_bounds__(T) void phased_probe(Ptrs p, int R, int64_t chunks, int mode, Meet* meet) {
     extern __shared__ u32x4 lds[];
     static_assert(S <= V && V % S == 0, "ring");
@@ -138,11 +140,14 @@ __global__ __launch_bounds__(T) void phased_probe(Ptrs p, int R, int64_t chunks,
     const u32x4* const mine = lds + tid;
     int gen = 0;
     const int64_t sweeps = (chunks + G - 1) / G;
+    constexpr bool WAVEC = LAY == 1;
     constexpr int64_t VS = WAVEC ? 64 * 16 : (int64_t)T * 16;
+    constexpr int64_t WVS = LAY >= 1 ? 64 * 16 : (int64_t)T * 16;
     for (int64_t it = 0; it < sweeps; ++it) {
         const int64_t chunk = it * G + place;
         const bool live = chunk < chunks;
         const int64_t base = WAVEC ? (chunk * V * T + (int64_t)(tid >> 6) * V * 64 + (tid & 63)) * 16 : (chunk * V * T + tid) * 16;
+        const int64_t wbase = LAY >= 1 ? (chunk * V * T + (int64_t)(tid >> 6) * V * 64 + (tid & 63)) * 16 : base;
         u32x4 acc[V];
 #pragma unroll
         for (int v = 0; v < V; ++v) acc[v] = u32x4{0, 0, 0, 0};
@@ -166,13 +171,24 @@ __global__ __launch_bounds__(T) void phased_probe(Ptrs p, int R, int64_t chunks,
                 }
             }
         }
+        if (LAY == 2) {      // read as slabs, write with each wave on V KiB in a row: the sums change hands through LDS
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+#pragma unroll
+            for (int v = 0; v < V; ++v) lds[v * T + tid] = acc[v];
+            __syncthreads();
+            const int wb = (tid >> 6) * V * 64 + (tid & 63);
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v] = lds[wb + v * 64];
+            if (mode != 1) __syncthreads();
+        }
         if (mode == 1) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); __syncthreads(); ++gen; meet_arrive(meet, gen, G); meet_wait(meet, gen); }
         if (blockIdx.x == 0 && tid == 0 && it < 64) meet->stamps[3 * it + 1] = __builtin_amdgcn_s_memrealtime();
         if (live) {
             for (int r = 0; r < R; ++r) {
-                char* dst = p.p[r] + base;
+                char* dst = p.p[r] + wbase;
 #pragma unroll
-                for (int v = 0; v < V; ++v) st_stream(dst + (int64_t)v * VS, acc[v]);
+                for (int v = 0; v < V; ++v) st_stream(dst + (int64_t)v * WVS, acc[v]);
             }
         }
         if (mode == 1) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); __syncthreads(); ++gen; meet_arrive(meet, gen, G); meet_wait(meet, gen); }
@@ -294,15 +310,17 @@ int main(int argc, char** argv) {
                 extra = buf;
             };
             // the 84 KiB keep a second workgroup off the CU
-            const int lds = std::max(84 * 1024, S * T * 16);
-            if (T == 512 && V == 16 && S == 4 && !L) go(phased_probe<512, 16, 4, false>, lds);
-            else if (T == 512 && V == 16 && S == 4 && L) go(phased_probe<512, 16, 4, true>, lds);
-            else if (T == 512 && V == 16 && S == 8 && !L) go(phased_probe<512, 16, 8, false>, lds);
-            else if (T == 256 && V == 32 && S == 8 && !L) go(phased_probe<256, 32, 8, false>, lds);
-            else if (T == 256 && V == 32 && S == 8 && L) go(phased_probe<256, 32, 8, true>, lds);
-            else if (T == 256 && V == 32 && S == 16 && L) go(phased_probe<256, 32, 16, true>, lds);
-            else if (T == 1024 && V == 8 && S == 8 && !L) go(phased_probe<1024, 8, 8, false>, lds);
-            else if (T == 256 && V == 16 && S == 16 && !L) go(phased_probe<256, 16, 16, false>, lds);
+            const int lds = std::max(84 * 1024, L == 2 ? T * V * 16 : S * T * 16);
+            if (T == 512 && V == 16 && S == 4 && L == 0) go(phased_probe<512, 16, 4, 0>, lds);
+            else if (T == 512 && V == 16 && S == 4 && L == 1) go(phased_probe<512, 16, 4, 1>, lds);
+            else if (T == 512 && V == 16 && S == 4 && L == 2) go(phased_probe<512, 16, 4, 2>, lds);
+            else if (T == 512 && V == 16 && S == 8 && L == 0) go(phased_probe<512, 16, 8, 0>, lds);
+            else if (T == 256 && V == 32 && S == 8 && L == 0) go(phased_probe<256, 32, 8, 0>, lds);
+            else if (T == 256 && V == 32 && S == 8 && L == 1) go(phased_probe<256, 32, 8, 1>, lds);
+            else if (T == 256 && V == 32 && S == 8 && L == 2) go(phased_probe<256, 32, 8, 2>, lds);
+            else if (T == 256 && V == 32 && S == 16 && L == 1) go(phased_probe<256, 32, 16, 1>, lds);
+            else if (T == 1024 && V == 8 && S == 8 && L == 0) go(phased_probe<1024, 8, 8, 0>, lds);
+            else if (T == 256 && V == 16 && S == 16 && L == 0) go(phased_probe<256, 16, 16, 0>, lds);
             else { std::printf("{\"case\": \"%s\", \"error\": \"shape not built\"}\n", c.c_str()); continue; }
             moved = 2.0 * R * (double)chunks * T * V * 16;
         } else if ((c.rfind("read:", 0) == 0 || c.rfind("write:", 0) == 0 || c.rfind("copy:", 0) == 0) && f.size() == 1) {
