@@ -276,17 +276,29 @@ def cpu_baseline(jsons, world: int, sample_elems: int, np_dtype: str, label: str
                       f"full bytes on the CPU), median of {reps} runs after 1 warm-up, {med * 1e3:.1f} ms"}
 
 
+def kernel_source_sha256() -> str:
+    """Hash of the kernel source the library was built from: a counter profile names the one it measured."""
+    import hashlib
+    with open(os.path.join(ROOT, "pccl_amd", "csrc", "kernels.hip"), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
 def committed_traffic(kernel: str, stem: str | None):
     """HBM bytes per launch from the committed rocprofv3 counter summary of `kernel` on the workload
-    `stem` (FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy), with the file it comes from."""
+    `stem` (FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy), with the file it comes from.  The figure is
+    only handed on while the profile was taken on the kernel source that is in the tree now (the file
+    records its hash): after a kernel change `traffic` is null until the profile has been retaken."""
     if not stem:
         return None, None
     rel = os.path.join("profiles", f"{kernel}_{stem}.traffic.json")
     try:
         with open(os.path.join(ROOT, rel)) as f:
-            return json.load(f).get("hbm_bytes_per_launch"), rel
+            rec = json.load(f)
     except (OSError, ValueError):
         return None, None
+    if rec.get("kernels_hip_sha256") != kernel_source_sha256():
+        return None, rel + " (taken on another version of kernels.hip: not used)"
+    return rec.get("hbm_bytes_per_launch"), rel
 
 
 def c4_traffic(kernel: str, kind: str, nbytes: int):

@@ -866,7 +866,11 @@ bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
     const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
     if (2 * loads < stores) return false;
-    return chunks >= (int64_t)device_cu_count(ctx->device);
+    // with meetings it pays from one chunk per CU on (8-rank bf16 ring, 16 MiB per rank: 0.611 against
+    // 0.621 of peak; 32 MiB: 0.694 against 0.764); a plan that mostly reads runs without meetings and
+    // wins from half of that (8-rank fp16 reduce_scatter, 16 MB per rank: 32.6 -> 29.3 us; 8 MB: 18.6 -> 25.8)
+    const int64_t cus = device_cu_count(ctx->device);
+    return loads >= 4 * stores ? 2 * chunks >= cus : chunks >= cus;
 }
 
 int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtrs& ptrs, hipStream_t stream) {

@@ -537,18 +537,31 @@ def test_damaged_documents_are_errors_not_crashes():
 def test_bench_finds_the_committed_counter_figures():
     """bench.py copies the counter-measured HBM bytes per launch of its kernel from the committed
     rocprofv3 summary of the same workload and names that file (`roofline.traffic_source`): the files
-    it looks for exist, hold a positive byte count and sit beside a summary that names their kernel."""
+    it looks for exist, hold a positive byte count, sit beside a summary that names their kernel and
+    record the hash of the kernel source they were taken on - a figure from another version of the
+    kernels is not handed on."""
+    import hashlib
     import importlib.util
+    import json
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     spec = importlib.util.spec_from_file_location("bench_under_test", os.path.join(root, "bench.py"))
     bench = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(bench)
-    wanted = [("column_slot_kernel", "ring_allreduce_R8_bf16_512MiB"), ("level_kernel", "ring_allreduce_R8_bf16_512MiB"),
-              ("persistent_kernel", "ring_allreduce_R8_bf16_512MiB"), ("column_slot_kernel", "rhd_allreduce_R16_f32_64MiB"),
-              ("column_slot_kernel", "tree_allreduce_R32_int32_sum_96MiB"), ("column_slot_kernel", "tree_allreduce_R32_f32_max_96MiB")]
+    current = hashlib.sha256(open(os.path.join(root, "pccl_amd", "csrc", "kernels.hip"), "rb").read()).hexdigest()
+    assert bench.kernel_source_sha256() == current
+    allreduces = ["ring_allreduce_R8_bf16_512MiB", "rhd_allreduce_R16_f32_64MiB", "tree_allreduce_R32_int32_sum_96MiB", "tree_allreduce_R32_f32_max_96MiB"]
+    wanted = [(k, stem) for k in ("phased_kernel", "column_slot_kernel") for stem in allreduces]
+    wanted += [("level_kernel", "ring_allreduce_R8_bf16_512MiB"), ("persistent_kernel", "ring_allreduce_R8_bf16_512MiB"),
+               ("phased_kernel", "ring_reduce_scatter_R8_f16_512MB_staged"), ("column_slot_kernel", "ring_allgather_R8_f16_512MB_staged")]
     for kernel, stem in wanted:
+        path = os.path.join(root, "profiles", f"{kernel}_{stem}.traffic.json")
+        rec = json.load(open(path))
+        assert rec["hbm_bytes_per_launch"] > 0 and len(rec["kernels_hip_sha256"]) == 64, (kernel, stem)
         nbytes, rel = bench.committed_traffic(kernel, stem)
-        assert rel == f"profiles/{kernel}_{stem}.traffic.json" and nbytes and nbytes > 0, (kernel, stem)
+        if rec["kernels_hip_sha256"] == current:
+            assert rel == f"profiles/{kernel}_{stem}.traffic.json" and nbytes == rec["hbm_bytes_per_launch"], (kernel, stem)
+        else:
+            assert nbytes is None and rel.startswith(f"profiles/{kernel}_{stem}.traffic.json") and "not used" in rel
         summary = os.path.join(root, "profiles", f"{kernel}_{stem}.md")
         assert os.path.exists(summary) and kernel in open(summary).read()
     assert bench.committed_traffic("column_slot_kernel", None) == (None, None)
