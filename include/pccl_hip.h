@@ -261,9 +261,8 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * "phased" = "-1" | "0" | "1" (column plans in chain form - ring allreduce, staged reduce_scatter and
  * allgather, trees under an operator that may be re-associated, balanced trees of float sums - on the
  * phased runner: one persistent workgroup per CU, the whole chip reads, meets, writes, meets; -1, the
- * default: when the tensors give every CU at least one 128 KiB chunk of each rank - every second CU
- * for a plan that loads four times what it stores, a reduce_scatter - and the plan does not store more
- * than twice what it loads, which leaves an allgather on the slot runner);
+ * default: when the tensors give at least every second CU a 128 KiB chunk of each rank and the plan
+ * does not store more than twice what it loads, which leaves an allgather on the slot runner);
  * "phased_shape" = "-1" | "0" | "1" (its workgroup: 512 threads x 16 vectors, or 256 x 32; -1: by rank
  * count); "phased_exchange" = "-1" | "0" | "1" (the 256 x 32 shape on chains: 1, and -1, read as slabs
  * and write with each wave on 32 KiB in a row, the sums changing hands through LDS in between; 0: each

@@ -866,11 +866,11 @@ bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
     const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
     if (2 * loads < stores) return false;
-    // with meetings it pays from one chunk per CU on (8-rank bf16 ring, 16 MiB per rank: 0.611 against
-    // 0.621 of peak; 32 MiB: 0.694 against 0.764); a plan that mostly reads runs without meetings and
-    // wins from half of that (8-rank fp16 reduce_scatter, 16 MB per rank: 32.6 -> 29.3 us; 8 MB: 18.6 -> 25.8)
-    const int64_t cus = device_cu_count(ctx->device);
-    return loads >= 4 * stores ? 2 * chunks >= cus : chunks >= cus;
+    // it pays from one chunk per two CUs on (8-rank bf16 ring in place: 16 MiB per rank, 128 chunks,
+    // 0.613 -> 0.637 of peak; 32 MiB 0.679 -> 0.748; 8 MiB 0.563 -> 0.368.  8-rank fp16 reduce_scatter:
+    // 16 MB per rank 32.6 -> 29.3 us, 8 MB 18.6 -> 25.8).  Quarter chunks for the sizes below were
+    // measured (512 threads x 4 vectors) and are no better than the slot runner there.
+    return 2 * chunks >= (int64_t)device_cu_count(ctx->device);
 }
 
 int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtrs& ptrs, hipStream_t stream) {
