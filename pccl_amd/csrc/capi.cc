@@ -474,6 +474,7 @@ struct pccl_hip_ctx {
     int phased = -1;                      // chain plans on the phased runner (whole chip reads, then writes): 1 whenever the
                                           // plan is a chain plan, 0 never, -1 when it is and the tensors are large enough
     int phased_exchange = -1;             // 256 x 32 shapes: the sums change hands through LDS between read and write phase (-1 chosen, 0, 1)
+    int phased_sweeps = -1;               // sweeps read before their sums are written: 1, 2 (512 x 16 only), -1: 2 for plans that mostly read
     int phased_shape = -1;                // its workgroup: 0 = 512 threads x 16 vectors, 1 = 256 x 32 (a wave's vectors contiguous), -1 chosen
     bool phased_barriers = true;          // its workgroups meet between the phases (0: they run free, for comparison)
     int phased_timeout_us = 1000;         // how long a workgroup waits at a meeting point before the launch goes on unsynchronised
@@ -892,11 +893,23 @@ int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtr
     // 0.820 -> 0.840; 16-rank bf16 ring 0.335 -> 0.327 ms); trees gain nothing from it and keep their shape
     if (ctx->phased_exchange != 0 && L.shape == 1) L.shape = 3;
     L.num_blocks = ctx->num_blocks;
-    // a plan that mostly reads (a reduce_scatter: R chunks in, one out) gains nothing from meeting:
-    // its write phases are too short to matter (8 x 64 MB fp16: 89 us without, 94 us with)
+    // a plan that mostly reads (a reduce_scatter: R chunks in, one out) has write phases too short to be
+    // worth a meeting per sweep (8 x 64 MB fp16: 89 us without, 94 us with).  It reads two sweeps and
+    // then writes both (shape 4: bare kernels of that traffic, 8 x 512 MiB in, 8 x 64 MiB out, 0.788 of
+    // peak without meetings, 0.804 with one write phase per sweep, 0.865 per two sweeps, 0.868 per three)
     const int64_t loads = direct ? P.direct_slot_load_bytes : P.slot_load_bytes;
     const int64_t stores = direct ? P.direct_slot_store_bytes : P.slot_store_bytes;
-    L.barriers = ctx->phased_barriers && loads < 4 * stores ? 1 : 0;
+    const bool mostly_reads = loads >= 4 * stores;
+    // (from four sweeps on: 8-rank fp16 reduce_scatter 512 / 256 MB per rank 0.806 -> 0.846 / 0.830 -> 0.848 of
+    // peak, 64 / 32 / 16 MB - two sweeps, one, half a one - 0.837 -> 0.827 / 0.826 -> 0.759 / 0.631 -> 0.563).
+    // The 512 x 16 shape of the other chains (up to 8 ranks) gains from it as well, from two sweeps on:
+    // fewer, longer phases (8-rank bf16 ring in place, 64 / 128 / 256 / 512 MiB per rank: 0.764 -> 0.787,
+    // 0.783 -> 0.786, 0.792 -> 0.801, 0.793 -> 0.798)
+    const int64_t cus = device_cu_count(ctx->device);
+    const bool pays = mostly_reads ? L.total_chunks >= 4 * cus : (L.shape == 0 && L.total_chunks >= 2 * cus);
+    const bool two_sweeps = !tree_shape && (ctx->phased_sweeps == 2 || (ctx->phased_sweeps < 0 && ctx->phased_shape < 0 && pays));
+    if (two_sweeps) L.shape = 4;
+    L.barriers = ctx->phased_barriers && (two_sweeps || !mostly_reads) ? 1 : 0;
     L.sync = (PhaseSync*)e.phase_sync.p;
     L.timeout_ticks = (uint64_t)ctx->phased_timeout_us * 100ull;
     return launch_phased(L, ptrs, stream);
@@ -1358,6 +1371,11 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased_shape must be -1 (automatic), 0 (512 threads x 16 vectors) or 1 (256 x 32)");
             ctx->phased_shape = x;
         }
+        else if (k == "phased_sweeps") {
+            const int x = std::atoi(value);
+            if (x != -1 && x != 1 && x != 2) return fail(PCCL_ERR_INVALID, "phased_sweeps must be -1 (automatic), 1 or 2");
+            ctx->phased_sweeps = x;
+        }
         else if (k == "phased_exchange") {
             const int x = std::atoi(value);
             if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased_exchange must be -1 (automatic), 0 or 1");
@@ -1424,6 +1442,7 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
         else if (k == "phased") v = std::to_string(ctx->phased);
         else if (k == "phased_shape") v = std::to_string(ctx->phased_shape);
         else if (k == "phased_exchange") v = std::to_string(ctx->phased_exchange);
+        else if (k == "phased_sweeps") v = std::to_string(ctx->phased_sweeps);
         else if (k == "phased_barriers") v = std::to_string((int)ctx->phased_barriers);
         else if (k == "phased_timeout_us") v = std::to_string(ctx->phased_timeout_us);
         else if (k == "lds_slots") v = std::to_string((int)ctx->lds_slots);

@@ -110,7 +110,8 @@ struct PhasedLaunch {
     int32_t dtype;
     int32_t shape;            // 0: 512 threads x 16 vectors, 1: 256 threads x 32 vectors (each wave a contiguous 32 KiB),
                               // 2: 256 x 32 with the code for balanced trees as well; 3: as 1, but read as slabs and
-                              // written with each wave on 32 KiB in a row (the sums change hands through LDS)
+                              // written with each wave on 32 KiB in a row (the sums change hands through LDS);
+                              // 4: as 0, two sweeps read before their sums are written
     int32_t num_blocks;       // 0: one workgroup per CU
     int32_t barriers;         // 1: all workgroups read together, then write together; 0: no meeting
     PhaseSync* sync;

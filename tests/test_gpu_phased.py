@@ -59,12 +59,13 @@ def test_chain_and_tree_plans_in_place_and_staged(engine_factory, case):
         for blocks, barriers, timeout in ((0, 1, 1000), (5, 1, 1000), (8, 0, 1000), (16, 1, 0)):
             # shapes: 512 x 16; 256 x 32 with each wave on 32 KiB in a row; the same read as slabs, the sums
             # changing hands through LDS before they are written (trees choose their shape themselves)
-            for shape, exchange in (((-1, -1),) if tree else ((0, 0), (1, 0), (1, 1))):
-                what = f"blocks={blocks} barriers={barriers} timeout={timeout} shape={shape} exchange={exchange}"
+            # and 512 x 16 reading two sweeps before it writes their sums
+            for shape, exchange, sweeps in (((-1, -1, -1),) if tree else ((0, 0, 1), (1, 0, 1), (1, 1, 1), (-1, -1, 2))):
+                what = f"blocks={blocks} barriers={barriers} timeout={timeout} shape={shape} exchange={exchange} sweeps={sweeps}"
                 print(f"{name}: {what}", flush=True)
                 eng.set_option("num_blocks", blocks); eng.set_option("phased_barriers", barriers)
                 eng.set_option("phased_timeout_us", timeout); eng.set_option("phased_shape", shape)
-                eng.set_option("phased_exchange", exchange)
+                eng.set_option("phased_exchange", exchange); eng.set_option("phased_sweeps", sweeps)
                 bufs = [t.cuda() for t in x]
                 eng.execute_inplace(name, bufs, sync=True)
                 _check(bufs, want, f"in place, {what}")
@@ -72,7 +73,7 @@ def test_chain_and_tree_plans_in_place_and_staged(engine_factory, case):
                 _check(outs, want, f"staged, {what}")
     finally:
         for key, val in (("phased", -1), ("num_blocks", 0), ("phased_barriers", 1), ("phased_timeout_us", 1000), ("phased_shape", -1),
-                         ("phased_exchange", -1)):
+                         ("phased_exchange", -1), ("phased_sweeps", -1)):
             eng.set_option(key, val)
 
 
@@ -103,14 +104,14 @@ def test_staged_reduce_scatter_and_allgather(engine_factory, method):
             assert bits_equal(w, whole)
     eng.set_option("phased", 1)
     try:
-        for blocks in (0, 7):
-            eng.set_option("num_blocks", blocks)
+        for blocks, sweeps in ((0, -1), (7, -1), (5, 1), (3, 2)):      # -1: two sweeps per write phase for the reduce_scatter
+            eng.set_option("num_blocks", blocks); eng.set_option("phased_sweeps", sweeps)
             out_elems = chunk if method == "build_reduce_scatter" else n
             outs = [torch.empty(out_elems, dtype=torch.float16, device="cuda") for _ in range(world)]
             eng.execute_operation(name, [t.cuda() for t in x], outs)
-            _check(outs, want, f"{method} blocks={blocks}")
+            _check(outs, want, f"{method} blocks={blocks} sweeps={sweeps}")
     finally:
-        eng.set_option("phased", -1); eng.set_option("num_blocks", 0)
+        eng.set_option("phased", -1); eng.set_option("num_blocks", 0); eng.set_option("phased_sweeps", -1)
 
 
 def test_automatic_choice_and_what_is_not_a_chain(engine_factory):
@@ -245,8 +246,8 @@ def test_nans_infinities_and_zeros_through_chains_and_trees(engine_factory, case
     assert eng.op_info(name)["chain_segments" if not gather else "staged_chain_segments"] > 0
     eng.set_option("phased", 1)
     try:
-        for exchange in (0, 1):
-            eng.set_option("phased_exchange", exchange)
+        for exchange, sweeps in ((0, -1), (1, -1), (-1, 2)):
+            eng.set_option("phased_exchange", exchange); eng.set_option("phased_sweeps", sweeps)
             if gather:
                 outs = [torch.empty(n, dtype=x[0].dtype, device="cuda") for _ in range(world)]
                 eng.execute_operation(name, [t.cuda() for t in x], outs)
@@ -257,4 +258,4 @@ def test_nans_infinities_and_zeros_through_chains_and_trees(engine_factory, case
                 _check(bufs, want, f"in place, exchange={exchange}")
                 assert eng.get_option(f"runner_inplace:{name}") == "phased_kernel"
     finally:
-        eng.set_option("phased", -1); eng.set_option("phased_exchange", -1)
+        eng.set_option("phased", -1); eng.set_option("phased_exchange", -1); eng.set_option("phased_sweeps", -1)
