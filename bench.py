@@ -308,6 +308,24 @@ def c4_traffic(kernel: str, kind: str, nbytes: int):
     return committed_traffic(kernel, f"ring_{kind}_R8_f16_512MB_staged")
 
 
+def release_cached_memory() -> None:
+    """Hands torch's cached blocks back to the driver.  Called where the next configuration uses
+    tensors of other sizes, so that no configuration runs on pieces split off larger cached blocks
+    (32 x 96 MiB carved out of cached 512 MiB blocks: 0.828 of peak against 0.842 on blocks of their
+    own).  Where the next configuration uses the same sizes it takes the blocks over from the cache:
+    memory that a process has freed to the driver and allocated again has been seen to be slower on
+    this GPU (8 x 512 MB reduce_scatter, same process, same call: 0.808 of peak against 0.85 on the
+    process's first allocations; not in every order of allocations).  PCCL_BENCH_FREE_TO_DRIVER=1
+    releases after every configuration, for comparison."""
+    import torch
+    torch.cuda.empty_cache()
+
+
+def release_between_equal_sizes() -> None:
+    if os.environ.get("PCCL_BENCH_FREE_TO_DRIVER", "0") == "1":
+        release_cached_memory()
+
+
 def timed_inplace(eng, name, bufs, steps, warmup):
     """K timed executions in place: wall time per step and per-launch HIP-event times."""
     import torch
@@ -501,7 +519,7 @@ def run_inplace(args, wl: Workload, dev) -> int:
         result["data"] = "synthetic (GPU generator: tuning run)"
     del bufs, pristine
     eng.close()
-    torch.cuda.empty_cache()
+    release_between_equal_sizes()     # the 512 MB pair of configuration 4 comes next, on blocks of the same size
     if not args.no_cpu_baseline:
         np_dtype = "uint16" if wl.dtype in ("bf16", "f16") else "int32" if wl.dtype == "int32" else "float32"
         result["cpu_baseline"] = cpu_baseline(wl.jsons, wl.world, wl.n, np_dtype, wl.name + ": the same graphs", args.cpu_reps)
@@ -552,7 +570,6 @@ def brief_inplace(args, wl: Workload, dev) -> dict:
         return out
     finally:
         eng.close()
-        torch.cuda.empty_cache()
 
 
 def brief_c4(args, dev, nbytes: int) -> list:
@@ -614,21 +631,26 @@ def brief_c4(args, dev, nbytes: int) -> list:
         finally:
             eng.close()
             del x, outs
-            torch.cuda.empty_cache()
+            release_between_equal_sizes()     # the allgather's tensors have the reduce_scatter's sizes, swapped
     return out
 
 
 def other_configs(args, dev) -> list:
     """Configurations 3, 5 (both element types) and the 512 MB pair of 4, each verified and timed like
     its own `--config` run, for the default run's JSON line."""
-    rows = []
     saved = args.c5_dtype
     try:
-        rows.append(brief_inplace(args, workload_c3(args, dev), dev))
+        # the 512 MB pair first: its tensors have the size of the headline's, whose blocks it takes over
+        c4 = brief_c4(args, dev, 512 << 20)
+        release_cached_memory()
+        rows = [brief_inplace(args, workload_c3(args, dev), dev)]
+        release_cached_memory()
         for dt in ("int32", "float32"):
             args.c5_dtype = dt
             rows.append(brief_inplace(args, workload_c5(args, dev), dev))
-        rows.extend(brief_c4(args, dev, 512 << 20))
+            release_between_equal_sizes()
+        release_cached_memory()
+        rows.extend(c4)
     finally:
         args.c5_dtype = saved
     return rows

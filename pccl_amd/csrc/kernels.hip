@@ -1463,38 +1463,32 @@ __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs
     }
 }
 
-// The same runner for plans that store little (a reduce_scatter: R chunks in, one out): a write phase
-// per sweep would be too short to be worth a meeting and without meetings the stores sprinkle the
-// reads, so KK sweeps are read before their sums are written, with meetings around the longer write
-// phase (bare kernels of this traffic, 8 x 512 MiB in and 8 x 64 MiB out: 0.788 of peak without
-// meetings, 0.804 with a write phase per sweep, 0.865 per two sweeps, 0.868 per three).  Chains as
-// slabs only; a kernel of its own, so that the one above keeps the code it was tuned with.
+// The same runner with KK sweeps read before their sums are written: the phases are KK times as long
+// and the meetings KK times fewer.  Worth most for plans that store little (a reduce_scatter: R
+// chunks in, one out), where a write phase per sweep would be too short to be worth a meeting and
+// without meetings the stores sprinkle the reads (bare kernels of this traffic, 8 x 512 MiB in and
+// 8 x 64 MiB out: 0.788 of peak without meetings, 0.804 with a write phase per sweep, 0.865 per two
+// sweeps, 0.868 per three); an allreduce in place on 8 ranks gains half a point to two points.
+// Chains read and written as slabs only; a kernel of its own, so that the one above keeps the code
+// it was tuned with.
 template <int DT, int T, int V, int S, int GR, int KK>
 __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtrs ptrs) {
     extern __shared__ u32x4 lds[];
     __shared__ int s_flag;
     static_assert((size_t)S * T * 16 <= 159u * 1024, "the fetch ring must fit a CU's LDS");
-    constexpr int LAY = 0;
-    constexpr bool TREE = false;
-    static_assert(KK >= 1 && KK * V <= 32, "the sums of KK sweeps stay in registers");
+    static_assert(KK >= 1 && KK <= 2 && KK * V <= 32, "the sums of KK sweeps stay in registers; one call of read_sweep per sweep below");
     constexpr int ES = ElemBytes<DT>::value;
     constexpr int VE = 16 / ES;
     constexpr int64_t CHUNK_V = (int64_t)T * V;
-    constexpr int VS = LAY == 1 ? 64 * 16 : T * 16;          // bytes between a thread's consecutive vectors while it reads
-    constexpr int WVS = LAY >= 1 ? 64 * 16 : T * 16;         // ... and while it writes
+    constexpr int VS = T * 16;                   // bytes between a thread's consecutive vectors: the chunk as V slabs
     const int tid = threadIdx.x;
     const int G = gridDim.x;
     // workgroup b runs on XCD b % 8: every XCD takes a contiguous eighth of each sweep
     const int place = (G & 7) == 0 ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
-    // thread's first vector inside a chunk: each wave a contiguous V KiB, or the chunk as V slabs of T vectors
-    const uint32_t wavec = (uint32_t)(tid >> 6) * V * 64 + (tid & 63);
-    const uint32_t toff = (LAY == 1 ? wavec : (uint32_t)tid) * 16;
-    const uint32_t wtoff = (LAY >= 1 ? wavec : (uint32_t)tid) * 16;
+    const uint32_t toff = (uint32_t)tid * 16;
     const int64_t sweeps = (L.total_chunks + G - 1) / G;
     bool meet = L.barriers != 0;
     int gen = 0;
-    // KK sweeps are read before their sums are written (KK > 1: plans that store little, where a write
-    // phase per sweep would be too short to be worth a meeting)
     for (int64_t it0 = 0; it0 < sweeps; it0 += KK) {
         u32x4 acc[KK][V];
         DevChainSegment seg[KK];
@@ -1511,79 +1505,43 @@ __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtr
             seg[k] = DevChainSegment{};
             vbase[k] = 0;
             whole[k] = false;
-            if (live) {
-                int lo = 0;
-                if (L.seg_chunks > 0) {
-                    const uint32_t per = (uint32_t)L.seg_chunks;
-                    lo = (per & (per - 1)) == 0 ? (int)((uint32_t)chunk >> __builtin_ctz(per)) : (int)((uint32_t)chunk / per);
-                } else {
-                    int hi = L.num_segs;
-                    while (hi - lo > 1) {
-                        const int mid = (lo + hi) >> 1;
-                        if (as_const(L.segs)[mid].first_chunk <= chunk) lo = mid; else hi = mid;
-                    }
-                }
-                seg[k] = load_const(L.segs + lo);
-                vbase[k] = seg[k].first_vec + (chunk - seg[k].first_chunk) * CHUNK_V;
-                whole[k] = vbase[k] * VE >= seg[k].start && (vbase[k] + CHUNK_V) * VE <= seg[k].end;
-                const PCCL_CONST int32_t* srcs = as_const(L.srcs) + seg[k].src_start;   // dwords: uniform reads become scalar loads
-                if (whole[k]) {
-                    bool done = false;
-                    if constexpr (TREE) {
-                        if (seg[k].tree_depth > 1) { tree_read<DT, T, V, S, VS>(acc[k], srcs, seg[k].n_src, seg[k].tree_depth, ptrs, lds, vbase[k] * 16, toff, tid); done = true; }
-                    }
-                    if (done) {}
-                    else if (seg[k].redop == PCCL_SUM) chain_read<DT, PCCL_SUM, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
-                    else if (seg[k].redop == PCCL_MAX) chain_read<DT, PCCL_MAX, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
-                    else chain_read<DT, PCCL_MIN, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
-                } else {
-                    // a chunk that the segment's ends cut: vector by vector, loads and stores together
-                    for (int64_t j = tid; j < CHUNK_V; j += T) {
-                        const int64_t vec = vbase[k] + j;
-                        int64_t e0 = vec * VE, e1 = e0 + VE;
-                        if (e0 < seg[k].start) e0 = seg[k].start;
-                        if (e1 > seg[k].end) e1 = seg[k].end;
-                        if (e0 >= e1) continue;
-                        u32x4 x = ldv(ptrs.p[kMaxR + srcs[0]] + vec * 16);
-                        if (!TREE || seg[k].tree_depth == 0) {
-                            for (int i = 1; i < seg[k].n_src; ++i) x = vec_op<DT>(ldv(ptrs.p[kMaxR + srcs[i]] + vec * 16), x, seg[k].redop);
-                        } else {
-                            u32x4 parked[6];
-                            for (int i = 0; i < seg[k].n_src; ++i) {
-                                u32x4 y = i == 0 ? x : ldv(ptrs.p[kMaxR + srcs[i]] + vec * 16);
-                                bool placed = false;
-#pragma unroll
-                                for (int lvl = 0; lvl < 6; ++lvl) {
-                                    if (!placed && lvl < seg[k].tree_depth) {
-                                        if (i >> lvl & 1) y = vec_op<DT>(parked[lvl], y, seg[k].redop);
-                                        else { parked[lvl] = y; placed = true; }
-                                    }
-                                }
-                                if (!placed) x = y;
-                            }
-                        }
-                        for (uint64_t m = seg[k].store_mask; m; m &= m - 1)
-                            store_vector_part<DT>(ptrs.p[__builtin_ctzll(m)] + vec * 16, x, (int)(e0 - vec * VE), (int)(e1 - vec * VE));
-                    }
+            if (!live) return;
+            int lo = 0;
+            if (L.seg_chunks > 0) {
+                const uint32_t per = (uint32_t)L.seg_chunks;
+                lo = (per & (per - 1)) == 0 ? (int)((uint32_t)chunk >> __builtin_ctz(per)) : (int)((uint32_t)chunk / per);
+            } else {
+                int hi = L.num_segs;
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (as_const(L.segs)[mid].first_chunk <= chunk) lo = mid; else hi = mid;
                 }
             }
-            if constexpr (LAY == 2) {
-                if (whole[k]) {                 // uniform over the workgroup: the barriers are reached by all or by none
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                    __syncthreads();            // every wave has consumed its ring slots: the space is free
-#pragma unroll
-                    for (int v = 0; v < V; ++v) lds[v * T + tid] = acc[k][v];       // position v T + t of the chunk
-                    __syncthreads();
-#pragma unroll
-                    for (int v = 0; v < V; ++v) acc[k][v] = lds[wavec + v * 64];
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    __syncthreads();            // all have their sums before the next fetches land here
+            seg[k] = load_const(L.segs + lo);
+            vbase[k] = seg[k].first_vec + (chunk - seg[k].first_chunk) * CHUNK_V;
+            whole[k] = vbase[k] * VE >= seg[k].start && (vbase[k] + CHUNK_V) * VE <= seg[k].end;
+            const PCCL_CONST int32_t* srcs = as_const(L.srcs) + seg[k].src_start;   // dwords: uniform reads become scalar loads
+            if (whole[k]) {
+                if (seg[k].redop == PCCL_SUM) chain_read<DT, PCCL_SUM, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
+                else if (seg[k].redop == PCCL_MAX) chain_read<DT, PCCL_MAX, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
+                else chain_read<DT, PCCL_MIN, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
+            } else {
+                // a chunk that the segment's ends cut: vector by vector, loads and stores together
+                for (int64_t j = tid; j < CHUNK_V; j += T) {
+                    const int64_t vec = vbase[k] + j;
+                    int64_t e0 = vec * VE, e1 = e0 + VE;
+                    if (e0 < seg[k].start) e0 = seg[k].start;
+                    if (e1 > seg[k].end) e1 = seg[k].end;
+                    if (e0 >= e1) continue;
+                    u32x4 x = ldv(ptrs.p[kMaxR + srcs[0]] + vec * 16);
+                    for (int i = 1; i < seg[k].n_src; ++i) x = vec_op<DT>(ldv(ptrs.p[kMaxR + srcs[i]] + vec * 16), x, seg[k].redop);
+                    for (uint64_t m = seg[k].store_mask; m; m &= m - 1)
+                        store_vector_part<DT>(ptrs.p[__builtin_ctzll(m)] + vec * 16, x, (int)(e0 - vec * VE), (int)(e1 - vec * VE));
                 }
             }
         };
         read_sweep(std::integral_constant<int, 0>{});
         if constexpr (KK > 1) read_sweep(std::integral_constant<int, 1>{});
-        static_assert(KK <= 2, "one call of read_sweep per sweep of a group");
         if (meet) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
@@ -1597,7 +1555,7 @@ __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtr
                 for (uint64_t m = seg[k].store_mask; m; m &= m - 1) {
                     char* const dst = ptrs.p[__builtin_ctzll(m)] + vbase[k] * 16;
 #pragma unroll
-                    for (int v = 0; v < V; ++v) stv_nt_s(dst, wtoff + v * WVS, acc[k][v]);
+                    for (int v = 0; v < V; ++v) stv_nt_s(dst, toff + v * VS, acc[k][v]);
                 }
             }
         };
