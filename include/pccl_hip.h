@@ -250,7 +250,8 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * the output tensors directly instead of staging through the engine's rank buffers);
  * "lds_slots" = "1" | "0" (column runner keeps values it re-reads in per-thread LDS slots, so each
  * rank buffer is read and written at most once per position; "0" re-reads them through memory);
- * "slot_threads" = 0 | 64 | 128 | 256 | 512 | 1024 (workgroup size of that runner, 0 = from the rank count);
+ * "slot_threads" = 0 | 64 | 128 | 256 | 512 | 1024 (workgroup size of that runner, 0 = from the rank count
+ * and the plan's traffic);
  * "slot_vecs" = 0 | 1 | 2 | 4 (16-byte vectors per thread of that runner: a workgroup's tile is
  * slot_threads x slot_vecs vectors of every rank; 0 = from the rank count); "slot_lds_kib" = 0..160
  * (least LDS a workgroup of that runner asks for, which bounds the workgroups per CU; 0 = chosen);
@@ -287,7 +288,10 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
  * (rank, id) order, empty when there are none; PCCL_ERR_INVALID if `cap` is too small for the text -, and
  * "runner_inplace:NAME" / "runner_staged:NAME": the kernel an in-place / staged execution of operation
  * NAME would launch now - "phased_kernel", "column_slot_kernel", "column_kernel", "level_kernel",
- * "persistent_kernel", "gather_kernel", or "staging + ..." - which links the operation): what the
+ * "persistent_kernel", "gather_kernel", or "staging + ..." - which links the operation; and
+ * "slot_shape:NAME": the slot runner's workgroup for operation NAME as "threads x vectors", e.g.
+ * "256x2", or "0x0" if its column plan does not run there - chosen from the rank count, and larger
+ * for plans that store at least four times what they load): what the
  * environment switches PCCL_NUM_BLOCKS / PCCL_DISABLE_FUSED / PCCL_TRACE_RANGES left in a new context
  * can be read back here.  No counterpart in the reference. */
 int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t cap);

@@ -614,9 +614,24 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
         for (const ColInstr& in : P.col_instrs)
             if ((in.a_src == SRC_MEM && !in.a_first) || (in.b_src == SRC_MEM && !in.b_first) || (in.store & STORE_KIND) == 1) reads_back = true;
         e.slot_threads = 0; e.slot_vecs = 1; e.slot_lds_bytes = 0;
-        if (ctx->lds_slots && (ctx->slot_threads > 0 || reads_back || ctx->R <= 16)) {
+        // Plans that mostly write (an allgather: one chunk in, R out; both the in-place and the staged
+        // form) want larger workgroups whose waves each store whole tiles of a rank.  Measured on
+        // MI355X, fp16 ring allgather as a staged call, fraction of the 8 TB/s: 32 ranks x 8 / 24 /
+        // 96 MiB on the slot runner with 256 threads 0.715 / 0.778 / 0.670 against 0.694 / 0.715 /
+        // 0.650 for the register runner; 8 ranks x 256 / 512 MiB with 1024 threads x 1 vector 0.752 /
+        // 0.759 against 0.735 / 0.740 for 256 x 2 - below that size the smaller tiles win (128 MiB
+        // 0.729 against 0.752, 32 MiB 0.64 against 0.70), and so they do at 16 ranks up to 16 MiB.
+        const bool mostly_writes = P.slot_store_bytes >= 4 * P.slot_load_bytes && P.slot_load_bytes > 0 &&
+                                   (P.direct_segs.empty() || P.direct_slot_store_bytes >= 4 * P.direct_slot_load_bytes);
+        const bool automatic = ctx->slot_threads == 0 && ctx->slot_vecs == 0 && ctx->slot_direct;
+        const int64_t rank_bytes = P.tensor_elems * elem_size(P.dtype);
+        if (ctx->lds_slots && (ctx->slot_threads > 0 || reads_back || ctx->R <= 16 || (mostly_writes && ctx->R <= 32))) {
             const int R = ctx->R;
-            const SlotShape sh = slot_shape(R, ctx->slot_threads, ctx->slot_vecs, ctx->slot_direct);
+            SlotShape sh = slot_shape(R, ctx->slot_threads, ctx->slot_vecs, ctx->slot_direct);
+            if (automatic && mostly_writes) {
+                if (R > 16) sh = slot_shape(R, 256, 1, true);
+                else if (R > 4 && R <= 8 && rank_bytes >= ((int64_t)256 << 20)) sh = slot_shape(R, 1024, 1, true);
+            }
             const std::string why = slot_shape_error(R, sh);
             if (!why.empty()) throw Error{PCCL_ERR_INVALID, why};
             const int threads = sh.threads, vecs = sh.vecs;
@@ -1471,6 +1486,15 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
             else if (!column_ok || !P.position_aligned) v = ctx->mode == Mode::Persistent ? "persistent_kernel" : "level_kernel";
             else if (wants_phased(ctx, e, staged)) v = "phased_kernel";
             else v = e.slot_threads > 0 ? "column_slot_kernel" : "column_kernel";
+        }
+        else if (k.rfind("slot_shape:", 0) == 0) {
+            // the slot runner's workgroup for that operation as linked now: "threads x vectors", "0x0" if
+            // its column plan runs on the register runner or it has none
+            OpEntry& e = find_entry(ctx, k.c_str() + 11);
+            HIP_TRY(hipSetDevice(ctx->device));
+            refresh_link(ctx, e, nullptr, false);
+            link_entry(ctx, e);
+            v = e.slot_threads > 0 ? std::to_string(e.slot_threads) + "x" + std::to_string(e.slot_vecs) : "0x0";
         }
         else return fail(PCCL_ERR_INVALID, "unknown option '" + k + "'");
         if (v.size() + 1 > cap) return fail(PCCL_ERR_INVALID, "value buffer too small");

@@ -223,6 +223,55 @@ def test_slot_runner_workgroup_shapes(engine_factory, seed):
             eng.set_option(key, val)
 
 
+@pytest.mark.parametrize("world", [8, 24, 32])
+def test_plans_that_mostly_write_take_larger_workgroups(engine_factory, world):
+    """An allgather stores R times what it loads: up to 32 ranks it runs on the slot runner, with 256
+    threads beyond 16 ranks (the register runner otherwise takes programs of that many ranks that
+    read nothing back), and on 5 to 8 ranks with 1024 threads from 256 MiB per rank on.  An
+    allreduce of the same ranks keeps the shape chosen from the rank count.  Results against the
+    oracle at sizes with cut tiles, staged and in place."""
+    n = world * (1000 + 37)
+    jsons = graph_jsons("ring", "build_allgather", world, n, "float16", "sm", 1)
+    chunk = n // world
+    x = seeded_inputs("randn", world, chunk, "float16", seed=world)
+    want = oracle_buffers(jsons, x, "float16", buffer_elems=n, place=lambda r: r * chunk)
+    eng = engine_factory(world)
+    for r, j in enumerate(jsons):
+        eng.register_operation_json("ag", j, r)
+    shape = eng.get_option("slot_shape:ag")
+    assert shape == ("256x2" if world == 8 else "256x1"), shape
+    assert eng.get_option("runner_staged:ag") == "column_slot_kernel"
+    outs = [torch.zeros(n, dtype=torch.float16, device="cuda") for _ in range(world)]
+    eng.execute_operation("ag", [t.cuda() for t in x], outs)
+    for r in range(world):
+        assert bits_equal(outs[r], want[r]), f"staged, rank {r}: {mismatch_report(outs[r], want[r])}"
+    bufs = []
+    for r in range(world):
+        b = torch.zeros(n, dtype=torch.float16)
+        b[r * chunk:(r + 1) * chunk] = x[r]
+        bufs.append(b.cuda())
+    eng.execute_inplace("ag", bufs, sync=True)
+    for r in range(world):
+        assert bits_equal(bufs[r], want[r]), f"in place, rank {r}: {mismatch_report(bufs[r], want[r])}"
+    # the same ranks, an allreduce: as many loads as stores
+    ar = graph_jsons("ring", "build_allreduce", world, n, "float16", "sm", 1)
+    for r, j in enumerate(ar):
+        eng.register_operation_json("ar", j, r)
+    assert eng.get_option("slot_shape:ar") == ("256x2" if world == 8 else "0x0")
+    if world == 8:
+        # the size from which 1024 threads pay is too large for the oracle: only the choice is checked here
+        # (the full-size configuration tests run it)
+        big = graph_jsons("ring", "build_allgather", world, 1 << 27, "float16", "sm", 1)
+        for r, j in enumerate(big):
+            eng.register_operation_json("ag_big", j, r)
+        assert eng.get_option("slot_shape:ag_big") == "1024x1"
+        eng.set_option("slot_vecs", 2)                       # a shape that is asked for is kept
+        try:
+            assert eng.get_option("slot_shape:ag_big") == "256x2"
+        finally:
+            eng.set_option("slot_vecs", 0)
+
+
 def test_slot_shape_options_are_checked_where_they_are_set(engine_factory):
     """A workgroup shape that the LDS cannot hold is refused by set_option itself, against the shape
     linking would choose with the other option left automatic, and the refused value is not kept:
