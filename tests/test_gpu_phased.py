@@ -163,6 +163,40 @@ def test_more_workgroups_than_fit_at_once(engine_factory):
         eng.set_option("phased", -1); eng.set_option("num_blocks", 0); eng.set_option("phased_timeout_us", 1000)
 
 
+def test_two_launches_of_one_operation_on_two_streams(engine_factory):
+    """In-place calls on different tensors may overlap on the GPU.  Two phased launches of one
+    operation then share its meeting block and lose their phases, which costs time and nothing else:
+    both results are exact, and the next launch on its own meets normally again."""
+    world, n = 8, 600 * CHUNK_VECS * 8                # bf16: 600 chunks of every rank, more than two sweeps
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 1)
+    xa = seeded_inputs("randn", world, n, "bfloat16", seed=21)
+    xb = seeded_inputs("randn", world, n, "bfloat16", seed=22)
+    want_a, want_b = oracle_buffers(jsons, xa, "bfloat16"), oracle_buffers(jsons, xb, "bfloat16")
+    eng = engine_factory(world)
+    _register(eng, "ph_two", jsons)
+    eng.set_option("phased", 1)
+    try:
+        a = [t.cuda() for t in xa]
+        eng.execute_inplace("ph_two", a, sync=True)          # linked and uploaded
+        _check(a, want_a, "alone")
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        for rep in range(3):
+            a, b = [t.cuda() for t in xa], [t.cuda() for t in xb]
+            torch.cuda.synchronize()
+            with torch.cuda.stream(s1):
+                eng.execute_inplace("ph_two", a)
+            with torch.cuda.stream(s2):
+                eng.execute_inplace("ph_two", b)
+            torch.cuda.synchronize()
+            _check(a, want_a, f"first of two, repetition {rep}")
+            _check(b, want_b, f"second of two, repetition {rep}")
+        a = [t.cuda() for t in xa]
+        eng.execute_inplace("ph_two", a, sync=True)
+        _check(a, want_a, "alone again")
+    finally:
+        eng.set_option("phased", -1)
+
+
 def test_phased_launches_recorded_into_a_graph(engine_factory):
     """A phased launch is one kernel and needs no set-up per launch (the meeting block cleans itself),
     so it can be recorded and replayed; every replay against the oracle, eager work in between."""
