@@ -281,7 +281,9 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * csrc/plugins/cuda/cuda_device.cc:313-319: "d2d_input_copy", "execute", "d2d_output_copy", and
  * inside "execute" "fused_kernel" for the column runner or "executor_kernel" for the level and
  * persistent runners; the marker library is loaded at run time and PCCL_ERR_UNSUPPORTED is returned
- * if there is none; the environment variable PCCL_TRACE_RANGES=1 sets it for new contexts). */
+ * if there is none; the environment variable PCCL_TRACE_RANGES=1 sets it for new contexts).
+ * Every value except "mode" is a whole number written as text; anything else ("on", "4k"), a value out
+ * of the option's range and an unknown key return PCCL_ERR_INVALID and leave the option as it was. */
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
 /* The current value of an option as text (the keys of pccl_hip_set_option, "num_vranks", "signals" -
  * the semaphores that executions so far have left above zero, as "rank:id=count" joined by commas in

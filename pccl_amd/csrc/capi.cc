@@ -2,6 +2,8 @@
 #include <dlfcn.h>
 #include <hip/hip_runtime_api.h>
 
+#include <cerrno>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <atomic>
@@ -1333,6 +1335,21 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank, c
     return guarded([&] { return register_graph(ctx, name, vrank, graph_from_triggers(triggers, meta, n, collective_type)); });
 }
 
+// An option value that has to be a whole number: "on", "True" or "4x" are refused, not read as 0 or 4.
+static long long whole_number(const std::string& key, const char* value) {
+    errno = 0;
+    char* end = nullptr;
+    const long long x = std::strtoll(value, &end, 10);
+    if (end == value || *end != '\0' || errno != 0)
+        throw Error{PCCL_ERR_INVALID, "option '" + key + "' takes a whole number, got '" + value + "'"};
+    return x;
+}
+static int int_value(const std::string& key, const char* value) {
+    const long long x = whole_number(key, value);
+    if (x < INT32_MIN || x > INT32_MAX) throw Error{PCCL_ERR_INVALID, "option '" + key + "': " + value + " is out of range"};
+    return (int)x;
+}
+
 int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
     return guarded([&] {
         if (!ctx || !key || !value) return fail(PCCL_ERR_INVALID, "null argument");
@@ -1345,17 +1362,17 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             else if (v == "stepwise") ctx->mode = Mode::Stepwise;
             else if (v == "persistent") ctx->mode = Mode::Persistent;
             else return fail(PCCL_ERR_INVALID, "mode must be auto, column, stepwise or persistent");
-        } else if (k == "num_blocks") ctx->num_blocks = std::atoi(value);
-        else if (k == "timing") ctx->timing = std::atoi(value) != 0;
+        } else if (k == "num_blocks") ctx->num_blocks = int_value(k, value);
+        else if (k == "timing") ctx->timing = int_value(k, value) != 0;
         else if (k == "trace_ranges") {
-            ctx->trace_ranges = std::atoi(value) != 0;
+            ctx->trace_ranges = int_value(k, value) != 0;
             if (ctx->trace_ranges && !marker_api().push) { ctx->trace_ranges = false; return fail(PCCL_ERR_UNSUPPORTED, "trace_ranges: no roctx marker library could be loaded"); }
         }
-        else if (k == "fuse_staging") ctx->fuse_staging = std::atoi(value) != 0;
-        else if (k == "wait_timeout_ms") { ctx->wait_timeout_ms = std::atoi(value); if (ctx->wait_timeout_ms < 0) ctx->wait_timeout_ms = 0; }   // 0: give up on the first predecessor that is not ready
+        else if (k == "fuse_staging") ctx->fuse_staging = int_value(k, value) != 0;
+        else if (k == "wait_timeout_ms") { ctx->wait_timeout_ms = int_value(k, value); if (ctx->wait_timeout_ms < 0) ctx->wait_timeout_ms = 0; }   // 0: give up on the first predecessor that is not ready
         else if (k == "test_host_epoch_limit" || k == "test_graph_epoch_limit") {
             // for tests: bring the point where the persistent runner's launch numbers wrap within reach
-            const long long x = std::atoll(value);
+            const long long x = whole_number(k, value);
             if (k == "test_host_epoch_limit") {
                 if (x < 2 || x > kHostEpochLimit) return fail(PCCL_ERR_INVALID, "test_host_epoch_limit must be 2 .. " + std::to_string(kHostEpochLimit));
                 ctx->host_epoch_limit = (int32_t)x;
@@ -1364,46 +1381,46 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
                 ctx->graph_epoch_limit = (int32_t)x;
             }
         }
-        else if (k == "check_races") { ctx->check_races = std::atoi(value) != 0; relink = true; }
+        else if (k == "check_races") { ctx->check_races = int_value(k, value) != 0; relink = true; }
         else if (k == "vecs_per_thread") {
-            int u = std::atoi(value);
+            int u = int_value(k, value);
             if (u != 1 && u != 2 && u != 4) return fail(PCCL_ERR_INVALID, "vecs_per_thread must be 1, 2 or 4");
             ctx->vecs_per_thread = u; relink = true;
         }
         else if (k == "slot_store_waves") {
-            const int v = std::atoi(value);
+            const int v = int_value(k, value);
             if (v < -1 || v > 1) return fail(PCCL_ERR_INVALID, "slot_store_waves must be -1 (automatic), 0 or 1");
             ctx->slot_store_waves = v;
         }
-        else if (k == "level_graph") ctx->level_graph = std::atoi(value) != 0;
+        else if (k == "level_graph") ctx->level_graph = int_value(k, value) != 0;
         else if (k == "phased") {
-            const int x = std::atoi(value);
+            const int x = int_value(k, value);
             if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased must be -1 (automatic), 0 or 1");
             ctx->phased = x;
         }
         else if (k == "phased_shape") {
-            const int x = std::atoi(value);
+            const int x = int_value(k, value);
             if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased_shape must be -1 (automatic), 0 (512 threads x 16 vectors) or 1 (256 x 32)");
             ctx->phased_shape = x;
         }
         else if (k == "phased_sweeps") {
-            const int x = std::atoi(value);
+            const int x = int_value(k, value);
             if (x != -1 && x != 1 && x != 2) return fail(PCCL_ERR_INVALID, "phased_sweeps must be -1 (automatic), 1 or 2");
             ctx->phased_sweeps = x;
         }
         else if (k == "phased_exchange") {
-            const int x = std::atoi(value);
+            const int x = int_value(k, value);
             if (x < -1 || x > 1) return fail(PCCL_ERR_INVALID, "phased_exchange must be -1 (automatic), 0 or 1");
             ctx->phased_exchange = x;
         }
-        else if (k == "phased_barriers") ctx->phased_barriers = std::atoi(value) != 0;
-        else if (k == "phased_timeout_us") { ctx->phased_timeout_us = std::atoi(value); if (ctx->phased_timeout_us < 0) ctx->phased_timeout_us = 0; }
-        else if (k == "lds_slots") { ctx->lds_slots = std::atoi(value) != 0; relink = true; }
+        else if (k == "phased_barriers") ctx->phased_barriers = int_value(k, value) != 0;
+        else if (k == "phased_timeout_us") { ctx->phased_timeout_us = int_value(k, value); if (ctx->phased_timeout_us < 0) ctx->phased_timeout_us = 0; }
+        else if (k == "lds_slots") { ctx->lds_slots = int_value(k, value) != 0; relink = true; }
         else if (k == "slot_direct" || k == "slot_threads" || k == "slot_vecs") {
             // checked against the shape linking would choose with the new value in place
             int threads = ctx->slot_threads, vecs = ctx->slot_vecs;
             bool direct = ctx->slot_direct;
-            const int x = std::atoi(value);
+            const int x = int_value(k, value);
             if (k == "slot_threads") {
                 if (x != 0 && x != 64 && x != 128 && x != 256 && x != 512 && x != 1024) return fail(PCCL_ERR_INVALID, "slot_threads must be 0 (automatic), 64, 128, 256, 512 or 1024");
                 threads = x;
@@ -1417,12 +1434,12 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value) {
             ctx->slot_threads = threads; ctx->slot_vecs = vecs; ctx->slot_direct = direct; relink = true;
         }
         else if (k == "slot_lds_kib") {
-            int b = std::atoi(value);
+            int b = int_value(k, value);
             if (b < 0 || b > 160) return fail(PCCL_ERR_INVALID, "slot_lds_kib must be 0 (automatic) to 160");
             ctx->slot_lds_kib = b; relink = true;
         }
         else if (k == "step_tile_bytes") {
-            int64_t b = std::atoll(value);
+            int64_t b = whole_number(k, value);
             if (b < 0 || b % 4096) return fail(PCCL_ERR_INVALID, "step_tile_bytes must be 0 (automatic) or a positive multiple of 4096");
             ctx->step_tile_bytes = b; relink = true;
         } else return fail(PCCL_ERR_INVALID, "unknown option '" + k + "'");

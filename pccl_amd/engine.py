@@ -99,6 +99,10 @@ class Engine:
         return self._L.pccl_hip_last_error().decode(errors="replace")
 
     def set_option(self, key: str, value) -> None:
+        """Option `key` (see pccl_hip_set_option in include/pccl_hip.h) takes text or a whole number;
+        True and False are passed as 1 and 0."""
+        if isinstance(value, bool):
+            value = int(value)
         _lib.check(self._L.pccl_hip_set_option(self._h, key.encode(), str(value).encode()))
 
     def get_option(self, key: str) -> str:

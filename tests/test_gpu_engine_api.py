@@ -35,7 +35,7 @@ def test_reference_style_per_rank_flow(engine_factory, tmp_path):
     torch.cuda.synchronize()
     for r in range(world):
         assert (out[r] != world * (world + 1) / 2).sum().item() == 0
-    eng.reset_signals("test_allreduce")            # a no-op here, must not fail
+    eng.reset_signals("test_allreduce")            # no counts are left here: nothing to clear, must not fail
     # a second round reuses the registration; the last rank may use the synchronising form
     for r in range(world - 1):
         eng.rank(r).execute_operation_async("test_allreduce", inp[r], out[r])
@@ -461,3 +461,62 @@ def test_tensors_of_the_wrong_element_size_are_refused(engine_factory):
     as_int16 = [t.view(torch.int16) for t in right]          # same element size: the bytes are what counts
     eng.execute_inplace("ar_bf16_only", as_int16, sync=True)
     assert torch.all(right[1].float() == 4)
+
+
+OPTIONS = {   # key: (values that are taken and read back as written, values that are refused)
+    "mode": (["column", "stepwise", "persistent", "auto"], ["fast", ""]),
+    "num_blocks": ([7, 0], ["many"]),
+    "timing": ([1, 0], ["on"]),
+    "fuse_staging": ([0, 1], ["yes"]),
+    "wait_timeout_ms": ([5, 2000], ["1s"]),
+    "check_races": ([0, 1], ["no"]),
+    "vecs_per_thread": ([2, 4, 1], [3, 0, "two"]),
+    "slot_direct": ([0, 1], ["direct"]),
+    "slot_store_waves": ([0, 1, -1], [2, -2]),
+    "level_graph": ([1, 0], ["graph"]),
+    "phased": ([0, 1, -1], [2, -2, "always"]),
+    "phased_shape": ([0, 1, -1], [2, 4]),
+    "phased_exchange": ([0, 1, -1], [2]),
+    "phased_sweeps": ([1, 2, -1], [0, 3, "two"]),
+    "phased_barriers": ([0, 1], ["x"]),
+    "phased_timeout_us": ([50, 1000], ["1ms"]),
+    "lds_slots": ([0, 1], ["lds"]),
+    "slot_threads": ([64, 512, 0], [100, 2048]),
+    "slot_vecs": ([2, 1, 0], [3, 8]),
+    "slot_lds_kib": ([96, 0], [161, -1, "64k"]),
+    "step_tile_bytes": ([8192, 0], [1000, -4096, "4k"]),
+}
+
+
+def test_every_option_reads_back_and_refuses_what_it_cannot_take(engine_factory):
+    """set_option / get_option over every key of the header: a value that is taken reads back as it
+    was written, a value that is refused (out of range, not a whole number) raises with the key's name
+    or its range in the message and leaves the option as it was, True and False arrive as 1 and 0, and
+    an unknown key is an error for both calls."""
+    eng = engine_factory(4)
+    for key, (good, bad) in OPTIONS.items():
+        start = eng.get_option(key)
+        try:
+            for v in good:
+                eng.set_option(key, v)
+                assert eng.get_option(key) == str(v), key
+            kept = eng.get_option(key)
+            for v in bad:
+                with pytest.raises(PcclError) as e:
+                    eng.set_option(key, v)
+                assert e.value.code == ERR_INVALID, (key, v)
+                assert key in str(e.value) or "must be" in str(e.value), str(e.value)
+                assert eng.get_option(key) == kept, (key, v)
+        finally:
+            eng.set_option(key, start)
+    eng.set_option("timing", True)
+    assert eng.get_option("timing") == "1"
+    eng.set_option("timing", False)
+    assert eng.get_option("timing") == "0"
+    for call in (lambda: eng.set_option("no_such_option", 1), lambda: eng.get_option("no_such_option")):
+        with pytest.raises(PcclError, match="unknown option") as e:
+            call()
+        assert e.value.code == ERR_INVALID
+    assert eng.get_option("num_vranks") == "4"
+    with pytest.raises(PcclError, match="Unknown operation"):
+        eng.get_option("slot_shape:nobody")
