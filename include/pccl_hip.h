@@ -269,8 +269,8 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * and write with each wave on 32 KiB in a row, the sums changing hands through LDS in between; 0: each
  * wave on 32 KiB in a row for reads as well); "phased_sweeps" = "-1" | "1" | "2" (sweeps the 512 x 16
  * shape reads before it writes their sums: two make the phases longer and the meetings fewer; -1: two
- * for plans on up to 8 ranks from two sweeps on, and for plans that load four times what they store
- * from four sweeps on, which run without meetings below that); "phased_barriers" = "1" | "0" (0: no
+ * from two sweeps on for plans on up to 8 ranks and for plans that load four times what they store,
+ * which run without meetings below that); "phased_barriers" = "1" | "0" (0: no
  * meetings, for comparison); "phased_timeout_us" (how long a workgroup waits at a meeting before the
  * launch goes on unsynchronised: meetings order nothing; the environment variable PCCL_PHASED sets
  * "phased" for new contexts);

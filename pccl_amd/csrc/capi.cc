@@ -911,19 +911,21 @@ int launch_phased_plan(pccl_hip_ctx* ctx, OpEntry& e, bool direct, const RankPtr
     if (ctx->phased_exchange != 0 && L.shape == 1) L.shape = 3;
     L.num_blocks = ctx->num_blocks;
     // a plan that mostly reads (a reduce_scatter: R chunks in, one out) has write phases too short to be
-    // worth a meeting per sweep (8 x 64 MB fp16: 89 us without, 94 us with).  It reads two sweeps and
-    // then writes both (shape 4: bare kernels of that traffic, 8 x 512 MiB in, 8 x 64 MiB out, 0.788 of
-    // peak without meetings, 0.804 with one write phase per sweep, 0.865 per two sweeps, 0.868 per three)
+    // worth a meeting per sweep (8 x 64 MB fp16: 89 us without, 94 us with).  It reads two sweeps in one
+    // fetch stream and then writes both (shape 4: bare kernels of that traffic, 8 x 512 MiB in, 8 x
+    // 64 MiB out, 0.788 of peak without meetings, 0.804 with one write phase per sweep, 0.865 per two
+    // sweeps, 0.868 per three), from two sweeps on; below, it runs without meetings
     const int64_t loads = direct ? P.direct_slot_load_bytes : P.slot_load_bytes;
     const int64_t stores = direct ? P.direct_slot_store_bytes : P.slot_store_bytes;
     const bool mostly_reads = loads >= 4 * stores;
-    // (from four sweeps on: 8-rank fp16 reduce_scatter 512 / 256 MB per rank 0.806 -> 0.846 / 0.830 -> 0.848 of
-    // peak, 64 / 32 / 16 MB - two sweeps, one, half a one - 0.837 -> 0.827 / 0.826 -> 0.759 / 0.631 -> 0.563).
-    // The 512 x 16 shape of the other chains (up to 8 ranks) gains from it as well, from two sweeps on:
-    // fewer, longer phases (8-rank bf16 ring in place, 64 / 128 / 256 / 512 MiB per rank: 0.764 -> 0.787,
-    // 0.783 -> 0.786, 0.792 -> 0.801, 0.793 -> 0.798)
+    // (8-rank fp16 reduce_scatter, one sweep per write phase without meetings -> two with: 512 / 256 /
+    // 128 / 64 MB per rank 0.805 -> 0.852, 0.831 -> 0.846, 0.834 -> 0.844, 0.832 -> 0.846 of peak; 32 / 16 MB,
+    // one sweep and half a one, 0.815 -> 0.764 / 0.619 -> 0.547).  The 512 x 16 shape of the other
+    // chains (up to 8 ranks) gains from it as well, from two sweeps on: fewer, longer phases (8-rank ring
+    // in place, 512 MiB per rank: bf16 0.778 -> 0.790, f16 0.770 -> 0.787, f32 0.782 -> 0.792, int32
+    // 0.788 -> 0.795 on one box; bf16 64 / 128 / 256 MiB 0.771 -> 0.785, 0.784 -> 0.784, 0.791 -> 0.799)
     const int64_t cus = device_cu_count(ctx->device);
-    const bool pays = mostly_reads ? L.total_chunks >= 4 * cus : (L.shape == 0 && L.total_chunks >= 2 * cus);
+    const bool pays = L.total_chunks >= 2 * cus && (mostly_reads || L.shape == 0);
     const bool two_sweeps = !tree_shape && (ctx->phased_sweeps == 2 || (ctx->phased_sweeps < 0 && ctx->phased_shape < 0 && pays));
     if (two_sweeps) L.shape = 4;
     L.barriers = ctx->phased_barriers && (two_sweeps || !mostly_reads) ? 1 : 0;

@@ -1261,6 +1261,53 @@ __device__ __forceinline__ void chain_read(u32x4 (&acc)[V], const PCCL_CONST int
     }
 }
 
+// The same for two chunks read in one phase (kept apart from chain_read, whose code the one-sweep
+// kernels were tuned with: with these flags added there, the compiler scheduled the 32-rank f32 MAX
+// kernel differently, 0.84 -> 0.79 of peak).  CIN: the ring already holds this chunk's first S
+// fetches (the call before ended with COUT); COUT: the last rank's refills go on into `after`, the
+// first source of the chunk read next, so that no fetch-free gap separates the two chunks.
+template <int DT, int OP, int T, int V, int S, int VS, int GR, bool CIN, bool COUT>
+__device__ __forceinline__ void chain_read_linked(u32x4 (&acc)[V], const PCCL_CONST int32_t* srcs, int n, const RankPtrs& ptrs,
+                                           u32x4* lds, int64_t chunk_byte0, uint32_t toff, int tid, const char* after = nullptr) {
+    static_assert(V % S == 0 && S <= V && S % GR == 0, "the slot of a vector must not depend on the rank; groups of GR vectors per wait");
+    u32x4* const my = lds + (tid & ~63);
+    const u32x4* const mine = lds + tid;
+    const char* cur = ptrs.p[kMaxR + srcs[0]] + chunk_byte0;
+    if constexpr (!CIN) {
+#pragma unroll
+        for (int q = 0; q < S; ++q) load_lds_nt(cur, toff + q * VS, my + q * T);
+    }
+    for (int k = 0; k < n; ++k) {
+        const bool last_rank = k + 1 == n;
+        const char* next = !last_rank ? ptrs.p[kMaxR + srcs[k + 1]] + chunk_byte0 : COUT ? after : cur;
+#pragma unroll
+        for (int v = 0; v < V; v += GR) {
+            // the GR oldest fetches have landed when at most S - GR are outstanding
+            if (!COUT && v + S >= V && last_rank) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(S - GR) : "memory");
+            u32x4 x[GR];
+#pragma unroll
+            for (int g = 0; g < GR; ++g) x[g] = mine[((v + g) % S) * T];
+#pragma unroll
+            for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_phase<DT, OP>(x[g], acc[v + g]);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
+#pragma unroll
+            for (int g = 0; g < GR; ++g) {
+                const int w = v + g;
+                if (w + S < V) load_lds_nt(cur, toff + (w + S) * VS, my + (w % S) * T);
+                else if (COUT || !last_rank) load_lds_nt(next, toff + (w + S - V) * VS, my + (w % S) * T);
+            }
+        }
+        cur = next;
+    }
+    if constexpr (kDeferredNan<DT>) {
+        if (n > 1) {      // a single source is a copy: its bits are kept as they are
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v] = canon_nan<DT>(acc[v]);
+        }
+    }
+}
+
 template <int V, class F, int... Vs>
 __device__ __forceinline__ void fill_by_index(u32x4 (&out)[V], F&& f, std::integer_sequence<int, Vs...>) {
     ((out[Vs] = f(Vs)), ...);
@@ -1468,9 +1515,12 @@ __global__ __launch_bounds__(T) void phased_kernel(PhasedLaunch L, RankPtrs ptrs
 // chunks in, one out), where a write phase per sweep would be too short to be worth a meeting and
 // without meetings the stores sprinkle the reads (bare kernels of this traffic, 8 x 512 MiB in and
 // 8 x 64 MiB out: 0.788 of peak without meetings, 0.804 with a write phase per sweep, 0.865 per two
-// sweeps, 0.868 per three); an allreduce in place on 8 ranks gains half a point to two points.
-// Chains read and written as slabs only; a kernel of its own, so that the one above keeps the code
-// it was tuned with.
+// sweeps, 0.868 per three); an allreduce in place on 8 ranks gains one to two points.  Two whole
+// chunks are read as ONE fetch stream: the ring runs on from the last rank of the first chunk into
+// the first rank of the second, so no fetch-free gap (one memory latency, chip-wide) separates them;
+// without that the f32 and f16 forms, whose NaN pass sits in that gap, lost what the longer phases
+// gained.  Chains read and written as slabs only; a kernel of its own, so that the one above keeps
+// the code it was tuned with.
 template <int DT, int T, int V, int S, int GR, int KK>
 __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtrs ptrs) {
     extern __shared__ u32x4 lds[];
@@ -1494,9 +1544,9 @@ __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtr
         DevChainSegment seg[KK];
         int64_t vbase[KK];
         bool whole[KK];
-        // (a generic lambda called once per constant k: the compiler does not unroll a loop with this body,
+        // (generic lambdas called once per constant k: the compiler does not unroll a loop with these bodies,
         // and with k a variable the per-sweep state would not stay in scalar registers)
-        auto read_sweep = [&](auto kc) __attribute__((always_inline)) {
+        auto find_sweep = [&](auto kc) __attribute__((always_inline)) {
             constexpr int k = decltype(kc)::value;
             const int64_t chunk = (it0 + k) * G + place;
             const bool live = it0 + k < sweeps && chunk < L.total_chunks;
@@ -1505,7 +1555,7 @@ __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtr
             seg[k] = DevChainSegment{};
             vbase[k] = 0;
             whole[k] = false;
-            if (!live) return;
+            if (!live) return false;
             int lo = 0;
             if (L.seg_chunks > 0) {
                 const uint32_t per = (uint32_t)L.seg_chunks;
@@ -1520,11 +1570,17 @@ __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtr
             seg[k] = load_const(L.segs + lo);
             vbase[k] = seg[k].first_vec + (chunk - seg[k].first_chunk) * CHUNK_V;
             whole[k] = vbase[k] * VE >= seg[k].start && (vbase[k] + CHUNK_V) * VE <= seg[k].end;
+            return true;
+        };
+        // CIN / COUT: the fetch ring runs on from this sweep's chunk into the next one's (chain_read_linked)
+        auto read_sweep = [&](auto kc, auto cin, auto cout, const char* after) __attribute__((always_inline)) {
+            constexpr int k = decltype(kc)::value;
+            constexpr bool CIN = decltype(cin)::value, COUT = decltype(cout)::value;
             const PCCL_CONST int32_t* srcs = as_const(L.srcs) + seg[k].src_start;   // dwords: uniform reads become scalar loads
             if (whole[k]) {
-                if (seg[k].redop == PCCL_SUM) chain_read<DT, PCCL_SUM, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
-                else if (seg[k].redop == PCCL_MAX) chain_read<DT, PCCL_MAX, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
-                else chain_read<DT, PCCL_MIN, T, V, S, VS, GR>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid);
+                if (seg[k].redop == PCCL_SUM) chain_read_linked<DT, PCCL_SUM, T, V, S, VS, GR, CIN, COUT>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid, after);
+                else if (seg[k].redop == PCCL_MAX) chain_read_linked<DT, PCCL_MAX, T, V, S, VS, GR, CIN, COUT>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid, after);
+                else chain_read_linked<DT, PCCL_MIN, T, V, S, VS, GR, CIN, COUT>(acc[k], srcs, seg[k].n_src, ptrs, lds, vbase[k] * 16, toff, tid, after);
             } else {
                 // a chunk that the segment's ends cut: vector by vector, loads and stores together
                 for (int64_t j = tid; j < CHUNK_V; j += T) {
@@ -1540,8 +1596,22 @@ __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtr
                 }
             }
         };
-        read_sweep(std::integral_constant<int, 0>{});
-        if constexpr (KK > 1) read_sweep(std::integral_constant<int, 1>{});
+        constexpr std::integral_constant<int, 0> k0{};
+        constexpr std::integral_constant<int, 1> k1{};
+        constexpr std::false_type no{};
+        constexpr std::true_type yes{};
+        const bool live0 = find_sweep(k0);
+        bool live1 = false;
+        if constexpr (KK > 1) live1 = find_sweep(k1);
+        if (KK > 1 && whole[0] && whole[KK - 1]) {
+            // both chunks whole: one fetch stream through both
+            const char* after = ptrs.p[kMaxR + as_const(L.srcs)[seg[KK - 1].src_start]] + vbase[KK - 1] * 16;
+            read_sweep(k0, no, yes, after);
+            if constexpr (KK > 1) read_sweep(k1, yes, no, nullptr);
+        } else {
+            if (live0) read_sweep(k0, no, no, nullptr);
+            if constexpr (KK > 1) { if (live1) read_sweep(k1, no, no, nullptr); }
+        }
         if (meet) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();

@@ -238,6 +238,7 @@ def test_plans_that_mostly_write_take_larger_workgroups(engine_factory, world):
     eng = engine_factory(world)
     for r, j in enumerate(jsons):
         eng.register_operation_json("ag", j, r)
+    eng.set_option("phased", -1)                     # whatever PCCL_PHASED says: the automatic choice is what is tested
     shape = eng.get_option("slot_shape:ag")
     assert shape == ("256x2" if world == 8 else "256x1"), shape
     assert eng.get_option("runner_staged:ag") == "column_slot_kernel"
