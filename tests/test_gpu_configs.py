@@ -303,3 +303,40 @@ def test_config3_full_size_against_the_cpu_oracle(engine_factory):
     engine.execute_inplace("c3_oracle", bufs, sync=True)
     for r in range(world):
         assert bits_equal(bufs[r], want[r]), f"rank {r}"
+
+
+@pytest.mark.parametrize("runner", ["phased", "slot", "stepwise", "persistent"])
+def test_rank_buffers_larger_than_4_gib(engine_factory, runner):
+    """Byte offsets inside a rank buffer pass 2^32 (element offsets stay below the 2^31 of the trigger
+    layout): a 2-rank f32 ring allreduce on 5 GiB per rank, in place, on every runner.  Both ranks must
+    hold x0 + x1, which is the same bits in either order, over the whole buffer including its last
+    vectors; a staged reduce_scatter of the same size checks the far end of the input windows."""
+    world, n = 2, 1_342_177_280 + 12                       # 5 GiB and three vectors
+    x = dev_inputs("randn", world, n, "float32", seed=11)
+    want = x[0] + x[1]
+    eng = engine_factory(world)
+    jsons = graph_jsons("ring", "build_allreduce", world, n, "float32", "sm", 1)
+    register(eng, "big", jsons, {"phased": "column", "slot": "column"}.get(runner, runner))
+    eng.set_option("phased", 1 if runner == "phased" else 0)
+    try:
+        bufs = [t.clone() for t in x]
+        print(f"{runner}: in place, {n} elements per rank", flush=True)
+        eng.execute_inplace("big", bufs, sync=True)
+        if runner in ("phased", "slot"):
+            assert eng.get_option("runner_inplace:big") == ("phased_kernel" if runner == "phased" else "column_slot_kernel")
+        for r in range(world):
+            assert same_bits(bufs[r], want), f"rank {r}"
+        del bufs
+        rs = graph_jsons("ring", "build_reduce_scatter", world, n, "float32", "sm", 1)
+        for r, j in enumerate(rs):
+            eng.register_operation_json("big_rs", j, r)
+        chunk = n // world
+        outs = [torch.empty(chunk, dtype=torch.float32, device="cuda") for _ in range(world)]
+        print(f"{runner}: staged reduce_scatter", flush=True)
+        eng.execute_operation("big_rs", x, outs)
+        for r in range(world):
+            assert same_bits(outs[r], want[r * chunk:(r + 1) * chunk]), f"reduce_scatter rank {r}"
+    finally:
+        eng.set_option("mode", "auto"); eng.set_option("phased", -1)
+        del x, want
+        torch.cuda.empty_cache()
