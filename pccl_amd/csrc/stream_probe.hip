@@ -13,6 +13,10 @@
 //                            the writes, 2 meet before the reads only; L = 1: a wave's vectors contiguous;
 //                            L = 2: read as slabs, written with a wave's vectors contiguous (the sums
 //                            change hands through LDS between the phases)
+//          sweeps:K:A        the 512 x 16 phased shape (ring of 4, meetings) reading K sweeps - K chunks
+//                            of every rank, one after the other - before their sums are written; A = 1:
+//                            the sums go to every rank (an allreduce in place), A = 0: to one rank per
+//                            chunk (the traffic of a reduce_scatter); K = 0: one sweep, no meetings
 //          read:T / write:T / copy:T   streams only: every workgroup of T threads reads (writes) one
 //                            1 KiB-per-wave tile of every rank; copy: rank r to rank (r + ranks / 2)
 // Every case prints one JSON line; results are checked on the host for the cases that compute.
@@ -196,6 +200,62 @@ __global__ __launch_bounds__(T) void phased_probe(Ptrs p, int R, int64_t chunks,
     }
 }
 
+// ---- sweeps: K sweeps read before their sums are written ---------------------------------------------
+template <int KK, bool ALL, bool MEET>
+__global__ __launch_bounds__(512) void sweeps_probe(Ptrs p, int R, int64_t chunks, Meet* meet) {
+    constexpr int T = 512, V = 16, S = 4;
+    extern __shared__ u32x4 lds[];
+    const int tid = threadIdx.x;
+    const int G = gridDim.x;
+    const int place = (blockIdx.x & 7) * (G >> 3) + (blockIdx.x >> 3);
+    u32x4* const my = lds + (tid & ~63);
+    const u32x4* const mine = lds + tid;
+    int gen = 0;
+    const int64_t sweeps = (chunks + G - 1) / G;
+    constexpr int64_t VS = (int64_t)T * 16;
+    for (int64_t it0 = 0; it0 < sweeps; it0 += KK) {
+        u32x4 acc[KK][V];
+#pragma unroll
+        for (int k = 0; k < KK; ++k) {
+            const int64_t chunk = (it0 + k) * G + place;
+            const int64_t base = (chunk * V * T + tid) * 16;
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[k][v] = u32x4{0, 0, 0, 0};
+            if (it0 + k < sweeps && chunk < chunks) {
+#pragma unroll
+                for (int q = 0; q < S; ++q) lds_direct(p.p[0] + base + (int64_t)q * VS, my + q * T);
+                for (int r = 0; r < R; ++r) {
+                    const bool last_rank = r + 1 == R;
+                    const char* cur = p.p[r];
+                    const char* next = p.p[last_rank ? r : r + 1];
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        if (last_rank && v + S >= V) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                        else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(S - 1) : "memory");
+                        acc[k][v] += mine[(v % S) * T];
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        if (v + S < V) lds_direct(cur + base + (int64_t)(v + S) * VS, my + (v % S) * T);
+                        else if (!last_rank) lds_direct(next + base + (int64_t)(v + S - V) * VS, my + (v % S) * T);
+                    }
+                }
+            }
+        }
+        if (MEET) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); __syncthreads(); ++gen; meet_arrive(meet, gen, G); meet_wait(meet, gen); }
+#pragma unroll
+        for (int k = 0; k < KK; ++k) {
+            const int64_t chunk = (it0 + k) * G + place;
+            if (it0 + k < sweeps && chunk < chunks) {
+                for (int r = ALL ? 0 : (int)(chunk % R); r < (ALL ? R : (int)(chunk % R) + 1); ++r) {
+                    char* dst = p.p[r] + (chunk * V * T + tid) * 16;
+#pragma unroll
+                    for (int v = 0; v < V; ++v) st_stream(dst + (int64_t)v * VS, acc[k][v]);
+                }
+            }
+        }
+        if (MEET) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); __syncthreads(); ++gen; meet_arrive(meet, gen, G); meet_wait(meet, gen); }
+    }
+}
+
 // ---- streams only ----------------------------------------------------------------------------------
 // kind 0: read every rank, 1: write every rank, 2: copy rank r to rank r + R / 2
 __global__ __launch_bounds__(1024) void stream_kernel(Ptrs p, int R, int64_t tiles, int run_shift, int kind, u32x4* sink) {
@@ -323,6 +383,44 @@ int main(int argc, char** argv) {
             else if (T == 256 && V == 16 && S == 16 && L == 0) go(phased_probe<256, 16, 16, 0>, lds);
             else { std::printf("{\"case\": \"%s\", \"error\": \"shape not built\"}\n", c.c_str()); continue; }
             moved = 2.0 * R * (double)chunks * T * V * 16;
+        } else if (c.rfind("sweeps:", 0) == 0 && f.size() == 2) {
+            const int K = f[0];
+            const bool all = f[1] != 0;
+            constexpr int T = 512, V = 16;
+            const int64_t chunks = bytes / ((int64_t)T * V * 16);
+            const int lds = 84 * 1024;                      // keeps a second workgroup off the CU
+            auto go = [&](auto k) {
+                CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+                auto launch = [&]() {
+                    CHECK(hipMemsetAsync(meet, 0, sizeof(Meet), 0));
+                    hipLaunchKernelGGL(k, dim3(cus), dim3(T), (size_t)lds, 0, p, R, chunks, meet);
+                    CHECK(hipGetLastError());
+                };
+                fill(); launch(); CHECK(hipDeviceSynchronize());
+                // the sum wherever it was written, a rank's own value elsewhere
+                const uint32_t sum = (uint32_t)R * (R + 1) / 2;
+                const size_t cw = (size_t)T * V * 4;
+                for (int r = 0; r < R && ok; r += std::max(1, R - 1)) {
+                    CHECK(hipMemcpy(host.data(), p.p[r], bytes, hipMemcpyDeviceToHost));
+                    for (int64_t ch = 0; ch < chunks && ok; ++ch)
+                        for (size_t i = 0; i < cw; i += 251)
+                            if (host[ch * cw + i] != ((all || ch % R == r) ? sum : (uint32_t)(r + 1))) { ok = false; break; }
+                }
+                fill();     // an allreduce in place would otherwise sum sums
+                timed(launch);
+                Meet hm; CHECK(hipMemcpy(&hm, meet, sizeof(hm), hipMemcpyDeviceToHost));
+                if (hm.failed) ok = false;
+            };
+            if (K == 0 && all) go(sweeps_probe<1, true, false>);
+            else if (K == 0) go(sweeps_probe<1, false, false>);
+            else if (K == 1 && all) go(sweeps_probe<1, true, true>);
+            else if (K == 1) go(sweeps_probe<1, false, true>);
+            else if (K == 2 && all) go(sweeps_probe<2, true, true>);
+            else if (K == 2) go(sweeps_probe<2, false, true>);
+            else if (K == 3 && all) go(sweeps_probe<3, true, true>);
+            else if (K == 3) go(sweeps_probe<3, false, true>);
+            else { std::printf("{\"case\": \"%s\", \"error\": \"K must be 0 .. 3\"}\n", c.c_str()); continue; }
+            moved = (double)(all ? 2 * R : R + 1) * (double)chunks * T * V * 16;
         } else if ((c.rfind("read:", 0) == 0 || c.rfind("write:", 0) == 0 || c.rfind("copy:", 0) == 0) && f.size() == 1) {
             const int T = f[0], kind = c[0] == 'r' ? 0 : c[0] == 'w' ? 1 : 2;
             if (T % 64 || T < 64 || T > 1024 || (kind == 2 && R % 2)) { std::printf("{\"case\": \"%s\", \"error\": \"shape not available\"}\n", c.c_str()); continue; }
