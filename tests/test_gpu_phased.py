@@ -197,9 +197,11 @@ def test_two_launches_of_one_operation_on_two_streams(engine_factory):
         eng.set_option("phased", -1)
 
 
-def test_phased_launches_recorded_into_a_graph(engine_factory):
+@pytest.mark.parametrize("sweeps", [1, 2])
+def test_phased_launches_recorded_into_a_graph(engine_factory, sweeps):
     """A phased launch is one kernel and needs no set-up per launch (the meeting block cleans itself),
-    so it can be recorded and replayed; every replay against the oracle, eager work in between."""
+    so it can be recorded and replayed, with one sweep per write phase or two; every replay against
+    the oracle, eager work in between."""
     world, n = 8, 16 * CHUNK_VECS * 8                  # 16 chunks
     jsons = graph_jsons("ring", "build_allreduce", world, n, "bfloat16", "sm", 2)
     x = seeded_inputs("randn", world, n, "bfloat16", seed=13)
@@ -207,6 +209,8 @@ def test_phased_launches_recorded_into_a_graph(engine_factory):
     eng = engine_factory(world)
     _register(eng, "ph_graph", jsons)
     eng.set_option("phased", 1)
+    eng.set_option("phased_sweeps", sweeps)
+    eng.set_option("num_blocks", 5)                    # four sweeps of five workgroups: meetings inside the recorded launch
     try:
         src = [t.cuda() for t in x]
         bufs = [t.clone() for t in src]
@@ -229,7 +233,7 @@ def test_phased_launches_recorded_into_a_graph(engine_factory):
             torch.cuda.synchronize()
             _check(bufs, want, f"replay {rep}")
     finally:
-        eng.set_option("phased", -1)
+        eng.set_option("phased", -1); eng.set_option("phased_sweeps", -1); eng.set_option("num_blocks", 0)
 
 
 SPECIAL_BITS = {   # quiet NaNs with payloads, a signalling NaN, infinities, zeros, the smallest denormal, the largest finite values
