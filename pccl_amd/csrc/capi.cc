@@ -622,7 +622,8 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
         // 96 MiB on the slot runner with 256 threads 0.715 / 0.778 / 0.670 against 0.694 / 0.715 /
         // 0.650 for the register runner; 8 ranks x 256 / 512 MiB with 1024 threads x 1 vector 0.752 /
         // 0.759 against 0.735 / 0.740 for 256 x 2 - below that size the smaller tiles win (128 MiB
-        // 0.729 against 0.752, 32 MiB 0.64 against 0.70), and so they do at 16 ranks up to 16 MiB.
+        // 0.729 against 0.752, 32 MiB 0.64 against 0.70); 16 ranks x 64 / 256 MiB with 512 threads 0.723-0.732 /
+        // 0.738-0.741 against 0.702 / 0.706-0.710 for 256, and 0.70 against 0.80 at 16 MiB.
         const bool mostly_writes = P.slot_store_bytes >= 4 * P.slot_load_bytes && P.slot_load_bytes > 0 &&
                                    (P.direct_segs.empty() || P.direct_slot_store_bytes >= 4 * P.direct_slot_load_bytes);
         const bool automatic = ctx->slot_threads == 0 && ctx->slot_vecs == 0 && ctx->slot_direct;
@@ -633,6 +634,7 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
             if (automatic && mostly_writes) {
                 if (R > 16) sh = slot_shape(R, 256, 1, true);
                 else if (R > 4 && R <= 8 && rank_bytes >= ((int64_t)256 << 20)) sh = slot_shape(R, 1024, 1, true);
+                else if (R > 8 && rank_bytes >= ((int64_t)64 << 20)) sh = slot_shape(R, 512, 1, true);
             }
             const std::string why = slot_shape_error(R, sh);
             if (!why.empty()) throw Error{PCCL_ERR_INVALID, why};

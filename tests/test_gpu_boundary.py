@@ -266,6 +266,10 @@ def test_plans_that_mostly_write_take_larger_workgroups(engine_factory, world):
         for r, j in enumerate(big):
             eng.register_operation_json("ag_big", j, r)
         assert eng.get_option("slot_shape:ag_big") == "1024x1"
+        eng16 = engine_factory(16)
+        for r, j in enumerate(graph_jsons("ring", "build_allgather", 16, 1 << 25, "float16", "sm", 1)):
+            eng16.register_operation_json("ag_big", j, r)
+        assert eng16.get_option("slot_shape:ag_big") == "512x1"     # 16 ranks: from 64 MiB per rank on
         eng.set_option("slot_vecs", 2)                       # a shape that is asked for is kept
         try:
             assert eng.get_option("slot_shape:ag_big") == "256x2"
