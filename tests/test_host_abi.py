@@ -538,7 +538,7 @@ def test_bench_finds_the_committed_counter_figures():
     """bench.py copies the counter-measured HBM bytes per launch of its kernel from the committed
     rocprofv3 summary of the same workload and names that file (`roofline.traffic_source`): the files
     it looks for exist, hold a positive byte count, sit beside a summary that names their kernel and
-    record the hash of the kernel source they were taken on - a figure from another version of the
+    quotes that count, and record the hash of the kernel source they were taken on - a figure from another version of the
     kernels is not handed on."""
     import hashlib
     import importlib.util
@@ -564,5 +564,7 @@ def test_bench_finds_the_committed_counter_figures():
             assert nbytes is None and rel.startswith(f"profiles/{kernel}_{stem}.traffic.json") and "not used" in rel
         summary = os.path.join(root, "profiles", f"{kernel}_{stem}.md")
         assert os.path.exists(summary) and kernel in open(summary).read()
+        # the summary quotes the byte count that the file holds (they are written together)
+        assert f"{rec['hbm_bytes_per_launch']:,}" in open(summary).read(), (kernel, stem)
     assert bench.committed_traffic("column_slot_kernel", None) == (None, None)
     assert bench.committed_traffic("column_slot_kernel", "no_such_workload") == (None, None)
