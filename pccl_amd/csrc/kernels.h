@@ -111,9 +111,12 @@ struct PhasedLaunch {
     int32_t shape;            // 0: 512 threads x 16 vectors, 1: 256 threads x 32 vectors (each wave a contiguous 32 KiB),
                               // 2: 256 x 32 with the code for balanced trees as well; 3: as 1, but read as slabs and
                               // written with each wave on 32 KiB in a row (the sums change hands through LDS);
-                              // 4: as 0, two sweeps read before their sums are written
+                              // 4: as 0, two sweeps read before their sums are written; 5: 256 x 32 slabs, the
+                              // chunks of `group` workgroups interleaved slab by slab (phased_kernel_linear)
     int32_t num_blocks;       // 0: one workgroup per CU
     int32_t barriers;         // 1: all workgroups read together, then write together; 0: no meeting
+    int32_t group;            // shape 5: workgroups whose chunks are interleaved (a power of two that divides the grid and every
+                              // segment's chunk count; all chunks whole)
     PhaseSync* sync;
     uint64_t timeout_ticks;   // 100 MHz ticks a workgroup waits at a meeting point before it goes on alone
 };

@@ -1651,6 +1651,134 @@ __global__ __launch_bounds__(T) void phased_kernel_pairs(PhasedLaunch L, RankPtr
     }
 }
 
+// The 256 x 32 shape with the chunks of K neighbouring workgroups INTERLEAVED slab by slab: the K
+// chunks of a group are consecutive chunks of one segment, and slab v of workgroup j of the group is
+// piece (v K + j) of that region, T vectors long.  At every step of a phase the group then reads or
+// writes K x 4 KiB in a row - with K = 128 or 256 the chip sweeps each rank buffer as one linear
+// stream 0.5 to 1 MiB wide instead of 256 separate streams 128 KiB apart.  Bare kernels, 8 ranks x
+// 512 MiB in place: 0.824-0.828 of the 8 TB/s against 0.776 for the same shape with a chunk per
+// workgroup and 0.802-0.806 for 512 x 16 (write phases 6.5-6.6 TB/s against 5.8 and 6.0-6.1); groups
+// of 64 give 0.81, of 32 and fewer nothing.  At 16 and 32 ranks the shape that writes 32 KiB runs per
+// wave stays ahead.  Chains only, every chunk whole (the host checks), one sweep per write phase.
+template <int DT, int OP, int T, int V, int S, int GR>
+__device__ __forceinline__ void chain_read_strided(u32x4 (&acc)[V], const PCCL_CONST int32_t* srcs, int n, const RankPtrs& ptrs,
+                                                   u32x4* lds, int64_t first_byte, uint32_t toff, uint32_t vs, int tid) {
+    static_assert(V % S == 0 && S <= V && S % GR == 0, "the slot of a vector must not depend on the rank; groups of GR vectors per wait");
+    u32x4* const my = lds + (tid & ~63);
+    const u32x4* const mine = lds + tid;
+    const char* cur = ptrs.p[kMaxR + srcs[0]] + first_byte;
+#pragma unroll
+    for (int q = 0; q < S; ++q) load_lds_nt(cur, toff + q * vs, my + q * T);
+    for (int k = 0; k < n; ++k) {
+        const bool last_rank = k + 1 == n;
+        const char* next = ptrs.p[kMaxR + srcs[last_rank ? k : k + 1]] + first_byte;
+#pragma unroll
+        for (int v = 0; v < V; v += GR) {
+            if (v + S >= V && last_rank) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(S - GR) : "memory");
+            u32x4 x[GR];
+#pragma unroll
+            for (int g = 0; g < GR; ++g) x[g] = mine[((v + g) % S) * T];
+#pragma unroll
+            for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_phase<DT, OP>(x[g], acc[v + g]);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
+#pragma unroll
+            for (int g = 0; g < GR; ++g) {
+                const int w = v + g;
+                if (w + S < V) load_lds_nt(cur, toff + (w + S) * vs, my + (w % S) * T);
+                else if (!last_rank) load_lds_nt(next, toff + (w + S - V) * vs, my + (w % S) * T);
+            }
+        }
+        cur = next;
+    }
+    if constexpr (kDeferredNan<DT>) {
+        if (n > 1) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v] = canon_nan<DT>(acc[v]);
+        }
+    }
+}
+
+template <int DT, int T, int V, int S, int GR>
+__global__ __launch_bounds__(T) void phased_kernel_linear(PhasedLaunch L, RankPtrs ptrs) {
+    extern __shared__ u32x4 lds[];
+    __shared__ int s_flag;
+    static_assert((size_t)S * T * 16 <= 159u * 1024, "the fetch ring must fit a CU's LDS");
+    constexpr int64_t CHUNK_V = (int64_t)T * V;
+    const int tid = threadIdx.x;
+    const int G = gridDim.x;
+    const int K = L.group;                               // a power of two that divides G and every segment's chunk count
+    const int kshift = __builtin_ctz((unsigned)K);
+    // workgroup b runs on XCD b % 8: every XCD takes a contiguous eighth of each sweep
+    const int place = (G & 7) == 0 ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const uint32_t toff = (uint32_t)tid * 16;
+    const uint32_t vs = (uint32_t)K * T * 16;            // bytes between a thread's consecutive vectors
+    const int64_t sweeps = (L.total_chunks + G - 1) / G;
+    bool meet = L.barriers != 0;
+    int gen = 0;
+    for (int64_t it = 0; it < sweeps; ++it) {
+        const int64_t chunk = it * G + place;
+        const bool live = chunk < L.total_chunks;
+        u32x4 acc[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] = u32x4{0, 0, 0, 0};
+        DevChainSegment seg{};
+        int64_t first_byte = 0;
+        if (live) {
+            int lo = 0;
+            if (L.seg_chunks > 0) {
+                const uint32_t per = (uint32_t)L.seg_chunks;
+                lo = (per & (per - 1)) == 0 ? (int)((uint32_t)chunk >> __builtin_ctz(per)) : (int)((uint32_t)chunk / per);
+            } else {
+                int hi = L.num_segs;
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (as_const(L.segs)[mid].first_chunk <= chunk) lo = mid; else hi = mid;
+                }
+            }
+            seg = load_const(L.segs + lo);
+            const int64_t rel = chunk - seg.first_chunk;            // the chunk's number inside its segment
+            const int64_t first_vec = seg.first_vec + ((rel >> kshift) << kshift) * CHUNK_V + (rel & (K - 1)) * T;
+            first_byte = first_vec * 16;
+            const PCCL_CONST int32_t* srcs = as_const(L.srcs) + seg.src_start;   // dwords: uniform reads become scalar loads
+            if (seg.redop == PCCL_SUM) chain_read_strided<DT, PCCL_SUM, T, V, S, GR>(acc, srcs, seg.n_src, ptrs, lds, first_byte, toff, vs, tid);
+            else if (seg.redop == PCCL_MAX) chain_read_strided<DT, PCCL_MAX, T, V, S, GR>(acc, srcs, seg.n_src, ptrs, lds, first_byte, toff, vs, tid);
+            else chain_read_strided<DT, PCCL_MIN, T, V, S, GR>(acc, srcs, seg.n_src, ptrs, lds, first_byte, toff, vs, tid);
+        }
+        if (meet) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            ++gen;
+            phase_arrive(L.sync, gen, G);
+            meet = phase_wait(L.sync, gen, L.timeout_ticks, &s_flag);
+        }
+        if (live) {
+            for (uint64_t m = seg.store_mask; m; m &= m - 1) {
+                char* const dst = ptrs.p[__builtin_ctzll(m)] + first_byte;
+#pragma unroll
+                for (int v = 0; v < V; ++v) stv_nt_s(dst, toff + v * vs, acc[v]);
+            }
+        }
+        if (meet && it + 1 < sweeps) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            ++gen;
+            phase_arrive(L.sync, gen, G);
+            meet = phase_wait(L.sync, gen, L.timeout_ticks, &s_flag);
+        }
+    }
+    // the last workgroup to leave clears the meeting block for the next launch
+    if (L.barriers != 0 && tid == 0) {
+        const int old = __hip_atomic_fetch_add(&L.sync->exited, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old + 1 == G) {
+            __hip_atomic_store(&L.sync->arrive, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->release, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->broken, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->exited, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------- launchers
 
 // Per-device facts, queried once.  Contexts on different threads may ask at the same time: the
@@ -1772,7 +1900,7 @@ static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads
 
 template <int DT>
 static int launch_phased_dt(const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
-    static std::atomic<int> allowed[5][kMaxDevices];
+    static std::atomic<int> allowed[6][kMaxDevices];
     // integer sums never arrive as trees (the planner re-associates them into chains), and the 8-bit
     // floats' arithmetic leaves no registers for the tree code
     constexpr bool kNoTrees = DT == PCCL_I32 || DT == PCCL_F8E4M3 || DT == PCCL_F8E5M2;
@@ -1784,6 +1912,13 @@ static int launch_phased_dt(const PhasedLaunch& L, const RankPtrs& ptrs, hipStre
             else return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, 1, 2, true>, allowed[2], 256, 8, L, ptrs, s);
         case 3: return launch_phased_kernel(phased_kernel<DT, 256, 32, 8, 2, 2, false>, allowed[3], 256, 32, L, ptrs, s);
         case 4: return launch_phased_kernel(phased_kernel_pairs<DT, 512, 16, 4, 2, 2>, allowed[4], 512, 4, L, ptrs, s);   // two sweeps per write phase
+        case 5: {
+            // the grid has to be what the host chose the group for
+            int64_t grid = L.num_blocks > 0 ? L.num_blocks : current_cus();
+            if (grid > L.total_chunks) grid = L.total_chunks;
+            if (L.group < 1 || (L.group & (L.group - 1)) || grid % L.group || L.total_chunks % L.group) return (int)hipErrorInvalidValue;
+            return launch_phased_kernel(phased_kernel_linear<DT, 256, 32, 8, 2>, allowed[5], 256, 8, L, ptrs, s);
+        }
         default: return (int)hipErrorInvalidValue;
     }
 }

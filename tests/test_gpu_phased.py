@@ -163,6 +163,63 @@ def test_more_workgroups_than_fit_at_once(engine_factory):
         eng.set_option("phased", -1); eng.set_option("num_blocks", 0); eng.set_option("phased_timeout_us", 1000)
 
 
+@pytest.mark.parametrize("case", [(4, "bfloat16", "sum", 1), (2, "float32", "max", 1), (8, "float16", "sum", 1), (2, "int32", "sum", 2), (3, "float32", "min", 1)])
+def test_chunks_of_neighbouring_workgroups_interleaved(engine_factory, case):
+    """Chains on up to 8 ranks whose segments are whole multiples of 128 chunks run with the chunks of
+    128 neighbouring workgroups interleaved slab by slab (shape 5): in place and staged against the
+    oracle, with the option that switches it off, and with a grid or a size that does not allow it."""
+    world, dtype, op, channels = case
+    es = 4 if dtype in ("float32", "int32") else 2
+    seg_elems = 128 * CHUNK_VECS * (16 // es)                  # 16 MiB of every rank per segment
+    n = world * channels * seg_elems
+    jsons = graph_jsons("ring", "build_allreduce", world, n, dtype, "sm", channels, reduce_op=op)
+    kind = "randint" if dtype == "int32" else "randn"
+    x = seeded_inputs(kind, world, n, dtype, seed=17 + world)
+    want = oracle_buffers(jsons, x, dtype)
+    eng = engine_factory(world)
+    _register(eng, "ph_lin", jsons)
+    eng.set_option("phased", 1)
+    try:
+        assert eng.get_option("phased_shape_inplace:ph_lin") == "shape=5 group=128 meetings=1"
+        assert eng.get_option("phased_shape_staged:ph_lin") == "shape=5 group=128 meetings=1"
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("ph_lin", bufs, sync=True)
+        _check(bufs, want, "interleaved, in place")
+        outs = eng.execute_operation("ph_lin", [t.cuda() for t in x])
+        _check(outs, want, "interleaved, staged")
+        eng.set_option("phased_barriers", 0)
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("ph_lin", bufs, sync=True)
+        _check(bufs, want, "interleaved, no meetings")
+        eng.set_option("phased_barriers", 1)
+        eng.set_option("phased_linear", 0)
+        assert eng.get_option("phased_shape_inplace:ph_lin").split()[0] in ("shape=0", "shape=4")     # 4 from two sweeps on
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("ph_lin", bufs, sync=True)
+        _check(bufs, want, "switched off")
+        eng.set_option("phased_linear", -1)
+        eng.set_option("num_blocks", 100)                       # a grid that 128 does not divide
+        assert not eng.get_option("phased_shape_inplace:ph_lin").startswith("shape=5")
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("ph_lin", bufs, sync=True)
+        _check(bufs, want, "grid of 100")
+        eng.set_option("num_blocks", 128)                       # one group per sweep
+        assert eng.get_option("phased_shape_inplace:ph_lin") == "shape=5 group=128 meetings=1"
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("ph_lin", bufs, sync=True)
+        _check(bufs, want, "grid of 128")
+        eng.set_option("num_blocks", 0)
+    finally:
+        eng.set_option("phased", -1); eng.set_option("phased_linear", -1); eng.set_option("num_blocks", 0); eng.set_option("phased_barriers", 1)
+    # segments that are no multiple of 128 chunks keep the other shapes
+    if world == 2:
+        n2 = n + world * channels * CHUNK_VECS * (16 // es)
+        eng2 = engine_factory(world)
+        _register(eng2, "ph_lin2", graph_jsons("ring", "build_allreduce", world, n2, dtype, "sm", channels, reduce_op=op))
+        eng2.set_option("phased", 1)
+        assert not eng2.get_option("phased_shape_inplace:ph_lin2").startswith("shape=5")
+
+
 def test_two_launches_of_one_operation_on_two_streams(engine_factory):
     """In-place calls on different tensors may overlap on the GPU.  Two phased launches of one
     operation then share its meeting block and lose their phases, which costs time and nothing else:
