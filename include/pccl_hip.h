@@ -270,7 +270,11 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * wave on 32 KiB in a row for reads as well); "phased_sweeps" = "-1" | "1" | "2" (sweeps the 512 x 16
  * shape reads before it writes their sums: two make the phases longer and the meetings fewer; -1: two
  * from two sweeps on for plans on up to 8 ranks and for plans that load four times what they store,
- * which run without meetings below that); "phased_barriers" = "1" | "0" (0: no
+ * which run without meetings below that); "phased_linear" = "-1" | "0" | "1" (the 256 x 32 shape with
+ * the chunks of 128 neighbouring workgroups interleaved slab by slab, so that the chip sweeps each rank
+ * buffer as one stream; possible on up to 8 ranks when every segment of the plan is a whole multiple of
+ * 128 chunks - 16 MiB of every rank - and 128 divides the grid; -1: wherever possible except for plans
+ * that load four times what they store; 1: for those as well); "phased_barriers" = "1" | "0" (0: no
  * meetings, for comparison); "phased_timeout_us" (how long a workgroup waits at a meeting before the
  * launch goes on unsynchronised: meetings order nothing; the environment variable PCCL_PHASED sets
  * "phased" for new contexts);
@@ -291,6 +295,9 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
  * "runner_inplace:NAME" / "runner_staged:NAME": the kernel an in-place / staged execution of operation
  * NAME would launch now - "phased_kernel", "column_slot_kernel", "column_kernel", "level_kernel",
  * "persistent_kernel", "gather_kernel", or "staging + ..." - which links the operation; and
+ * "phased_shape_inplace:NAME" / "phased_shape_staged:NAME": the phased runner's shape for operation
+ * NAME as "shape=N group=K meetings=M" (N: 0 = 512 threads x 16 vectors, 1 / 3 = 256 x 32 without / with
+ * the exchange, 2 = balanced trees, 4 = two sweeps per write phase, 5 = interleaved chunks), or "none";
  * "slot_shape:NAME": the slot runner's workgroup for operation NAME as "threads x vectors", e.g.
  * "256x2", or "0x0" if its column plan does not run there - chosen from the rank count, and larger
  * for plans that store at least four times what they load): what the

@@ -13,6 +13,8 @@
 //                            the writes, 2 meet before the reads only; L = 1: a wave's vectors contiguous;
 //                            L = 2: read as slabs, written with a wave's vectors contiguous (the sums
 //                            change hands through LDS between the phases)
+//                            L = 3 / 4 / 5: slabs, the chunks of 128 / 256 / 64 neighbouring workgroups interleaved
+//                            slab by slab - at every step the group reads or writes one contiguous piece of a rank
 //          sweeps:K:A        the 512 x 16 phased shape (ring of 4, meetings) reading K sweeps - K chunks
 //                            of every rank, one after the other - before their sums are written; A = 1:
 //                            the sums go to every rank (an allreduce in place), A = 0: to one rank per
@@ -145,13 +147,17 @@ __global__ __launch_bounds__(T) void phased_probe(Ptrs p, int R, int64_t chunks,
     int gen = 0;
     const int64_t sweeps = (chunks + G - 1) / G;
     constexpr bool WAVEC = LAY == 1;
-    constexpr int64_t VS = WAVEC ? 64 * 16 : (int64_t)T * 16;
-    constexpr int64_t WVS = LAY >= 1 ? 64 * 16 : (int64_t)T * 16;
+    constexpr bool GROUPED = LAY >= 3;
+    const int K = LAY == 3 ? 128 : LAY == 4 ? 256 : 64;                       // GROUPED: workgroups per group (the host checks that it divides the grid)
+    const int64_t VS = GROUPED ? (int64_t)K * T * 16 : WAVEC ? 64 * 16 : (int64_t)T * 16;
+    const int64_t WVS = GROUPED ? VS : LAY >= 1 ? 64 * 16 : (int64_t)T * 16;
     for (int64_t it = 0; it < sweeps; ++it) {
         const int64_t chunk = it * G + place;
         const bool live = chunk < chunks;
-        const int64_t base = WAVEC ? (chunk * V * T + (int64_t)(tid >> 6) * V * 64 + (tid & 63)) * 16 : (chunk * V * T + tid) * 16;
-        const int64_t wbase = LAY >= 1 ? (chunk * V * T + (int64_t)(tid >> 6) * V * 64 + (tid & 63)) * 16 : base;
+        // GROUPED: slab v of workgroup j of a group is piece (v K + j) of the group's K chunks
+        const int64_t base = GROUPED ? (((chunk / K) * V * K + chunk % K) * T + tid) * 16
+                           : WAVEC ? (chunk * V * T + (int64_t)(tid >> 6) * V * 64 + (tid & 63)) * 16 : (chunk * V * T + tid) * 16;
+        const int64_t wbase = GROUPED ? base : LAY >= 1 ? (chunk * V * T + (int64_t)(tid >> 6) * V * 64 + (tid & 63)) * 16 : base;
         u32x4 acc[V];
 #pragma unroll
         for (int v = 0; v < V; ++v) acc[v] = u32x4{0, 0, 0, 0};
@@ -371,6 +377,8 @@ int main(int argc, char** argv) {
             };
             // the 84 KiB keep a second workgroup off the CU
             const int lds = std::max(84 * 1024, L == 2 ? T * V * 16 : S * T * 16);
+            const int group = L == 3 ? 128 : L == 4 ? 256 : L == 5 ? 64 : 1;
+            if (cus % group || chunks % group) { std::printf("{\"case\": \"%s\", \"error\": \"the group does not divide the grid or the chunks\"}\n", c.c_str()); continue; }
             if (T == 512 && V == 16 && S == 4 && L == 0) go(phased_probe<512, 16, 4, 0>, lds);
             else if (T == 512 && V == 16 && S == 4 && L == 1) go(phased_probe<512, 16, 4, 1>, lds);
             else if (T == 512 && V == 16 && S == 4 && L == 2) go(phased_probe<512, 16, 4, 2>, lds);
@@ -378,6 +386,11 @@ int main(int argc, char** argv) {
             else if (T == 256 && V == 32 && S == 8 && L == 0) go(phased_probe<256, 32, 8, 0>, lds);
             else if (T == 256 && V == 32 && S == 8 && L == 1) go(phased_probe<256, 32, 8, 1>, lds);
             else if (T == 256 && V == 32 && S == 8 && L == 2) go(phased_probe<256, 32, 8, 2>, lds);
+            else if (T == 256 && V == 32 && S == 8 && L == 3) go(phased_probe<256, 32, 8, 3>, lds);
+            else if (T == 256 && V == 32 && S == 8 && L == 4) go(phased_probe<256, 32, 8, 4>, lds);
+            else if (T == 256 && V == 32 && S == 8 && L == 5) go(phased_probe<256, 32, 8, 5>, lds);
+            else if (T == 512 && V == 16 && S == 4 && L == 3) go(phased_probe<512, 16, 4, 3>, lds);
+            else if (T == 512 && V == 16 && S == 4 && L == 4) go(phased_probe<512, 16, 4, 4>, lds);
             else if (T == 256 && V == 32 && S == 16 && L == 1) go(phased_probe<256, 32, 16, 1>, lds);
             else if (T == 1024 && V == 8 && S == 8 && L == 0) go(phased_probe<1024, 8, 8, 0>, lds);
             else if (T == 256 && V == 16 && S == 16 && L == 0) go(phased_probe<256, 16, 16, 0>, lds);

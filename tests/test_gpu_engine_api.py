@@ -478,6 +478,7 @@ OPTIONS = {   # key: (values that are taken and read back as written, values tha
     "phased_shape": ([0, 1, -1], [2, 4]),
     "phased_exchange": ([0, 1, -1], [2]),
     "phased_sweeps": ([1, 2, -1], [0, 3, "two"]),
+    "phased_linear": ([0, 1, -1], [2, -2]),
     "phased_barriers": ([0, 1], ["x"]),
     "phased_timeout_us": ([50, 1000], ["1ms"]),
     "lds_slots": ([0, 1], ["lds"]),

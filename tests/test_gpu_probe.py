@@ -16,6 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 CASES = ("read:256 write:256 copy:256 tile:256:2:8:0 tile:256:1:8:1 tile:256:2:4:0 "
          "phased:512:16:4:0:0 phased:512:16:4:1:0 phased:512:16:4:2:0 phased:256:32:8:1:1 phased:256:32:8:1:2 phased:512:16:4:1:2 "
+         "phased:256:32:8:1:3 phased:256:32:8:1:4 phased:256:32:8:1:5 phased:512:16:4:1:3 "
          "sweeps:0:0 sweeps:1:0 sweeps:2:0 sweeps:3:0 sweeps:1:1 sweeps:2:1 sweeps:3:1")
 
 
