@@ -880,16 +880,32 @@ int launch_levels(pccl_hip_ctx* ctx, OpEntry& e, const StepwiseLaunch& L, const 
 // rank per CU on (8-rank bf16 ring allreduce, in place: 16 MiB per rank 54 us on either runner, 32 MiB
 // 88 against 97 us, 128 MiB 0.344 against 0.359 ms); smaller tensors stay with the slot runner, whose
 // many small workgroups start and end faster (4 MiB per rank: 17 against 44 us).
+// Whether the plan can run with the chunks of 128 neighbouring workgroups interleaved slab by slab
+// (phased_kernel_linear): chains on up to 8 ranks, every segment a whole multiple of 128 chunks, a
+// grid that 128 divides.
+constexpr int kLinearGroup = 128;
+bool linear_fits(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
+    const int64_t chunks = direct ? e.direct_chain_chunks : e.chain_chunks;
+    const int seg_chunks = direct ? e.direct_chain_seg_chunks : e.chain_seg_chunks;
+    const int tree_shape = direct ? e.direct_chain_tree : e.chain_tree;
+    const bool whole = direct ? e.direct_chain_whole : e.chain_whole;
+    int64_t grid = ctx->num_blocks > 0 ? ctx->num_blocks : device_cu_count(ctx->device);
+    if (grid > chunks) grid = chunks;
+    return !tree_shape && ctx->R <= 8 && whole && seg_chunks > 0 && seg_chunks % kLinearGroup == 0 && grid > 0 && grid % kLinearGroup == 0;
+}
+
 bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     const int64_t chunks = direct ? e.direct_chain_chunks : e.chain_chunks;
     const DevBuf& segs = direct ? e.direct_chain_segs : e.chain_segs;
     if (ctx->phased == 0 || chunks <= 0 || !segs.p || !e.phase_sync.p) return false;
     if (ctx->phased == 1) return true;
     // a plan that mostly writes (an allgather: one chunk in, R out) has no read phase to speak of and
-    // is faster with the slot runner's wave-dealt stores (8 x 512 MB fp16: 0.80 against 0.86 ms)
+    // is faster with the slot runner's wave-dealt stores (8 x 512 MB fp16: 0.80 against 0.83-0.86 ms) -
+    // unless its chunks can be interleaved, which is what its writes gain from (8 x 128 / 256 / 512 MB:
+    // 0.773 / 0.77 / 0.759 of peak against 0.75 / 0.735-0.74 / 0.76 on the slot runner)
     const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
     const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
-    if (2 * loads < stores) return false;
+    if (2 * loads < stores) return ctx->phased_linear != 0 && ctx->phased_shape < 0 && ctx->phased_sweeps < 0 && linear_fits(ctx, e, direct);
     // it pays from one chunk per two CUs on (8-rank bf16 ring in place: 16 MiB per rank, 128 chunks,
     // 0.613 -> 0.637 of peak; 32 MiB 0.679 -> 0.748; 8 MiB 0.563 -> 0.368.  8-rank fp16 reduce_scatter:
     // 16 MB per rank 32.6 -> 29.3 us, 8 MB 18.6 -> 25.8).  Quarter chunks for the sizes below were
@@ -942,13 +958,8 @@ PhasedLaunch phased_launch_for(pccl_hip_ctx* ctx, OpEntry& e, bool direct) {
     // on one box).  Plans that mostly read keep the two-sweep shape: their gain is on the read side.
     L.group = 0;
     {
-        constexpr int K = 128;
-        int64_t grid = ctx->num_blocks > 0 ? ctx->num_blocks : cus;
-        if (grid > L.total_chunks) grid = L.total_chunks;
-        const bool whole = direct ? e.direct_chain_whole : e.chain_whole;
-        const bool fits = !tree_shape && ctx->R <= 8 && whole && L.seg_chunks > 0 && L.seg_chunks % K == 0 && grid % K == 0;
         const bool wanted = ctx->phased_linear == 1 || (ctx->phased_linear < 0 && ctx->phased_shape < 0 && ctx->phased_sweeps < 0 && !mostly_reads);
-        if (fits && wanted) { L.shape = 5; L.group = K; }
+        if (wanted && linear_fits(ctx, e, direct)) { L.shape = 5; L.group = kLinearGroup; }
     }
     L.barriers = ctx->phased_barriers && (two_sweeps || L.shape == 5 || !mostly_reads) ? 1 : 0;
     L.sync = (PhaseSync*)e.phase_sync.p;

@@ -220,6 +220,41 @@ def test_chunks_of_neighbouring_workgroups_interleaved(engine_factory, case):
         assert not eng2.get_option("phased_shape_inplace:ph_lin2").startswith("shape=5")
 
 
+def test_allgather_on_interleaved_chunks(engine_factory):
+    """A plan that mostly writes stays on the slot runner unless its chunks can be interleaved: an
+    allgather of 16 MiB pieces goes to the phased runner's shape 5 by itself (staged and in place),
+    one of 8 MiB pieces does not.  Against the oracle; an allgather only copies."""
+    world, dtype = 4, "float16"
+    chunk = 128 * CHUNK_VECS * 8                               # 16 MiB of fp16 per rank's piece
+    n = world * chunk
+    jsons = graph_jsons("ring", "build_allgather", world, n, dtype, "sm", 1)
+    x = seeded_inputs("randn", world, chunk, dtype, seed=5)
+    want = oracle_buffers(jsons, x, dtype, buffer_elems=n, place=lambda r: r * chunk)
+    eng = engine_factory(world)
+    _register(eng, "ag_lin", jsons)
+    eng.set_option("phased", -1)                               # the automatic choice, whatever PCCL_PHASED says
+    assert eng.get_option("runner_staged:ag_lin") == "phased_kernel"
+    assert eng.get_option("phased_shape_staged:ag_lin") == "shape=5 group=128 meetings=1"
+    outs = [torch.zeros(n, dtype=torch.float16, device="cuda") for _ in range(world)]
+    eng.execute_operation("ag_lin", [t.cuda() for t in x], outs)
+    _check(outs, want, "staged")
+    bufs = []
+    for r in range(world):
+        b = torch.zeros(n, dtype=torch.float16)
+        b[r * chunk:(r + 1) * chunk] = x[r]
+        bufs.append(b.cuda())
+    assert eng.get_option("phased_shape_inplace:ag_lin") == "shape=5 group=128 meetings=1"
+    eng.execute_inplace("ag_lin", bufs, sync=True)
+    _check(bufs, want, "in place")
+    eng.set_option("phased_linear", 0)
+    assert eng.get_option("runner_staged:ag_lin") == "column_slot_kernel"
+    eng.set_option("phased_linear", -1)
+    half = graph_jsons("ring", "build_allgather", world, n // 2, dtype, "sm", 1)
+    _register(eng, "ag_half", half)
+    assert eng.get_option("runner_staged:ag_half") == "column_slot_kernel"
+    assert eng.get_option("phased_shape_staged:ag_half") == "none"
+
+
 def test_two_launches_of_one_operation_on_two_streams(engine_factory):
     """In-place calls on different tensors may overlap on the GPU.  Two phased launches of one
     operation then share its meeting block and lose their phases, which costs time and nothing else:

@@ -552,7 +552,7 @@ def test_bench_finds_the_committed_counter_figures():
     allreduces = ["ring_allreduce_R8_bf16_512MiB", "rhd_allreduce_R16_f32_64MiB", "tree_allreduce_R32_int32_sum_96MiB", "tree_allreduce_R32_f32_max_96MiB"]
     wanted = [(k, stem) for k in ("phased_kernel", "column_slot_kernel") for stem in allreduces]
     wanted += [("level_kernel", "ring_allreduce_R8_bf16_512MiB"), ("persistent_kernel", "ring_allreduce_R8_bf16_512MiB"),
-               ("phased_kernel", "ring_reduce_scatter_R8_f16_512MB_staged"), ("column_slot_kernel", "ring_allgather_R8_f16_512MB_staged")]
+               ("phased_kernel", "ring_reduce_scatter_R8_f16_512MB_staged"), ("phased_kernel", "ring_allgather_R8_f16_512MB_staged")]
     for kernel, stem in wanted:
         path = os.path.join(root, "profiles", f"{kernel}_{stem}.traffic.json")
         rec = json.load(open(path))
