@@ -273,7 +273,8 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * which run without meetings below that); "phased_linear" = "-1" | "0" | "1" (the 256 x 32 shape with
  * the chunks of 128 neighbouring workgroups interleaved slab by slab, so that the chip sweeps each rank
  * buffer as one stream; possible on up to 8 ranks when every segment of the plan is a whole multiple of
- * 128 chunks - 16 MiB of every rank - and 128 divides the grid; -1: wherever possible except for plans
+ * 128 chunks - 16 MiB of every rank - and 128 divides the grid (groups of 64 for plans that mostly
+ * write, where 128 does not divide); -1: wherever possible except for plans
  * that load four times what they store; 1: for those as well); "phased_barriers" = "1" | "0" (0: no
  * meetings, for comparison); "phased_timeout_us" (how long a workgroup waits at a meeting before the
  * launch goes on unsynchronised: meetings order nothing; the environment variable PCCL_PHASED sets

@@ -881,17 +881,27 @@ int launch_levels(pccl_hip_ctx* ctx, OpEntry& e, const StepwiseLaunch& L, const 
 // 88 against 97 us, 128 MiB 0.344 against 0.359 ms); smaller tensors stay with the slot runner, whose
 // many small workgroups start and end faster (4 MiB per rank: 17 against 44 us).
 // Whether the plan can run with the chunks of 128 neighbouring workgroups interleaved slab by slab
-// (phased_kernel_linear): chains on up to 8 ranks, every segment a whole multiple of 128 chunks, a
-// grid that 128 divides.
+// (phased_kernel_linear), and in groups of how many: chains on up to 8 ranks, every segment a whole
+// multiple of 128 chunks and a grid that 128 divides; 0 if it cannot.
 constexpr int kLinearGroup = 128;
-bool linear_fits(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
+int linear_group(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct);
+bool linear_fits(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) { return linear_group(ctx, e, direct) > 0; }
+int linear_group(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     const int64_t chunks = direct ? e.direct_chain_chunks : e.chain_chunks;
     const int seg_chunks = direct ? e.direct_chain_seg_chunks : e.chain_seg_chunks;
     const int tree_shape = direct ? e.direct_chain_tree : e.chain_tree;
     const bool whole = direct ? e.direct_chain_whole : e.chain_whole;
     int64_t grid = ctx->num_blocks > 0 ? ctx->num_blocks : device_cu_count(ctx->device);
     if (grid > chunks) grid = chunks;
-    return !tree_shape && ctx->R <= 8 && whole && seg_chunks > 0 && seg_chunks % kLinearGroup == 0 && grid > 0 && grid % kLinearGroup == 0;
+    if (tree_shape || ctx->R > 8 || !whole || seg_chunks <= 0 || grid <= 0) return 0;
+    if (seg_chunks % kLinearGroup == 0 && grid % kLinearGroup == 0) return kLinearGroup;
+    // groups of 64 where 128 does not divide the segments: worth it for plans that mostly write only
+    // (8 x 64 MB fp16 allgather 0.727-0.729 -> 0.738-0.741 of peak; an allreduce gets from them what
+    // the two-sweep shape gives it anyway)
+    const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
+    const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
+    if (2 * loads < stores && seg_chunks % 64 == 0 && grid % 64 == 0) return 64;
+    return 0;
 }
 
 bool wants_phased(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
@@ -959,7 +969,7 @@ PhasedLaunch phased_launch_for(pccl_hip_ctx* ctx, OpEntry& e, bool direct) {
     L.group = 0;
     {
         const bool wanted = ctx->phased_linear == 1 || (ctx->phased_linear < 0 && ctx->phased_shape < 0 && ctx->phased_sweeps < 0 && !mostly_reads);
-        if (wanted && linear_fits(ctx, e, direct)) { L.shape = 5; L.group = kLinearGroup; }
+        if (wanted && linear_fits(ctx, e, direct)) { L.shape = 5; L.group = linear_group(ctx, e, direct); }
     }
     L.barriers = ctx->phased_barriers && (two_sweeps || L.shape == 5 || !mostly_reads) ? 1 : 0;
     L.sync = (PhaseSync*)e.phase_sync.p;

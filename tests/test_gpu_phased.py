@@ -249,10 +249,19 @@ def test_allgather_on_interleaved_chunks(engine_factory):
     eng.set_option("phased_linear", 0)
     assert eng.get_option("runner_staged:ag_lin") == "column_slot_kernel"
     eng.set_option("phased_linear", -1)
+    # pieces of 8 MiB (64 chunks): groups of 64, for plans that mostly write; of 4 MiB: the slot runner
     half = graph_jsons("ring", "build_allgather", world, n // 2, dtype, "sm", 1)
     _register(eng, "ag_half", half)
-    assert eng.get_option("runner_staged:ag_half") == "column_slot_kernel"
-    assert eng.get_option("phased_shape_staged:ag_half") == "none"
+    assert eng.get_option("phased_shape_staged:ag_half") == "shape=5 group=64 meetings=1"
+    xh = seeded_inputs("randn", world, chunk // 2, dtype, seed=6)
+    wanth = oracle_buffers(half, xh, dtype, buffer_elems=n // 2, place=lambda r: r * (chunk // 2))
+    outs = [torch.zeros(n // 2, dtype=torch.float16, device="cuda") for _ in range(world)]
+    eng.execute_operation("ag_half", [t.cuda() for t in xh], outs)
+    _check(outs, wanth, "groups of 64, staged")
+    quarter = graph_jsons("ring", "build_allgather", world, n // 4, dtype, "sm", 1)
+    _register(eng, "ag_quarter", quarter)
+    assert eng.get_option("runner_staged:ag_quarter") == "column_slot_kernel"
+    assert eng.get_option("phased_shape_staged:ag_quarter") == "none"
 
 
 def test_two_launches_of_one_operation_on_two_streams(engine_factory):
