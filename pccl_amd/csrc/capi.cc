@@ -379,6 +379,8 @@ struct OpEntry {
     int chain_seg_chunks = 0, direct_chain_seg_chunks = 0;   // > 0: every segment has this many chunks
     int chain_tree = 0, direct_chain_tree = 0;               // the plan holds balanced trees: the shape it runs on (0: none)
     bool chain_whole = false, direct_chain_whole = false;    // every chunk of the plan lies inside its segment (no cut chunks)
+    bool chain_alike = false, direct_chain_alike = false;    // the segments are adjacent in memory, with the same number of sources, operator
+                                                             // and store mask, their source lists one after the other
     int64_t total_tiles = 0, direct_tiles = 0;
     int seg_tiles = 0, direct_seg_tiles = 0;   // > 0: every segment of the plan has this many tiles
     int vecs_per_thread = 0;
@@ -684,7 +686,7 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
         if (!P.direct_segs.empty()) e.host.direct_segs = device_segments(P.direct_segs, &e.direct_tiles, &e.direct_seg_tiles);
         // chain plans for the phased runner (both of its workgroup shapes take chunks of the same size)
         static_assert(phased_chunk_vecs(0) == phased_chunk_vecs(1) && phased_chunk_vecs(0) == phased_chunk_vecs(2), "one chunk table serves all shapes");
-        auto chain_segments = [&](const std::vector<ChainSegment>& segs, int64_t* total, int* uniform, int* tree_shape, bool* all_whole) {
+        auto chain_segments = [&](const std::vector<ChainSegment>& segs, int64_t* total, int* uniform, int* tree_shape, bool* all_whole, bool* alike) {
             std::vector<DevChainSegment> ds(segs.size());
             int64_t chunks = 0;
             int depth = 0;
@@ -693,6 +695,10 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
             // 8-bit floats, whose arithmetic leaves no registers for it: those stay with the slot runner)
             *tree_shape = depth == 0 ? 0 : 2;
             *all_whole = !segs.empty();
+            *alike = !segs.empty() && depth == 0;
+            for (size_t i = 1; i < segs.size() && *alike; ++i)
+                *alike = segs[i].n_src == segs[0].n_src && segs[i].redop == segs[0].redop && segs[i].store_mask == segs[0].store_mask &&
+                         segs[i].src_start == segs[0].src_start + (int)i * segs[0].n_src && segs[i].start == segs[i - 1].end;
             if (depth > 0 && (P.dtype == PCCL_F8E4M3 || P.dtype == PCCL_F8E5M2)) { *total = 0; *uniform = 0; *all_whole = false; return std::vector<DevChainSegment>(); }
             const int64_t chunk_v = phased_chunk_vecs(*tree_shape);
             for (size_t i = 0; i < segs.size(); ++i) {
@@ -714,8 +720,8 @@ void link_host(pccl_hip_ctx* ctx, OpEntry& e) {
             return ds;
         };
         e.chain_chunks = e.direct_chain_chunks = 0;
-        e.host.chain_segs = chain_segments(P.chain_segs, &e.chain_chunks, &e.chain_seg_chunks, &e.chain_tree, &e.chain_whole);
-        e.host.direct_chain_segs = chain_segments(P.direct_chain_segs, &e.direct_chain_chunks, &e.direct_chain_seg_chunks, &e.direct_chain_tree, &e.direct_chain_whole);
+        e.host.chain_segs = chain_segments(P.chain_segs, &e.chain_chunks, &e.chain_seg_chunks, &e.chain_tree, &e.chain_whole, &e.chain_alike);
+        e.host.direct_chain_segs = chain_segments(P.direct_chain_segs, &e.direct_chain_chunks, &e.direct_chain_seg_chunks, &e.direct_chain_tree, &e.direct_chain_whole, &e.direct_chain_alike);
         e.host.chain_srcs.assign(P.chain_srcs.begin(), P.chain_srcs.end());
         if (e.host.chain_srcs.size() % 2) e.host.chain_srcs.push_back(0);
     }
@@ -884,9 +890,10 @@ int launch_levels(pccl_hip_ctx* ctx, OpEntry& e, const StepwiseLaunch& L, const 
 // (phased_kernel_linear), and in groups of how many: chains on up to 8 ranks, every segment a whole
 // multiple of 128 chunks and a grid that 128 divides; 0 if it cannot.
 constexpr int kLinearGroup = 128;
-int linear_group(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct);
+int linear_group(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct, int* group_segs = nullptr);
 bool linear_fits(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) { return linear_group(ctx, e, direct) > 0; }
-int linear_group(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
+int linear_group(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct, int* group_segs) {
+    if (group_segs) *group_segs = 1;
     const int64_t chunks = direct ? e.direct_chain_chunks : e.chain_chunks;
     const int seg_chunks = direct ? e.direct_chain_seg_chunks : e.chain_seg_chunks;
     const int tree_shape = direct ? e.direct_chain_tree : e.chain_tree;
@@ -895,12 +902,23 @@ int linear_group(const pccl_hip_ctx* ctx, const OpEntry& e, bool direct) {
     if (grid > chunks) grid = chunks;
     if (tree_shape || ctx->R > 8 || !whole || seg_chunks <= 0 || grid <= 0) return 0;
     if (seg_chunks % kLinearGroup == 0 && grid % kLinearGroup == 0) return kLinearGroup;
-    // groups of 64 where 128 does not divide the segments: worth it for plans that mostly write only
-    // (8 x 64 MB fp16 allgather 0.727-0.729 -> 0.738-0.741 of peak; an allreduce gets from them what
-    // the two-sweep shape gives it anyway)
+    // shorter segments: a group spans two of them - four for plans that mostly write - if they are alike
+    // (the rows of a group then belong to different segments: phased_kernel_linear_rows).  8-rank bf16
+    // ring in place on 4 channels against the two-sweep shape, fraction of peak: segments of 64 chunks
+    // (256 MiB per rank) 0.794-0.796 -> 0.816-0.819; of 32 chunks 0.784 / 0.816 -> 0.7855 / 0.7925; of 16
+    // chunks 0.777-0.784 -> 0.764.  fp16 allgather against the slot runner: 8 x 64 MB 0.733 -> 0.758-0.767,
+    // 8 x 32 MB 0.696-0.698 -> 0.711-0.713.
+    const bool alike = direct ? e.direct_chain_alike : e.chain_alike;
     const int64_t loads = direct ? e.prog.direct_slot_load_bytes : e.prog.slot_load_bytes;
     const int64_t stores = direct ? e.prog.direct_slot_store_bytes : e.prog.slot_store_bytes;
-    if (2 * loads < stores && seg_chunks % 64 == 0 && grid % 64 == 0) return 64;
+    const bool mostly_writes = 2 * loads < stores;
+    if (alike && grid % kLinearGroup == 0 && chunks % kLinearGroup == 0 && (seg_chunks == 64 || (seg_chunks == 32 && mostly_writes))) {
+        if (group_segs) *group_segs = kLinearGroup / seg_chunks;
+        return kLinearGroup;
+    }
+    // groups of 64 where that is not possible (segments of 64 chunks that are not alike): worth it for
+    // plans that mostly write only (8 x 64 MB fp16 allgather 0.727-0.729 -> 0.738-0.741 of peak)
+    if (mostly_writes && seg_chunks % 64 == 0 && grid % 64 == 0) return 64;
     return 0;
 }
 
@@ -969,7 +987,7 @@ PhasedLaunch phased_launch_for(pccl_hip_ctx* ctx, OpEntry& e, bool direct) {
     L.group = 0;
     {
         const bool wanted = ctx->phased_linear == 1 || (ctx->phased_linear < 0 && ctx->phased_shape < 0 && ctx->phased_sweeps < 0 && !mostly_reads);
-        if (wanted && linear_fits(ctx, e, direct)) { L.shape = 5; L.group = linear_group(ctx, e, direct); }
+        if (wanted && linear_fits(ctx, e, direct)) { int gs = 1; L.shape = 5; L.group = linear_group(ctx, e, direct, &gs); L.group_segs = gs; }
     }
     L.barriers = ctx->phased_barriers && (two_sweeps || L.shape == 5 || !mostly_reads) ? 1 : 0;
     L.sync = (PhaseSync*)e.phase_sync.p;
@@ -1572,7 +1590,7 @@ int pccl_hip_get_option(pccl_hip_ctx* ctx, const char* key, char* value, size_t 
             if (!plan || !wants_phased(ctx, e, staged)) v = "none";
             else {
                 const PhasedLaunch L = phased_launch_for(ctx, e, staged);
-                v = "shape=" + std::to_string(L.shape) + " group=" + std::to_string(L.group) + " meetings=" + std::to_string(L.barriers);
+                v = "shape=" + std::to_string(L.shape) + " group=" + std::to_string(L.group) + (L.group_segs > 1 ? " segments=" + std::to_string(L.group_segs) : std::string()) + " meetings=" + std::to_string(L.barriers);
             }
         }
         else if (k.rfind("slot_shape:", 0) == 0) {

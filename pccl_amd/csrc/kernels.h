@@ -117,6 +117,9 @@ struct PhasedLaunch {
     int32_t barriers;         // 1: all workgroups read together, then write together; 0: no meeting
     int32_t group;            // shape 5: workgroups whose chunks are interleaved (a power of two that divides the grid and every
                               // segment's chunk count; all chunks whole)
+    int32_t group_segs;       // shape 5: 1, or the segments a group spans (2 or 4: the segments are then `group` / group_segs
+                              // chunks long, adjacent in memory, with the same number of sources, operator and store mask,
+                              // their source lists one after the other in `srcs`)
     PhaseSync* sync;
     uint64_t timeout_ticks;   // 100 MHz ticks a workgroup waits at a meeting point before it goes on alone
 };

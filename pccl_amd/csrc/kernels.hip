@@ -1779,6 +1779,122 @@ __global__ __launch_bounds__(T) void phased_kernel_linear(PhasedLaunch L, RankPt
     }
 }
 
+// The interleaved shape for segments SHORTER than a group: a group of K workgroups spans NS adjacent
+// segments of K / NS chunks.  The group's region is V rows of K x T vectors; row v lies in segment
+// v / (V / NS) of the group, so the slabs of a thread belong to different segments and are combined in
+// different source orders: at step k of the chain, row v is fetched from the k-th source of ITS
+// segment.  The host has checked that the segments of the plan are adjacent in memory and have the
+// same number of sources, operator and store mask, their source lists one after the other.
+template <int DT, int OP, int T, int V, int S, int GR, int NS>
+__device__ __forceinline__ void chain_read_rows(u32x4 (&acc)[V], const PCCL_CONST int32_t* srcs0, int n, const RankPtrs& ptrs,
+                                                u32x4* lds, int64_t first_byte, uint32_t toff, uint32_t vs, int tid) {
+    static_assert(V % S == 0 && S <= V && S % GR == 0 && V % NS == 0, "slots must not depend on the rank; whole rows per segment");
+    constexpr int RP = V / NS;                   // rows per segment
+    u32x4* const my = lds + (tid & ~63);
+    const u32x4* const mine = lds + tid;
+    const char* pc[NS];
+    const char* pn[NS];
+#pragma unroll
+    for (int si = 0; si < NS; ++si) pc[si] = ptrs.p[kMaxR + srcs0[si * n]] + first_byte;
+#pragma unroll
+    for (int q = 0; q < S; ++q) load_lds_nt(pc[q / RP], toff + q * vs, my + q * T);
+    for (int k = 0; k < n; ++k) {
+        const bool last_rank = k + 1 == n;
+#pragma unroll
+        for (int si = 0; si < NS; ++si) pn[si] = last_rank ? pc[si] : ptrs.p[kMaxR + srcs0[si * n + k + 1]] + first_byte;
+#pragma unroll
+        for (int v = 0; v < V; v += GR) {
+            if (v + S >= V && last_rank) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(S - GR) : "memory");
+            u32x4 x[GR];
+#pragma unroll
+            for (int g = 0; g < GR; ++g) x[g] = mine[((v + g) % S) * T];
+#pragma unroll
+            for (int g = 0; g < GR; ++g) acc[v + g] = k == 0 ? x[g] : vec_phase<DT, OP>(x[g], acc[v + g]);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slots have been read before they are refilled
+#pragma unroll
+            for (int g = 0; g < GR; ++g) {
+                const int w = v + g;
+                if (w + S < V) load_lds_nt(pc[(w + S) / RP], toff + (w + S) * vs, my + (w % S) * T);
+                else if (!last_rank) load_lds_nt(pn[(w + S - V) / RP], toff + (w + S - V) * vs, my + (w % S) * T);
+            }
+        }
+#pragma unroll
+        for (int si = 0; si < NS; ++si) pc[si] = pn[si];
+    }
+    if constexpr (kDeferredNan<DT>) {
+        if (n > 1) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[v] = canon_nan<DT>(acc[v]);
+        }
+    }
+}
+
+template <int DT, int T, int V, int S, int GR, int NS>
+__global__ __launch_bounds__(T) void phased_kernel_linear_rows(PhasedLaunch L, RankPtrs ptrs) {
+    extern __shared__ u32x4 lds[];
+    __shared__ int s_flag;
+    static_assert((size_t)S * T * 16 <= 159u * 1024, "the fetch ring must fit a CU's LDS");
+    const int tid = threadIdx.x;
+    const int G = gridDim.x;
+    const int K = L.group;                               // a power of two that divides G; NS segments of K / NS chunks per group
+    const int kshift = __builtin_ctz((unsigned)K);
+    const int place = (G & 7) == 0 ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const uint32_t toff = (uint32_t)tid * 16;
+    const uint32_t vs = (uint32_t)K * T * 16;
+    const int64_t sweeps = (L.total_chunks + G - 1) / G;
+    bool meet = L.barriers != 0;
+    int gen = 0;
+    for (int64_t it = 0; it < sweeps; ++it) {
+        const int64_t chunk = it * G + place;
+        const bool live = chunk < L.total_chunks;
+        u32x4 acc[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] = u32x4{0, 0, 0, 0};
+        DevChainSegment seg{};
+        int64_t first_byte = 0;
+        if (live) {
+            const int64_t group = chunk >> kshift;
+            seg = load_const(L.segs + group * NS);          // the group's first segment; the others follow it in memory
+            first_byte = (seg.first_vec + (chunk & (K - 1)) * T) * 16;
+            const PCCL_CONST int32_t* srcs0 = as_const(L.srcs) + seg.src_start;
+            if (seg.redop == PCCL_SUM) chain_read_rows<DT, PCCL_SUM, T, V, S, GR, NS>(acc, srcs0, seg.n_src, ptrs, lds, first_byte, toff, vs, tid);
+            else if (seg.redop == PCCL_MAX) chain_read_rows<DT, PCCL_MAX, T, V, S, GR, NS>(acc, srcs0, seg.n_src, ptrs, lds, first_byte, toff, vs, tid);
+            else chain_read_rows<DT, PCCL_MIN, T, V, S, GR, NS>(acc, srcs0, seg.n_src, ptrs, lds, first_byte, toff, vs, tid);
+        }
+        if (meet) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            ++gen;
+            phase_arrive(L.sync, gen, G);
+            meet = phase_wait(L.sync, gen, L.timeout_ticks, &s_flag);
+        }
+        if (live) {
+            for (uint64_t m = seg.store_mask; m; m &= m - 1) {
+                char* const dst = ptrs.p[__builtin_ctzll(m)] + first_byte;
+#pragma unroll
+                for (int v = 0; v < V; ++v) stv_nt_s(dst, toff + v * vs, acc[v]);
+            }
+        }
+        if (meet && it + 1 < sweeps) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            ++gen;
+            phase_arrive(L.sync, gen, G);
+            meet = phase_wait(L.sync, gen, L.timeout_ticks, &s_flag);
+        }
+    }
+    if (L.barriers != 0 && tid == 0) {
+        const int old = __hip_atomic_fetch_add(&L.sync->exited, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old + 1 == G) {
+            __hip_atomic_store(&L.sync->arrive, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->release, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->broken, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&L.sync->exited, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------- launchers
 
 // Per-device facts, queried once.  Contexts on different threads may ask at the same time: the
@@ -1900,7 +2016,7 @@ static int launch_phased_kernel(K kernel, std::atomic<int>* allowed, int threads
 
 template <int DT>
 static int launch_phased_dt(const PhasedLaunch& L, const RankPtrs& ptrs, hipStream_t s) {
-    static std::atomic<int> allowed[6][kMaxDevices];
+    static std::atomic<int> allowed[8][kMaxDevices];
     // integer sums never arrive as trees (the planner re-associates them into chains), and the 8-bit
     // floats' arithmetic leaves no registers for the tree code
     constexpr bool kNoTrees = DT == PCCL_I32 || DT == PCCL_F8E4M3 || DT == PCCL_F8E5M2;
@@ -1917,6 +2033,14 @@ static int launch_phased_dt(const PhasedLaunch& L, const RankPtrs& ptrs, hipStre
             int64_t grid = L.num_blocks > 0 ? L.num_blocks : current_cus();
             if (grid > L.total_chunks) grid = L.total_chunks;
             if (L.group < 1 || (L.group & (L.group - 1)) || grid % L.group || L.total_chunks % L.group) return (int)hipErrorInvalidValue;
+            if (L.group_segs > 1) {
+                if (L.seg_chunks <= 0 || L.seg_chunks * L.group_segs != L.group) return (int)hipErrorInvalidValue;
+                switch (L.group_segs) {
+                    case 2: return launch_phased_kernel(phased_kernel_linear_rows<DT, 256, 32, 8, 2, 2>, allowed[6], 256, 8, L, ptrs, s);
+                    case 4: return launch_phased_kernel(phased_kernel_linear_rows<DT, 256, 32, 8, 2, 4>, allowed[7], 256, 8, L, ptrs, s);
+                    default: return (int)hipErrorInvalidValue;
+                }
+            }
             return launch_phased_kernel(phased_kernel_linear<DT, 256, 32, 8, 2>, allowed[5], 256, 8, L, ptrs, s);
         }
         default: return (int)hipErrorInvalidValue;

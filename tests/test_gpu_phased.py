@@ -220,6 +220,44 @@ def test_chunks_of_neighbouring_workgroups_interleaved(engine_factory, case):
         assert not eng2.get_option("phased_shape_inplace:ph_lin2").startswith("shape=5")
 
 
+@pytest.mark.parametrize("case", [(2, "float32", "sum", 1, 64), (4, "bfloat16", "sum", 2, 64), (8, "float16", "max", 1, 64),
+                                  (2, "int32", "sum", 2, 64), (4, "float32", "min", 1, 32), (3, "bfloat16", "sum", 1, 128)])
+def test_interleaved_groups_that_span_several_segments(engine_factory, case):
+    """Segments of 64 chunks: a group of 128 workgroups spans two of them, and the rows of a thread
+    belong to different segments with different source orders.  In place and staged against the
+    oracle; segments of 32 chunks keep the other shapes (unless the plan mostly writes: the allgather
+    test), and with three ranks of 128 chunks the plain interleaved kernel runs."""
+    world, dtype, op, channels, seg_chunks = case
+    es = 4 if dtype in ("float32", "int32") else 2
+    n = world * channels * seg_chunks * CHUNK_VECS * (16 // es)
+    jsons = graph_jsons("ring", "build_allreduce", world, n, dtype, "sm", channels, reduce_op=op)
+    kind = "randint" if dtype == "int32" else "randn"
+    x = seeded_inputs(kind, world, n, dtype, seed=31 + world + seg_chunks)
+    want = oracle_buffers(jsons, x, dtype)
+    eng = engine_factory(world)
+    _register(eng, "ph_rows", jsons)
+    eng.set_option("phased", 1)
+    try:
+        total = world * channels * seg_chunks
+        how = eng.get_option("phased_shape_inplace:ph_rows")
+        if total % 128 == 0 and seg_chunks >= 64:
+            spans = 128 // seg_chunks
+            assert how == ("shape=5 group=128 meetings=1" if spans == 1 else f"shape=5 group=128 segments={spans} meetings=1"), how
+        else:
+            assert not how.startswith("shape=5"), how
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("ph_rows", bufs, sync=True)
+        _check(bufs, want, f"in place ({how})")
+        outs = eng.execute_operation("ph_rows", [t.cuda() for t in x])
+        _check(outs, want, f"staged ({how})")
+        eng.set_option("num_blocks", 128)
+        bufs = [t.cuda() for t in x]
+        eng.execute_inplace("ph_rows", bufs, sync=True)
+        _check(bufs, want, "grid of 128")
+    finally:
+        eng.set_option("phased", -1); eng.set_option("num_blocks", 0)
+
+
 def test_allgather_on_interleaved_chunks(engine_factory):
     """A plan that mostly writes stays on the slot runner unless its chunks can be interleaved: an
     allgather of 16 MiB pieces goes to the phased runner's shape 5 by itself (staged and in place),
@@ -249,19 +287,29 @@ def test_allgather_on_interleaved_chunks(engine_factory):
     eng.set_option("phased_linear", 0)
     assert eng.get_option("runner_staged:ag_lin") == "column_slot_kernel"
     eng.set_option("phased_linear", -1)
-    # pieces of 8 MiB (64 chunks): groups of 64, for plans that mostly write; of 4 MiB: the slot runner
+    # pieces of 8 MiB (64 chunks): a group spans two of them
     half = graph_jsons("ring", "build_allgather", world, n // 2, dtype, "sm", 1)
     _register(eng, "ag_half", half)
-    assert eng.get_option("phased_shape_staged:ag_half") == "shape=5 group=64 meetings=1"
+    assert eng.get_option("phased_shape_staged:ag_half") == "shape=5 group=128 segments=2 meetings=1"
     xh = seeded_inputs("randn", world, chunk // 2, dtype, seed=6)
     wanth = oracle_buffers(half, xh, dtype, buffer_elems=n // 2, place=lambda r: r * (chunk // 2))
     outs = [torch.zeros(n // 2, dtype=torch.float16, device="cuda") for _ in range(world)]
     eng.execute_operation("ag_half", [t.cuda() for t in xh], outs)
-    _check(outs, wanth, "groups of 64, staged")
+    _check(outs, wanth, "two segments per group, staged")
+    # pieces of 4 MiB (32 chunks): four segments per group, for a plan that mostly writes
     quarter = graph_jsons("ring", "build_allgather", world, n // 4, dtype, "sm", 1)
     _register(eng, "ag_quarter", quarter)
-    assert eng.get_option("runner_staged:ag_quarter") == "column_slot_kernel"
-    assert eng.get_option("phased_shape_staged:ag_quarter") == "none"
+    assert eng.get_option("phased_shape_staged:ag_quarter") == "shape=5 group=128 segments=4 meetings=1"
+    xq = seeded_inputs("randn", world, chunk // 4, dtype, seed=7)
+    wantq = oracle_buffers(quarter, xq, dtype, buffer_elems=n // 4, place=lambda r: r * (chunk // 4))
+    outs = [torch.zeros(n // 4, dtype=torch.float16, device="cuda") for _ in range(world)]
+    eng.execute_operation("ag_quarter", [t.cuda() for t in xq], outs)
+    _check(outs, wantq, "four segments per group, staged")
+    # pieces of 1 MiB: too small for any of it, the slot runner
+    tiny = graph_jsons("ring", "build_allgather", world, n // 16, dtype, "sm", 1)
+    _register(eng, "ag_tiny", tiny)
+    assert eng.get_option("runner_staged:ag_tiny") == "column_slot_kernel"
+    assert eng.get_option("phased_shape_staged:ag_tiny") == "none"
 
 
 def test_two_launches_of_one_operation_on_two_streams(engine_factory):
