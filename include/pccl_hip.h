@@ -273,8 +273,9 @@ int pccl_hip_register_triggers(pccl_hip_ctx* ctx, const char* name, int vrank,
  * which run without meetings below that); "phased_linear" = "-1" | "0" | "1" (the 256 x 32 shape with
  * the chunks of 128 neighbouring workgroups interleaved slab by slab, so that the chip sweeps each rank
  * buffer as one stream; possible on up to 8 ranks when every segment of the plan is a whole multiple of
- * 128 chunks - 16 MiB of every rank - and 128 divides the grid (groups of 64 for plans that mostly
- * write, where 128 does not divide); -1: wherever possible except for plans
+ * 128 chunks - 16 MiB of every rank - and 128 divides the grid; also for segments of 64 chunks - of 32
+ * for plans that mostly write - that lie one after the other and have the same sources count, operator
+ * and store mask, a group then spanning several of them; -1: wherever possible except for plans
  * that load four times what they store; 1: for those as well); "phased_barriers" = "1" | "0" (0: no
  * meetings, for comparison); "phased_timeout_us" (how long a workgroup waits at a meeting before the
  * launch goes on unsynchronised: meetings order nothing; the environment variable PCCL_PHASED sets
@@ -297,7 +298,7 @@ int pccl_hip_set_option(pccl_hip_ctx* ctx, const char* key, const char* value);
  * NAME would launch now - "phased_kernel", "column_slot_kernel", "column_kernel", "level_kernel",
  * "persistent_kernel", "gather_kernel", or "staging + ..." - which links the operation; and
  * "phased_shape_inplace:NAME" / "phased_shape_staged:NAME": the phased runner's shape for operation
- * NAME as "shape=N group=K meetings=M" (N: 0 = 512 threads x 16 vectors, 1 / 3 = 256 x 32 without / with
+ * NAME as "shape=N group=K [segments=S] meetings=M" (N: 0 = 512 threads x 16 vectors, 1 / 3 = 256 x 32 without / with
  * the exchange, 2 = balanced trees, 4 = two sweeps per write phase, 5 = interleaved chunks), or "none";
  * "slot_shape:NAME": the slot runner's workgroup for operation NAME as "threads x vectors", e.g.
  * "256x2", or "0x0" if its column plan does not run there - chosen from the rank count, and larger
